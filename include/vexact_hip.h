@@ -1,0 +1,180 @@
+/*
+ * vexact_hip.h - C ABI of libvexact_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * batch-invariant inference hot path of verl-project/vexact.
+ *
+ * Conventions (every entry point):
+ *   - returns 0 on success or a negative VX_ERR_* code; never throws, never allocates, never
+ *     synchronises and never reads device memory on the host, so every call is safe under HIP
+ *     graph capture;
+ *   - all data pointers are device pointers owned by the caller; `stream` is the HIP stream to
+ *     launch on; strides and leading dimensions are in ELEMENTS unless the name says bytes;
+ *   - launch geometry depends only on the sizes passed by value, never on device data;
+ *   - dtype codes: 0 = float32, 1 = bfloat16, 2 = float16;
+ *   - batch invariance: the bits of an output row depend on that row's own inputs only (not on
+ *     the number of rows, their order, or which other rows share the launch).
+ *
+ * The reference has no C FFI; each entry point names the Python/Triton function of
+ * /root/reference it replaces (file:line).
+ */
+#ifndef VEXACT_HIP_H_
+#define VEXACT_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* hipStream_t;
+
+#define VX_OK 0
+#define VX_ERR_ARG (-1)         /* null pointer, negative size, bad stride */
+#define VX_ERR_UNSUPPORTED (-2) /* shape / dtype / alignment / layout outside the fast paths */
+#define VX_ERR_WORKSPACE (-3)   /* workspace pointer missing or too small */
+#define VX_ERR_LAUNCH (-4)      /* hipLaunch reported an error */
+
+int vx_abi_version(void);
+const char* vx_status_string(int code);
+
+/* ---- row reductions ------------------------------------------------------------------- */
+
+/* mean over the middle dim of an (M, N, K) strided view, output (M, K) with strides (o0, o1).
+ * Replaces mean_kernel / mean_dim, vexact/batch_invariant_ops/batch_invariant_ops.py:336-473. */
+int vx_mean_dim(const void* in, void* out, int dtype, int64_t M, int64_t N, int64_t K, int64_t s0,
+                int64_t s1, int64_t s2, int64_t o0, int64_t o1, hipStream_t stream);
+
+/* RMSNorm over the last dim of [rows, n].
+ *   mode 0: y = round(x * (1/sqrt(mean(x^2) + eps)) * w)          (one rounding)
+ *           replaces _rms_norm_kernel / _rms_norm_forward, batch_invariant_ops.py:637-687
+ *   mode 1: y = round(w * round(x * (1/sqrt(mean(x^2) + eps))))   (HuggingFace Qwen3 RMSNorm as it
+ *           executes when its .mean(-1) is routed through mean_dim, batch_invariant_ops.py:619-622)
+ * residual (optional): the row is first replaced by round(x + residual) and that sum is written to
+ * sum_out (optional; may alias x or residual). */
+int vx_rms_norm(const void* x, const void* residual, const void* weight, void* y, void* sum_out,
+                int dtype, int64_t rows, int64_t n, int64_t x_stride, int64_t res_stride,
+                int64_t y_stride, int64_t sum_stride, float eps, int mode, hipStream_t stream);
+
+/* log_softmax over the last dim of [rows, n]; needs vx_log_softmax_workspace_bytes(rows, n) bytes.
+ * Replaces _log_softmax_kernel / log_softmax, batch_invariant_ops.py:231-333. */
+int64_t vx_log_softmax_workspace_bytes(int64_t rows, int64_t n);
+int vx_log_softmax(const void* x, void* y, int dtype, int64_t rows, int64_t n, int64_t x_stride,
+                   int64_t y_stride, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
+/* out[i] = logits[i, labels[i]] - logsumexp(logits[i, :]) in fp32 (same workspace as log_softmax).
+ * labels == NULL: use the first argmax of the row (greedy token), also written to tokens_out.
+ * Replaces logprobs_from_logits_flash_attn, vexact/batch_invariant_ops/standalone_logprobs.py:28-55. */
+int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* tokens_out, int dtype,
+                int64_t rows, int64_t n, int64_t x_stride, void* workspace, int64_t workspace_bytes,
+                hipStream_t stream);
+
+/* ---- dense GEMM ----------------------------------------------------------------------- */
+
+/* C[M,N] = X[M,K] * W[N,K]^T (+ bias[N]), bf16 in/out, fp32 accumulate, K ascending, no split-K.
+ * Needs K % 8 == 0, ldx % 8 == 0, ldw % 8 == 0 and 16-byte aligned X, W (else VX_ERR_UNSUPPORTED).
+ * Replaces matmul_kernel_persistent / matmul_persistent, batch_invariant_ops.py:53-228. */
+int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, hipStream_t stream);
+/* Same, forcing the kernel: kind 0 = weight-streaming with 16*mt-row tiles (mt in 1,2,4),
+ * kind 1 = 128x128 LDS-tiled. Results are bit-identical across kinds (tested). */
+int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void* c, int64_t M,
+                            int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind,
+                            int mt, hipStream_t stream);
+/* Batched, fully strided fallback for any dtype code: one thread per output, fp32 FMA chain in
+ * ascending k. Covers the layouts / dtypes of matmul_persistent and _bmm_kernel / triton_bmm
+ * (batch_invariant_ops.py:484-606) that the fast path rejects. */
+int vx_gemm_generic(const void* a, const void* b, const void* bias, void* c, int dtype, int64_t batch,
+                    int64_t M, int64_t N, int64_t K, int64_t sab, int64_t sam, int64_t sak,
+                    int64_t sbb, int64_t sbk, int64_t sbn, int64_t scb, int64_t scm, int64_t scn,
+                    hipStream_t stream);
+/* out[n, k] = in[k, n] (bf16) - packs a [K, N] row-major operand for vx_gemm_bf16_nt. */
+int vx_transpose_bf16(const void* in, void* out, int64_t K, int64_t N, int64_t ld_in, int64_t ld_out,
+                      hipStream_t stream);
+
+/* ---- paged KV cache + attention -------------------------------------------------------- */
+
+/* cache.view(-1, row)[slot_mapping[t]] = src[t] for slot != -1; value / v_cache may be NULL.
+ * Replaces _store_cache_kernel / store_kvcache, vexact/batch_invariant_ops/kv_cache_context.py:259-314. */
+int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_cache,
+                     const int* slot_mapping, int64_t num_tokens, int64_t k_src_stride_bytes,
+                     int64_t v_src_stride_bytes, int64_t k_row_bytes, int64_t v_row_bytes,
+                     hipStream_t stream);
+
+/* Causal GQA attention, bf16, head dims (Dk, Dv) in {(32,32),(64,64),(128,128),(192,128),(256,256)}.
+ *   mode 0: paged decode - every sequence has at most one query token; KV is split into fixed
+ *           256-key chunks (absolute positions) and folded in ascending order; needs
+ *           vx_paged_attn_decode_workspace_bytes(num_seqs, Hq, Dv, max_pages * page_size) bytes
+ *   mode 1: paged general (chunked prefill, mixed batches) - same arithmetic per row as mode 0
+ *   mode 2: packed K/V [Tk, Hkv, D] with cu_seqlens_k (skp = row stride, no block table)
+ * q [total_q, Hq, Dk], k/v cache [blocks, page, Hkv, D], out [total_q, Hq, Dv];
+ * query i of a sequence sits at absolute position kv_len - q_len + i.
+ * Replaces _paged_attn_fwd_block_kernel / _PagedFlashAttentionVarlen.forward and the forward of
+ * _varlen_attn_fwd_block_kernel, vexact/batch_invariant_ops/triton_invariant_attention.py:433-692, 47-190. */
+int vx_attn_chunk_size(void);
+int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Dv,
+                                             int64_t max_kv_len);
+int vx_attention(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens_q,
+                 const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                 int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv, int64_t sqt,
+                 int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb, int64_t svp,
+                 int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride, int64_t max_pages,
+                 int page_size, float softmax_scale, int causal, int mode, int max_seqlen_q,
+                 void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
+/* ---- fused MoE ------------------------------------------------------------------------- */
+
+/* softmax(fp32) -> top-k (ties: lower expert first) -> optional renorm -> cast.
+ * Replaces the router in moe_block_forward, vexact/models/qwen3_moe/modeling_qwen3_moe.py:128-134. */
+int vx_router_topk(const void* logits, void* weights_out, void* idx_out, int64_t T, int E, int k,
+                   int64_t ld, int logits_bf16, int out_bf16, int idx_i64, int renorm,
+                   hipStream_t stream);
+
+/* Routing integers for T*k flat entries (all exact): splits[E], cu[E+1], scatter_index[T*k] (stable
+ * expert-major rank), sorted_token[T*k], sorted_flat[T*k], and a tile table of at most
+ * vx_moe_max_tiles(T*k, E, bm) row tiles (group id or -1, first row, rows).
+ * Replaces expert_histogram (group_gemm/kernel/moe.py:52-81), the double argsort
+ * (fused_moe.py:43) and _build_moe_indices (fused_moe.py:268-292). */
+int64_t vx_moe_max_tiles(int64_t n_entries, int E, int bm);
+int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,
+                 int* cu, int* scatter_index, int* sorted_token, int* sorted_flat, int* tile_group,
+                 int* tile_row0, int* tile_rows, int64_t max_tiles, hipStream_t stream);
+
+/* Grouped GEMM over the tile table: C[rows] = X[row_src[rows]] * W[group]^T, bf16.
+ *   epi 0: plain store (replaces group_gemm_same_nk, group_gemm/kernel/group_gemm.py:65-237)
+ *   epi 1: w = gate rows, w2 = up rows, C = round(round(round(silu(round(g))) * round(u)) * s) with
+ *          s = row_scale[row_scale_idx[row]] (adds the glue of fused_moe.py:75-88)
+ * bm (rows per tile) must match the tile table: 16 / 32 / 64 stream weights, 128 is LDS-tiled. */
+int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64_t ldw,
+                int64_t w_gstride, void* c, int64_t ldc, int64_t N, int64_t K, const int* tile_group,
+                const int* tile_row0, const int* tile_rows, int64_t max_tiles, int bm,
+                const int* row_src, const void* row_scale, const int* row_scale_idx, int epi,
+                hipStream_t stream);
+
+/* Replace expert_histogram / moe_scatter / moe_gather, group_gemm/kernel/moe.py:52-81, 304-335, 131-161.
+ * vx_moe_gather: y[t] = round(sum_i x[index[t, i]]) in slot order (fp32); with residual:
+ * y[t] = round(residual[t] + round(sum)). */
+int vx_expert_histogram(const void* idx, int idx_i64, int64_t n, int E, int* out, hipStream_t stream);
+int vx_moe_scatter(const void* x, void* out, const int* index, int64_t T, int k, int64_t H, int64_t ldx,
+                   int64_t ldo, hipStream_t stream);
+int vx_moe_gather(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                  int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, hipStream_t stream);
+
+/* ---- decoder-layer glue ---------------------------------------------------------------- */
+
+/* Per-head RMSNorm (mode 1 form) of q and k, bf16 rotary embedding from cos/sin tables
+ * [max_pos, D], q -> q_out [T, Hq, D], k -> k_out (optional) and k_cache slot, v -> v_cache slot.
+ * qkv rows are [q heads | k heads | v heads]. The scatter is store_kvcache
+ * (kv_cache_context.py:294-314); norm + rotary are the HuggingFace Qwen3 attention prologue the
+ * reference runs between its q/k/v projections and its attention call. */
+int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, const void* k_norm_w,
+                          const void* cos_table, const void* sin_table, const void* positions,
+                          int pos_i64, const int* slot_mapping, void* q_out, void* k_out,
+                          void* k_cache, void* v_cache, int64_t T, int Hq, int Hkv, int D, float eps,
+                          int64_t max_pos, hipStream_t stream);
+int vx_embedding(const void* table, const void* ids, int ids_i64, void* out, int64_t T, int64_t H,
+                 int64_t vocab, hipStream_t stream);
+int vx_fill_i32(int* p, int value, int64_t n, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VEXACT_HIP_H_ */

@@ -1,0 +1,36 @@
+"""CPU oracle for the batch-invariant hot path: TEST INFRASTRUCTURE ONLY.
+
+Plain torch-CPU / numpy restatements of the reference's algorithms (each function cites the
+reference file:line it follows). Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this package; the product (``vexact_amd``) never
+does, and has no CPU fallback.
+
+How each function is pinned (checked in ``tests/test_oracle_*.py``; none needs the reference
+imported, and the reference ships no stored golden vectors for these ops):
+
+=====================  ===========================================================================
+function               pinned by
+=====================  ===========================================================================
+matmul_ref             fp64 brute force on tiny inputs; exact integer-valued cases
+mean_dim_ref           fp64 brute force; constant rows
+rms_norm_ref (both)    fp64 brute force; unit-weight / constant-row closed forms; the two rounding
+                       variants differ by <= 1 bf16 ulp
+log_softmax_ref        torch.log_softmax (library routine); rows sum to 1 after exp; shift invariance
+logprobs_ref           gather of log_softmax_ref; fallback formula the reference itself states
+                       (standalone_logprobs.py:45-47)
+store_kvcache_ref      python-loop restatement vs vectorised indexing; slot -1 rows untouched
+paged gather           make_paged_kv_cache round trip (gather back == original sequences)
+eager_attention        fp64 softmax-attention brute force; q_len = kv_len = 1 => out == v; uniform
+                       keys => mean of visible values
+router_ref             brute-force python top-k with the documented tie rule; weights sum to 1
+routing_integers_ref   brute-force counting; numpy stable argsort twice (fused_moe.py:43)
+fused_moe_ref          k=1,w=1 => plain SwiGLU MLP; all tokens on one expert => dense formula;
+                       fp64 brute force on tiny shapes; HF-eager form within bf16 tolerance
+prepare_gen_ctx_ref    hand-worked example; vectorised numpy twin
+=====================  ===========================================================================
+
+Parity unpinned (arithmetic lives in third-party wheels that are not in the reference tree, and
+only invariance tests cover them there): the exact bit patterns of flash-attn 3/4 attention,
+flash-attn 2.8.4 cross-entropy, quack 0.3.4 grouped GEMM and veomni 0.1.9a5 fused MoE. Parity
+against those is by the closed forms above within the stated tolerances.
+"""

@@ -1,0 +1,247 @@
+"""GPU parity: paged / packed attention and the KV-cache scatter.
+
+Restates tests/batch_invariant_ops/test_triton_attention_varlen.py of the reference: paged vs
+eager oracle (atol = rtol = 3e-3 at |x| ~ 0.1, :390-415) and alone vs in-batch bitwise (:417-421),
+alias equality (:424-432), prefill last row == decode row bitwise (:435-454), the Qwen3-like
+16q/8kv/128 page-256 case incl. the packed twin (:457-493), MLA 192/128 (:496-558), backward raises
+(:561-569), wrapper shape (:572-598), error messages (:201-211, :24-30).
+"""
+
+import pytest
+import torch
+
+from oracle import attention as OA
+from tests.util import assert_bf16_close, assert_bitwise
+
+pytestmark = pytest.mark.gpu
+
+from vexact_amd.batch_invariant_ops import flash_attention_forward, triton_flash_attn_varlen_func as flash_attn_varlen_func  # noqa: E402
+from vexact_amd.batch_invariant_ops.kv_cache_context import (  # noqa: E402
+    clear_kv_cache_context,
+    set_kv_cache_context,
+    store_kvcache,
+)
+
+
+def _cu(lens):
+    out = [0]
+    for n in lens:
+        out.append(out[-1] + n)
+    return torch.tensor(out, dtype=torch.int32)
+
+
+def _run_paged(q_seqs, k_seqs, v_seqs, page_size, page_kw="page_table", perm=None, max_seqlen_q=None, pad_seqs=0):
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k_seqs, v_seqs, page_size, perm=perm)
+    q_lens = [q.shape[0] for q in q_seqs]
+    kv_lens = [k.shape[0] for k in k_seqs]
+    cu = _cu(q_lens)
+    used = torch.tensor(kv_lens, dtype=torch.int32)
+    if pad_seqs:  # graph-style padding: zero-length rows pointing at page 0
+        cu = torch.cat([cu, cu[-1:].repeat(pad_seqs)])
+        used = torch.cat([used, torch.zeros(pad_seqs, dtype=torch.int32)])
+        table = torch.cat([table, torch.zeros(pad_seqs, table.shape[1], dtype=torch.int32)])
+    out, _ = flash_attn_varlen_func(
+        torch.cat(q_seqs, dim=0).cuda(), k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=cu.cuda(),
+        max_seqlen_q=max(q_lens) if max_seqlen_q is None else max_seqlen_q, seqused_k=used.cuda(),
+        causal=True, **{page_kw: table.cuda()},
+    )
+    return out
+
+
+def _seqs(lens, heads, dim, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(n, heads, dim, generator=g) * scale).to(torch.bfloat16) for n in lens]
+
+
+@pytest.mark.parametrize(
+    ("q_lens", "kv_lens"),
+    [([1, 1, 1, 1], [17, 31, 40, 49]), ([24, 19], [24, 19]), ([24, 1, 17, 1], [24, 33, 17, 41]),
+     ([1, 1, 1], [255, 256, 257]), ([300, 5, 1], [300, 700, 1000])],
+)
+def test_paged_correctness_and_batch_invariance(q_lens, kv_lens):
+    qh, kh, d, page = 4, 2, 32, 16
+    q = _seqs(q_lens, qh, d, 1, 0.1)
+    k = _seqs(kv_lens, kh, d, 2, 0.1)
+    v = _seqs(kv_lens, kh, d, 3, 0.1)
+    out = _run_paged(q, k, v, page)
+    ref = torch.cat([OA.eager_attention(a, b, c, d**-0.5) for a, b, c in zip(q, k, v)], dim=0)
+    torch.testing.assert_close(out.cpu(), ref, atol=3e-3, rtol=3e-3)
+    off = 0
+    for a, b, c in zip(q, k, v):
+        one = _run_paged([a], [b], [c], page)
+        assert_bitwise(out[off : off + a.shape[0]], one, "alone vs batch")
+        off += a.shape[0]
+    # the general kernel gives the decode kernel's bits (max_seqlen_q unknown -> general path)
+    if max(q_lens) == 1:
+        assert_bitwise(_run_paged(q, k, v, page, max_seqlen_q=0), out, "general kernel on decode batch")
+    # padded sequences are no-ops
+    assert_bitwise(_run_paged(q, k, v, page, pad_seqs=3), out, "padded sequence rows")
+
+
+def test_page_table_aliases_match():
+    q, k, v = _seqs([1], 4, 32, 4), _seqs([33], 2, 32, 5), _seqs([33], 2, 32, 6)
+    assert_bitwise(_run_paged(q, k, v, 16, page_kw="page_table"), _run_paged(q, k, v, 16, page_kw="block_table"), "alias")
+
+
+@pytest.mark.parametrize("qh,kh,d,page,kv_lens", [(4, 2, 32, 16, [17, 33, 64]), (16, 8, 128, 256, list(range(74, 83))),
+                                                    (32, 4, 128, 16, [250, 256, 257, 600, 1030])])
+def test_prefill_decode_and_packed_bitwise_alignment(qh, kh, d, page, kv_lens):
+    qp = _seqs(kv_lens, qh, d, 7)
+    k = _seqs(kv_lens, kh, d, 8)
+    v = _seqs(kv_lens, kh, d, 9)
+    prefill = _run_paged(qp, k, v, page)
+    decode = _run_paged([x[-1:] for x in qp], k, v, page)
+    cu = _cu(kv_lens).cuda()
+    packed, _ = flash_attn_varlen_func(
+        torch.cat(qp).cuda(), torch.cat(k).cuda(), torch.cat(v).cuda(), cu_seqlens_q=cu, cu_seqlens_k=cu,
+        max_seqlen_q=max(kv_lens), max_seqlen_k=max(kv_lens), softmax_scale=d**-0.5, causal=True,
+    )
+    assert_bitwise(packed, prefill, "packed vs paged prefill")
+    off = 0
+    for s, n in enumerate(kv_lens):
+        assert_bitwise(prefill[off + n - 1], decode[s], f"prefill last row vs decode (seq {s})")
+        off += n
+    # chunked prefill: the last 5 rows computed as a 5-token chunk on a cached prefix
+    chunk = _run_paged([x[-5:] for x in qp], k, v, page)
+    off = 0
+    for s, n in enumerate(kv_lens):
+        assert_bitwise(prefill[off + n - 5 : off + n], chunk[5 * s : 5 * s + 5], f"chunk rows (seq {s})")
+        off += n
+
+
+def test_single_key_returns_value_exactly():
+    q, k, v = _seqs([1, 1], 4, 32, 10), _seqs([1, 1], 2, 32, 11), _seqs([1, 1], 2, 32, 12)
+    out = _run_paged(q, k, v, 16)
+    ref = torch.cat([x.repeat_interleave(2, dim=1) for x in v])
+    assert_bitwise(out, ref, "softmax over one key")
+
+
+def test_mla_head_dims_match_eager():
+    kv_lens, q_lens = [40, 70], [40, 1]
+    q, k, v = _seqs(q_lens, 16, 192, 13, 0.1), _seqs(kv_lens, 16, 192, 14, 0.1), _seqs(kv_lens, 16, 128, 15, 0.1)
+    out = _run_paged(q, k, v, 16)
+    assert out.shape == (41, 16, 128)
+    ref = torch.cat([OA.eager_attention(a, b, c, 192**-0.5) for a, b, c in zip(q, k, v)], dim=0)
+    torch.testing.assert_close(out.cpu(), ref, atol=3e-3, rtol=3e-3)
+
+
+def test_config2_shaped_decode_subset():
+    # config 2 geometry (16q / 8kv / 128, page 16, shuffled pages) on 6 sequences
+    g = torch.Generator().manual_seed(2)
+    kv_lens = torch.randint(128, 4097, (6,), generator=g).tolist()
+    q, k, v = _seqs([1] * 6, 16, 128, 16), _seqs(kv_lens, 8, 128, 17), _seqs(kv_lens, 8, 128, 18)
+    pages = sum((n + 15) // 16 for n in kv_lens)
+    perm = torch.randperm(pages + 50, generator=g)
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, 16, perm=perm, extra_pages=50)
+    cu = _cu([1] * 6)
+    used = torch.tensor(kv_lens, dtype=torch.int32)
+    out, _ = flash_attn_varlen_func(torch.cat(q).cuda(), k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=cu.cuda(),
+                                    max_seqlen_q=1, seqused_k=used.cuda(), page_table=table.cuda(), causal=True)
+    ref = OA.paged_attention_ref(torch.cat(q), k_cache, v_cache, cu, used, table, 128**-0.5)
+    assert_bf16_close(out, ref, max_ulp=2, atol_frac=2e-3, what="config-2 decode vs eager oracle")
+    for s in range(6):
+        one, _ = flash_attn_varlen_func(q[s].cuda(), k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=_cu([1]).cuda(),
+                                        max_seqlen_q=1, seqused_k=used[s : s + 1].cuda(),
+                                        page_table=table[s : s + 1].cuda(), causal=True)
+        assert_bitwise(one[0], out[s], f"sequence {s} alone on the same pages")
+
+
+def test_store_kvcache_exact_and_skips():
+    g = torch.Generator().manual_seed(19)
+    for dk, dv in ((128, 128), (192, 128)):
+        key = torch.randn(37, 4, dk, generator=g).to(torch.bfloat16)
+        val = torch.randn(37, 4, dv, generator=g).to(torch.bfloat16)
+        kc = torch.randn(8, 16, 4, dk, generator=g).to(torch.bfloat16)
+        vc = torch.randn(8, 16, 4, dv, generator=g).to(torch.bfloat16)
+        slots = torch.randperm(128, generator=g)[:37].to(torch.int32)
+        slots[[3, 11]] = -1
+        kc_ref, vc_ref = kc.clone(), vc.clone()
+        OA.store_kvcache_ref(key, val, kc_ref, vc_ref, slots)
+        kg, vg = kc.cuda(), vc.cuda()
+        store_kvcache(key.cuda(), val.cuda(), kg, vg, slots.cuda())
+        assert_bitwise(kg, kc_ref, "key cache")
+        assert_bitwise(vg, vc_ref, "value cache")
+
+
+def test_attention_wrapper_shape_and_cache_write():
+    qh, kh, d, page = 4, 2, 32, 16
+    q_lens, past = [3, 1], [5, 20]
+    kv_lens = [p + n for p, n in zip(past, q_lens)]
+    q, k, v = _seqs(q_lens, qh, d, 20, 0.1), _seqs(kv_lens, kh, d, 21, 0.1), _seqs(kv_lens, kh, d, 22, 0.1)
+    # cache holds only the past; the wrapper must write the new tokens
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, page)
+    slots, newk, newv = [], [], []
+    for s, (p, n) in enumerate(zip(past, q_lens)):
+        for pos in range(p, p + n):
+            slots.append(int(table[s, pos // page]) * page + pos % page)
+            k_cache.view(-1, kh, d)[slots[-1]] = 0
+            v_cache.view(-1, kh, d)[slots[-1]] = 0
+        newk.append(k[s][p:])
+        newv.append(v[s][p:])
+    kc, vc = k_cache.cuda(), v_cache.cuda()
+    set_kv_cache_context(
+        is_paged_attn=True, key_cache={0: kc}, value_cache={0: vc}, block_tables=table.cuda(),
+        context_lens=torch.tensor(kv_lens, dtype=torch.int32).cuda(),
+        slot_mapping=torch.tensor(slots, dtype=torch.int32).cuda(), query_start_loc=_cu(q_lens).cuda(), max_seqlen_q=3,
+    )
+    try:
+        module = torch.nn.Module()
+        module.layer_idx = 0
+        qq = torch.cat(q).transpose(0, 1).unsqueeze(0).cuda()
+        kk = torch.cat(newk).transpose(0, 1).unsqueeze(0).cuda()
+        vv = torch.cat(newv).transpose(0, 1).unsqueeze(0).cuda()
+        out, aux = flash_attention_forward(module, qq, kk, vv, None, scaling=d**-0.5)
+    finally:
+        clear_kv_cache_context()
+    assert aux is None and out.shape == (4, qh, d)
+    ref = torch.cat([OA.eager_attention(a, b, c, d**-0.5) for a, b, c in zip(q, k, v)], dim=0)
+    torch.testing.assert_close(out.cpu(), ref, atol=3e-3, rtol=3e-3)
+    full_k, _, _ = OA.make_paged_kv_cache(k, v, page)
+    assert_bitwise(kc, full_k, "wrapper wrote the new keys")
+
+
+def test_argument_errors():
+    q, k, v = _seqs([2], 4, 32, 23), _seqs([2], 2, 32, 24), _seqs([2], 2, 32, 25)
+    qg, kg, vg = q[0].cuda(), k[0].cuda(), v[0].cuda()
+    cu = _cu([2]).cuda()
+    with pytest.raises(ValueError, match="max_seqlen_k is required"):
+        flash_attn_varlen_func(qg, kg, vg, cu_seqlens_q=cu, cu_seqlens_k=cu, max_seqlen_q=2, causal=True)
+    with pytest.raises(ValueError, match="max_seqlen_q is required"):
+        flash_attn_varlen_func(qg, kg, vg, cu_seqlens_q=cu, cu_seqlens_k=cu, max_seqlen_k=2, causal=True)
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, 16)
+    used = torch.tensor([2], dtype=torch.int32).cuda()
+    with pytest.raises(ValueError, match="pass only one of page_table or block_table"):
+        flash_attn_varlen_func(qg, k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=cu, seqused_k=used,
+                               page_table=table.cuda(), block_table=table.cuda(), causal=True)
+    with pytest.raises(NotImplementedError):
+        flash_attn_varlen_func(qg, kg, vg, cu_seqlens_q=cu, cu_seqlens_k=cu, max_seqlen_q=2, max_seqlen_k=2, dropout_p=0.1)
+    with pytest.raises(NotImplementedError):
+        flash_attn_varlen_func(qg, kg, vg, cu_seqlens_q=cu, cu_seqlens_k=cu, max_seqlen_q=2, max_seqlen_k=2, softcap=1.0)
+    with pytest.raises(NotImplementedError):
+        flash_attn_varlen_func(qg, kg, vg, cu_seqlens_q=cu, cu_seqlens_k=cu, max_seqlen_q=2, max_seqlen_k=2, window_size=(4, 0))
+    with pytest.raises(NotImplementedError, match="only supports causal=True"):
+        flash_attn_varlen_func(qg, k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=cu, seqused_k=used,
+                               page_table=table.cuda(), causal=False)
+    with pytest.raises(ValueError, match="torch.int32"):
+        flash_attn_varlen_func(qg, k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=cu.long(), seqused_k=used,
+                               page_table=table.cuda(), causal=True)
+
+
+def test_paged_backward_raises():
+    q, k, v = _seqs([2], 4, 32, 26), _seqs([2], 2, 32, 27), _seqs([2], 2, 32, 28)
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, 16)
+    qg = q[0].cuda().requires_grad_(True)
+    out, _ = flash_attn_varlen_func(qg, k_cache.cuda(), v_cache.cuda(), cu_seqlens_q=_cu([2]).cuda(),
+                                    seqused_k=torch.tensor([2], dtype=torch.int32).cuda(), page_table=table.cuda(),
+                                    causal=True, max_seqlen_q=2)
+    with pytest.raises(NotImplementedError, match="paged triton flash_attn_varlen_func backward"):
+        out.sum().backward()
+
+
+def test_packed_non_causal_matches_eager():
+    q, k, v = _seqs([5, 9], 4, 64, 29, 0.2), _seqs([12, 9], 2, 64, 30, 0.2), _seqs([12, 9], 2, 64, 31, 0.2)
+    out, _ = flash_attn_varlen_func(torch.cat(q).cuda(), torch.cat(k).cuda(), torch.cat(v).cuda(),
+                                    cu_seqlens_q=_cu([5, 9]).cuda(), cu_seqlens_k=_cu([12, 9]).cuda(),
+                                    max_seqlen_q=9, max_seqlen_k=12, causal=False)
+    ref = torch.cat([OA.eager_attention(a, b, c, 64**-0.5, causal=False) for a, b, c in zip(q, k, v)])
+    torch.testing.assert_close(out.cpu(), ref, atol=3e-3, rtol=3e-3)

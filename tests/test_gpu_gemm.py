@@ -1,0 +1,130 @@
+"""GPU parity: batch-invariant GEMM. Restates tests/batch_invariant_ops/test_matmul.py:25-46 (row
+slice vs full batch, atol = rtol = 0) and the linspace variant of
+tests/batch_invariant_ops/test_batch_invariance.py:30-44, plus parity with the CPU oracle."""
+
+import pytest
+import torch
+
+from oracle import row_ops as O
+from tests.util import assert_bf16_close, assert_bitwise
+
+pytestmark = pytest.mark.gpu
+
+from vexact_amd import ops  # noqa: E402
+from vexact_amd.batch_invariant_ops import matmul_persistent, set_batch_invariant_mode, triton_bmm  # noqa: E402
+
+
+def _gen(shape, seed, dtype=torch.bfloat16, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("K,N", [(2048, 4096), (4096, 2048), (2048, 128), (768, 2048), (136, 200)])
+def test_bf16_linear_bits_do_not_depend_on_batch(K, N):
+    a = _gen((300, K), 1)
+    w = _gen((N, K), 2, scale=0.02)
+    ag, wg = a.cuda(), w.cuda()
+    full = matmul_persistent(ag, wg.t())
+    assert_bf16_close(full, O.matmul_ref(a, w.t()), max_ulp=2, what=f"mm {K}x{N} vs oracle")
+    for m in (1, 7, 16, 17, 33, 64, 65, 128, 256):
+        assert_bitwise(matmul_persistent(ag[:m], wg.t()), full[:m], f"mm first {m} rows")
+    assert_bitwise(matmul_persistent(ag[200:201], wg.t()), full[200:201], "mm row 200 alone")
+    assert_bitwise(matmul_persistent(ag[129:140], wg.t()), full[129:140], "mm rows 129..139")
+
+
+def test_stream_and_tiled_kernels_agree_bitwise():
+    a = _gen((130, 1024), 3)
+    w = _gen((328, 1024), 4, scale=0.05)
+    bias = _gen((328,), 5)
+    ag, wg, bg = a.cuda(), w.cuda(), bias.cuda()
+    ref = ops.gemm_nt_variant(ag, wg, kind=1, bias=bg)
+    for mt in (1, 2, 4):
+        assert_bitwise(ops.gemm_nt_variant(ag, wg, kind=0, mt=mt, bias=bg), ref, f"stream mt={mt} vs tiled")
+    assert_bf16_close(ref, O.matmul_ref(a, w.t(), bias), max_ulp=2, what="biased gemm vs oracle")
+
+
+def test_lm_head_shape_rows():
+    # config-1 shaped: [M, 2048] x [2048, 151936], rows of one draw
+    a = _gen((64, 2048), 6)
+    w = _gen((151936, 2048), 7, scale=0.02)
+    ag, wg = a.cuda(), w.cuda()
+    full = matmul_persistent(ag, wg.t())
+    for m in (1, 7):
+        assert_bitwise(matmul_persistent(ag[:m], wg.t()), full[:m], f"lm_head first {m}")
+    ref = O.matmul_ref(a[:4], w.t())
+    assert_bf16_close(full[:4], ref, max_ulp=2, what="lm_head vs oracle")
+
+
+def test_linspace_inputs():
+    a = torch.linspace(-100, 100, 32 * 512).reshape(32, 512).to(torch.bfloat16).cuda()
+    b = torch.linspace(-100, 100, 512 * 64).reshape(512, 64).to(torch.bfloat16).cuda()
+    full = matmul_persistent(a, b)
+    assert_bitwise(matmul_persistent(a[:1], b), full[:1], "linspace row 0")
+    assert_bf16_close(full, O.matmul_ref(a.cpu(), b.cpu()), max_ulp=2, what="linspace vs oracle")
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.float16, 2e-3)])
+def test_other_dtypes_and_layouts(dtype, tol):
+    a = _gen((37, 100), 8, dtype)
+    b = _gen((100, 53), 9, dtype)
+    bias = _gen((53,), 10, dtype)
+    got = matmul_persistent(a.cuda(), b.cuda(), bias.cuda())
+    ref = O.matmul_ref(a, b, bias)
+    torch.testing.assert_close(got.cpu().float(), ref.float(), atol=tol * 10, rtol=tol)
+    assert_bitwise(matmul_persistent(a[:1].cuda(), b.cuda(), bias.cuda()), got[:1], "generic row 0")
+    # bf16, K not a multiple of 8 -> generic kernel; transposed a
+    a2 = _gen((100, 37), 11).t()
+    b2 = _gen((100, 53), 12)
+    got2 = matmul_persistent(a2.cuda(), b2.cuda())
+    assert_bf16_close(got2, O.matmul_ref(a2, b2), max_ulp=2, what="generic bf16")
+
+
+def test_aten_overrides_and_mode_switch():
+    from vexact_amd.batch_invariant_ops import (
+        disable_batch_invariant_mode,
+        enable_batch_invariant_mode,
+        is_batch_invariant_mode_enabled,
+    )
+
+    a = _gen((64, 256), 13).cuda()
+    lin = torch.nn.Linear(256, 512, bias=True, dtype=torch.bfloat16, device="cuda")
+    assert not is_batch_invariant_mode_enabled()
+    with set_batch_invariant_mode(True):
+        assert is_batch_invariant_mode_enabled()
+        y = lin(a)
+        y1 = lin(a[:1])
+        assert_bitwise(y1, y[:1], "nn.Linear under the override")
+        assert_bitwise(y, matmul_persistent(a, lin.weight.t(), lin.bias), "override == direct call")
+        m = torch.mm(a, lin.weight.t())
+        assert_bitwise(m, matmul_persistent(a, lin.weight.t()), "aten::mm override")
+        x32 = a.float().pow(2)
+        assert_bitwise(x32.mean(-1, keepdim=True), ops.mean_dim(x32, -1, keepdim=True), "aten::mean.dim override")
+        ls = torch.log_softmax(a.float(), dim=-1)
+        assert_bitwise(ls, ops.log_softmax(a.float()), "aten::_log_softmax override")
+        with set_batch_invariant_mode(False):
+            assert not is_batch_invariant_mode_enabled()
+        assert is_batch_invariant_mode_enabled()
+        assert_bitwise(torch.mm(a, lin.weight.t()), m, "override restored after nested disable")
+    assert not is_batch_invariant_mode_enabled()
+    enable_batch_invariant_mode()
+    enable_batch_invariant_mode()
+    assert is_batch_invariant_mode_enabled()
+    disable_batch_invariant_mode()
+    assert not is_batch_invariant_mode_enabled()
+    enable_batch_invariant_mode()
+    assert_bitwise(torch.mm(a, lin.weight.t()), m, "enable -> disable -> enable")
+    disable_batch_invariant_mode()
+    torch.use_deterministic_algorithms(False)
+
+
+def test_bmm():
+    a = _gen((3, 5, 16), 14, torch.float32)
+    b = _gen((3, 16, 9), 15, torch.float32)
+    got = triton_bmm(a.cuda(), b.cuda())
+    torch.testing.assert_close(got.cpu(), torch.bmm(a, b), atol=1e-5, rtol=1e-5)
+    inv = _gen((1, 32, 1), 16, torch.float32)
+    pos = torch.arange(40, dtype=torch.float32).reshape(1, 1, 40)
+    got = triton_bmm(inv.cuda(), pos.cuda())
+    torch.testing.assert_close(got.cpu(), torch.bmm(inv, pos), atol=0, rtol=0)  # single products are exact
+    with pytest.raises(AssertionError):
+        triton_bmm(a.cuda()[0], b.cuda())

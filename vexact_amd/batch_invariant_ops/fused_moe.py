@@ -1,0 +1,92 @@
+"""Fused MoE expert forward on the HIP kernels.
+
+Mirrors ``fused_moe_forward`` of ``vexact/batch_invariant_ops/fused_moe.py:459-487`` and the
+``fc1_1_2_weight=`` form the Qwen3-MoE patch calls
+(``vexact/models/qwen3_moe/modeling_qwen3_moe.py:89-100``). Arithmetic follows
+``FusedMoeExpertFunction.forward`` (fused_moe.py:24-102): bf16 gate/up projections, bf16
+``silu(g) * u``, routing weight applied before the down projection, fp32 sum over a token's slots
+in slot order. Forward only.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import ops
+from .group_gemm.kernel.group_gemm import group_gemm_same_nk
+from .group_gemm.kernel.moe import expert_histogram, moe_gather, moe_scatter
+
+
+def _split_weights(fc1_1_weight, fc1_2_weight, fc1_1_2_weight):
+    if fc1_1_2_weight is not None:
+        two_i = fc1_1_2_weight.shape[1]
+        assert two_i % 2 == 0, "fused gate/up weight must have an even number of rows per expert"
+        inter = two_i // 2
+        return fc1_1_2_weight[:, :inter, :], fc1_1_2_weight[:, inter:, :]
+    assert fc1_1_weight is not None and fc1_1_weight.shape == fc1_1_weight.shape
+    assert fc1_2_weight is not None and fc1_1_weight.shape == fc1_2_weight.shape
+    if fc1_1_weight.stride() != fc1_2_weight.stride():
+        fc1_1_weight, fc1_2_weight = fc1_1_weight.contiguous(), fc1_2_weight.contiguous()
+    return fc1_1_weight, fc1_2_weight
+
+
+def fused_moe_forward(
+    num_experts: int,
+    routing_weights: torch.Tensor,
+    selected_experts: torch.Tensor,
+    hidden_states: torch.Tensor,
+    fc1_1_weight: Optional[torch.Tensor],
+    fc1_2_weight: Optional[torch.Tensor],
+    fc2_weight: torch.Tensor,
+    fc1_1_2_weight: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``hidden_states [T,H]``, ``routing_weights/selected_experts [T,k]``; expert weights either as
+    ``fc1_1_weight`` (gate) + ``fc1_2_weight`` (up), each ``[E,I,H]``, or fused ``fc1_1_2_weight [E,2I,H]``
+    (gate rows first); ``fc2_weight [E,H,I]``. Returns ``[T,H]`` bf16."""
+    routing_weights = routing_weights.bfloat16()
+    hidden_states = hidden_states.bfloat16()
+    gate_w, up_w = _split_weights(fc1_1_weight, fc1_2_weight, fc1_1_2_weight)
+    gate_w, up_w, down_w = gate_w.bfloat16(), up_w.bfloat16(), fc2_weight.bfloat16()
+    if gate_w.stride(2) != 1 or up_w.stride() != gate_w.stride():
+        gate_w, up_w = gate_w.contiguous(), up_w.contiguous()
+    if down_w.stride(2) != 1:
+        down_w = down_w.contiguous()
+    shape = hidden_states.shape
+    x = hidden_states.reshape(-1, shape[-1])
+    out = ops.fused_moe(
+        x, routing_weights.reshape(x.shape[0], -1), selected_experts.reshape(x.shape[0], -1), gate_w, up_w, down_w,
+        num_experts,
+    )
+    return out.reshape(shape)
+
+
+def fused_moe_forward_unfused(
+    num_experts: int,
+    routing_weights: torch.Tensor,
+    selected_experts: torch.Tensor,
+    hidden_states: torch.Tensor,
+    fc1_1_weight: torch.Tensor,
+    fc1_2_weight: torch.Tensor,
+    fc2_weight: torch.Tensor,
+) -> torch.Tensor:
+    """The same computation step by step through the public helpers (histogram, stable ranks,
+    scatter, three grouped GEMMs, elementwise glue in torch, gather), as the reference's
+    ``FusedMoeExpertFunction.forward`` lays it out. Must match ``fused_moe_forward`` bit for bit."""
+    routing_weights = routing_weights.bfloat16()
+    hidden_states = hidden_states.bfloat16()
+    splits = expert_histogram(selected_experts, num_experts)
+    scatter_index = selected_experts.flatten().argsort(stable=True).argsort().int().view(selected_experts.shape)
+    scatter_output = moe_scatter(hidden_states, scatter_index)
+    cumsum_t = torch.cumsum(splits, dim=0)
+    max_m = scatter_output.shape[0]
+    g = group_gemm_same_nk(scatter_output, fc1_1_weight, cumsum_t, max_m, transpose_b=True)
+    u = group_gemm_same_nk(scatter_output, fc1_2_weight, cumsum_t, max_m, transpose_b=True)
+    act = torch.ops.aten.silu(g) * u
+    w = routing_weights.reshape(-1, 1)
+    w_sorted = torch.empty_like(w)
+    w_sorted[scatter_index.flatten().long()] = w
+    hw = act * w_sorted
+    o = group_gemm_same_nk(hw, fc2_weight, cumsum_t, max_m, transpose_b=True)
+    return moe_gather(o, scatter_index).reshape(hidden_states.shape)

@@ -1,0 +1,170 @@
+"""Thread-local paged-KV context, block allocator, cache tensors and the cache scatter.
+
+Mirrors ``vexact/batch_invariant_ops/kv_cache_context.py`` of the reference: ``KVCacheContext``
+(:48-104), ``set/get/has_kv_cache_context`` (:107-138), ``KVCacheManager`` (:141-217),
+``KVCacheStore`` (:220-253) and ``store_kvcache`` (:294-314, HIP kernel here).
+"""
+
+from __future__ import annotations
+
+import heapq
+import threading
+from dataclasses import dataclass
+from typing import Iterable, Optional
+
+import torch
+
+from .. import ops
+
+_context_storage = threading.local()
+
+
+@dataclass(frozen=True)
+class KVCacheInfo:
+    layer_idxs: Iterable[int]
+    num_kv_heads: int
+    head_dim: int
+    page_size: int
+    max_blocks: int
+    device: torch.device
+    dtype: torch.dtype = torch.bfloat16
+
+
+@dataclass
+class KVCacheContext:
+    """What the attention wrapper needs for one forward pass.
+
+    ``block_tables [B, max_blocks]`` int32 (-1 padded), ``slot_mapping [T]`` int32 (-1 = do not
+    store), ``context_lens [B]`` int32 (past + new tokens), ``query_start_loc [B+1]`` int32,
+    ``max_seqlen_q`` host int.
+    """
+
+    is_paged_attn: bool = False
+    key_cache: Optional[dict] = None
+    value_cache: Optional[dict] = None
+    block_tables: Optional[torch.Tensor] = None
+    slot_mapping: Optional[torch.Tensor] = None
+    context_lens: Optional[torch.Tensor] = None
+    query_start_loc: Optional[torch.Tensor] = None
+    max_seqlen_q: Optional[int] = None
+
+    def __post_init__(self):
+        if self.is_paged_attn:
+            assert self.key_cache is not None, "key_cache required for paged attention"
+            assert self.value_cache is not None, "value_cache required for paged attention"
+            assert self.block_tables is not None, "block_tables required for paged attention"
+            assert self.context_lens is not None, "context_lens required for paged attention"
+        else:
+            assert self.query_start_loc is not None, "query_start_loc required for packed attention"
+            assert self.context_lens is not None, "context_lens required for packed attention"
+
+
+def set_kv_cache_context(
+    is_paged_attn: bool = False,
+    key_cache=None,
+    value_cache=None,
+    block_tables: Optional[torch.Tensor] = None,
+    context_lens: Optional[torch.Tensor] = None,
+    slot_mapping: Optional[torch.Tensor] = None,
+    query_start_loc: Optional[torch.Tensor] = None,
+    max_seqlen_q: Optional[int] = None,
+):
+    _context_storage.kv_cache_context = KVCacheContext(
+        is_paged_attn=is_paged_attn,
+        key_cache=key_cache,
+        value_cache=value_cache,
+        block_tables=block_tables,
+        context_lens=context_lens,
+        slot_mapping=slot_mapping,
+        query_start_loc=query_start_loc,
+        max_seqlen_q=max_seqlen_q,
+    )
+
+
+def get_kv_cache_context() -> Optional[KVCacheContext]:
+    return getattr(_context_storage, "kv_cache_context", None)
+
+
+def has_kv_cache_context() -> bool:
+    return hasattr(_context_storage, "kv_cache_context")
+
+
+def clear_kv_cache_context() -> None:
+    if hasattr(_context_storage, "kv_cache_context"):
+        del _context_storage.kv_cache_context
+
+
+class KVCacheManager:
+    """Block allocator: always hands out the lowest free block id, ``None`` when out of blocks.
+
+    Same observable behaviour as the reference allocator; the free list is a heap so an
+    allocation costs O(log n) instead of a scan of the free set.
+    """
+
+    def __init__(self, cache_config):
+        self.cache_config = cache_config
+        self.allocated_blocks: set[int] = set()
+        self._free_heap = list(range(cache_config.max_cache_blocks))  # already a valid heap
+        self.free_blocks_set = set(self._free_heap)
+
+    def _num_blocks_needed(self, num_tokens: int) -> int:
+        return (num_tokens + self.cache_config.page_size - 1) // self.cache_config.page_size
+
+    def allocate_blocks(self, total_tokens: int, num_current_blocks: int = 0):
+        delta = self._num_blocks_needed(total_tokens) - num_current_blocks
+        if delta <= 0:
+            return []
+        if len(self.free_blocks_set) < delta:
+            return None
+        allocated = []
+        while len(allocated) < delta:
+            block_id = heapq.heappop(self._free_heap)
+            if block_id not in self.free_blocks_set:  # stale heap entry
+                continue
+            self.free_blocks_set.remove(block_id)
+            self.allocated_blocks.add(block_id)
+            allocated.append(block_id)
+        return allocated
+
+    def num_free_blocks(self) -> int:
+        return len(self.free_blocks_set)
+
+    def num_allocated_blocks(self) -> int:
+        return len(self.allocated_blocks)
+
+    def free_blocks(self, block_ids):
+        for block_id in block_ids:
+            if block_id in self.allocated_blocks:
+                self.allocated_blocks.remove(block_id)
+                self.free_blocks_set.add(block_id)
+                heapq.heappush(self._free_heap, block_id)
+
+
+class KVCacheStore:
+    """Owns per-layer ``[num_blocks, page_size, Hkv, D]`` key/value tensors (zero initialised)."""
+
+    def __init__(self, hf_config, cache_config, device: torch.device):
+        self.hf_config = hf_config
+        self.cache_config = cache_config
+        self.device = device
+        self.page_size = cache_config.page_size
+        self.max_blocks = cache_config.max_cache_blocks
+        num_kv_heads = hf_config.num_key_value_heads
+        default_head_dim = getattr(hf_config, "head_dim", hf_config.hidden_size // hf_config.num_attention_heads)
+        k_head_dim = getattr(hf_config, "qk_head_dim", default_head_dim)
+        v_head_dim = getattr(hf_config, "v_head_dim", k_head_dim)
+        k_shape = (cache_config.max_cache_blocks, cache_config.page_size, num_kv_heads, k_head_dim)
+        v_shape = (cache_config.max_cache_blocks, cache_config.page_size, num_kv_heads, v_head_dim)
+        dtype = getattr(hf_config, "torch_dtype", None) or torch.bfloat16
+        self.key_cache: dict[int, torch.Tensor] = {}
+        self.value_cache: dict[int, torch.Tensor] = {}
+        for layer_idx in range(hf_config.num_hidden_layers):
+            self.key_cache[layer_idx] = torch.zeros(k_shape, device=device, dtype=dtype)
+            self.value_cache[layer_idx] = torch.zeros(v_shape, device=device, dtype=dtype)
+
+
+def store_kvcache(
+    key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor
+):
+    """``cache.view(-1, H*D)[slot] = src`` for every token whose slot is not -1 (K and V may differ in D)."""
+    ops.store_kvcache(key, value, k_cache, v_cache, slot_mapping)

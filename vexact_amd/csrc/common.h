@@ -1,0 +1,107 @@
+// Shared device helpers for the gfx950 (CDNA4) kernels: bf16 conversion, the one MFMA
+// instruction every matrix product goes through, and fixed-shape wavefront reductions.
+//
+// Batch-invariance rule used throughout: an output element is produced by one chain of
+// v_mfma_f32_16x16x32_bf16 instructions that walks the contraction index in ascending
+// 32-wide chunks, with the same (lane-group, slot) -> index mapping in every kernel. Tile
+// shapes may differ between kernels because MFMA rows and columns never mix.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vx {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef uint16_t bf16_t;  // storage type in global memory
+
+constexpr int kWave = 64;
+
+// Status codes returned over the C ABI.
+enum : int {
+  VX_OK = 0,
+  VX_ERR_ARG = -1,       // bad pointer / size / stride
+  VX_ERR_UNSUPPORTED = -2,
+  VX_ERR_WORKSPACE = -3,  // workspace too small
+  VX_ERR_LAUNCH = -4,
+};
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __builtin_bit_cast(float, (uint32_t)v << 16);
+}
+// round-to-nearest-even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  __bf16 h = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, h);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+__device__ __forceinline__ float bf16lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// D(16x16) += A(16x32) * B(32x16). Lane l supplies A[row l%16][k 8*(l/16) .. +8) and
+// B[k 8*(l/16) .. +8)][col l%16]; it receives D[4*(l/16) + r][l%16], r = 0..3.
+__device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// 16-byte global load that yields zeros when !ok. The address must be dereferenceable even
+// when !ok (callers clamp it); selecting on the loaded value instead of on the address keeps
+// the access a single global_load_dwordx4.
+__device__ __forceinline__ uint4 ldg16(const void* p, bool ok) {
+  uint4 v = *reinterpret_cast<const uint4*>(p);
+  v.x = ok ? v.x : 0u;
+  v.y = ok ? v.y : 0u;
+  v.z = ok ? v.z : 0u;
+  v.w = ok ? v.w : 0u;
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide sum over NW wavefronts through LDS; every thread gets the result. The order
+// (lane butterfly, then wave 0..NW-1 ascending) is the same for any grid size.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red /* >= NW floats */) {
+  v = wave_sum(v);
+  if constexpr (NW == 1) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float s = red[0];
+#pragma unroll
+  for (int i = 1; i < NW; i++) s += red[i];
+  return s;
+}
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  if constexpr (NW == 1) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float s = red[0];
+#pragma unroll
+  for (int i = 1; i < NW; i++) s = fmaxf(s, red[i]);
+  return s;
+}
+
+static inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? VX_OK : VX_ERR_LAUNCH;
+}
+
+}  // namespace vx

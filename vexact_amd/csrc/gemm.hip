@@ -1,0 +1,165 @@
+// Dense GEMM entry points.
+//   vx_gemm_bf16_nt : C = X * W^T (+bias), bf16, both operands K-contiguous (the nn.Linear case)
+//   vx_gemm_generic : any strides, f32 / bf16 / f16 - one thread per output element, K walked in
+//                     ascending order with fp32 FMAs; used for layouts the fast path rejects
+//   vx_transpose_bf16 : packs a [K, N] row-major operand to [N, K] so it can use the fast path
+// Replaces matmul_kernel_persistent / matmul_persistent
+// (vexact/batch_invariant_ops/batch_invariant_ops.py:53-228) and _bmm_kernel / triton_bmm (:484-606).
+#include "gemm_core.h"
+
+namespace vx {
+
+template <typename T> struct Cvt;
+template <> struct Cvt<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct Cvt<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+};
+template <> struct Cvt<_Float16> {
+  static __device__ __forceinline__ float ld(const _Float16* p) { return (float)*p; }
+  static __device__ __forceinline__ void st(_Float16* p, float v) { *p = (_Float16)v; }
+};
+
+// Batched, fully strided. 16x16 thread tile: threadIdx.x walks n so stores coalesce.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(
+    const T* __restrict__ a, const T* __restrict__ b, const T* __restrict__ bias, T* __restrict__ c,
+    int64_t M, int64_t N, int64_t K, int64_t sab, int64_t sam, int64_t sak, int64_t sbb, int64_t sbk,
+    int64_t sbn, int64_t scb, int64_t scm, int64_t scn) {
+  const int64_t n = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
+  const int64_t m = (int64_t)blockIdx.y * 16 + (threadIdx.x >> 4);
+  const int64_t bt = blockIdx.z;
+  if (m >= M || n >= N) return;
+  const T* ap = a + bt * sab + m * sam;
+  const T* bp = b + bt * sbb + n * sbn;
+  float acc = 0.f;
+  for (int64_t k = 0; k < K; k++) acc = fmaf(Cvt<T>::ld(ap + k * sak), Cvt<T>::ld(bp + k * sbk), acc);
+  if (bias) acc += Cvt<T>::ld(bias + n);
+  Cvt<T>::st(c + bt * scb + m * scm + n * scn, acc);
+}
+
+// out[n, k] = in[k, n]; 64x64 tiles through LDS
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(const bf16_t* __restrict__ in,
+                                                            bf16_t* __restrict__ out, int64_t K,
+                                                            int64_t N, int64_t ldi, int64_t ldo) {
+  __shared__ bf16_t t[64][66];
+  const int64_t k0 = (int64_t)blockIdx.y * 64, n0 = (int64_t)blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int r = ty; r < 64; r += 4)
+    if (k0 + r < K && n0 + tx < N) t[r][tx] = in[(k0 + r) * ldi + n0 + tx];
+  __syncthreads();
+  for (int r = ty; r < 64; r += 4)
+    if (n0 + r < N && k0 + tx < K) out[(n0 + r) * ldo + k0 + tx] = t[tx][r];
+}
+
+}  // namespace vx
+
+using namespace vx;
+
+extern "C" {
+
+int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int64_t M, int64_t N,
+                    int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, hipStream_t stream) {
+  if (!x || !w || !c || M < 0 || N <= 0 || K <= 0) return VX_ERR_ARG;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return VX_ERR_ARG;
+  if (!gemm_fast_ok(x, w, K, ldx, ldw)) return VX_ERR_UNSUPPORTED;
+  if (M == 0) return VX_OK;
+  GemmParams p = {};
+  p.x = (const bf16_t*)x; p.ldx = ldx;
+  p.w = (const bf16_t*)w; p.ldw = ldw;
+  p.bias = (const bf16_t*)bias;
+  p.c = (bf16_t*)c; p.ldc = ldc;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  if (M <= 64) {
+    const dim3 grid((unsigned)((N + 63) / 64), 1);
+    if (M <= 16) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+    else if (M <= 32) gemm_stream_kernel<2, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+    else gemm_stream_kernel<4, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  } else {
+    const int64_t mt = (M + TL_BM - 1) / TL_BM;
+    if (mt > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)mt);
+    gemm_tiled_kernel<EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  }
+  return launch_status();
+}
+
+// Forces one of the two kernels regardless of M (kind 0 = streaming with 16*mt rows per tile,
+// mt in {1,2,4}; kind 1 = tiled). For tests that check both kernels give the same bits.
+int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void* c, int64_t M,
+                            int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind,
+                            int mt, hipStream_t stream) {
+  if (!x || !w || !c || M <= 0 || N <= 0 || K <= 0) return VX_ERR_ARG;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return VX_ERR_ARG;
+  if (!gemm_fast_ok(x, w, K, ldx, ldw)) return VX_ERR_UNSUPPORTED;
+  GemmParams p = {};
+  p.x = (const bf16_t*)x; p.ldx = ldx;
+  p.w = (const bf16_t*)w; p.ldw = ldw;
+  p.bias = (const bf16_t*)bias;
+  p.c = (bf16_t*)c; p.ldc = ldc;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  if (kind == 0) {
+    if (mt != 1 && mt != 2 && mt != 4) return VX_ERR_ARG;
+    const int64_t bm = 16 * mt;
+    const int64_t my = (M + bm - 1) / bm;
+    if (my > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)my);
+    if (mt == 1) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+    else if (mt == 2) gemm_stream_kernel<2, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+    else gemm_stream_kernel<4, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  } else if (kind == 1) {
+    const int64_t my = (M + TL_BM - 1) / TL_BM;
+    if (my > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)my);
+    gemm_tiled_kernel<EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  } else {
+    return VX_ERR_ARG;
+  }
+  return launch_status();
+}
+
+int vx_gemm_generic(const void* a, const void* b, const void* bias, void* c, int dtype, int64_t batch,
+                    int64_t M, int64_t N, int64_t K, int64_t sab, int64_t sam, int64_t sak,
+                    int64_t sbb, int64_t sbk, int64_t sbn, int64_t scb, int64_t scm, int64_t scn,
+                    hipStream_t stream) {
+  if (!a || !b || !c || batch < 0 || M < 0 || N < 0 || K < 0) return VX_ERR_ARG;
+  if (batch == 0 || M == 0 || N == 0) return VX_OK;
+  const int64_t gx = (N + 15) / 16, gy = (M + 15) / 16;
+  if (gx > 0x7fffffffLL || gy > 65535 || batch > 65535) return VX_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
+  switch (dtype) {
+    case 0:
+      gemm_generic_kernel<float><<<grid, 256, 0, stream>>>((const float*)a, (const float*)b,
+                                                           (const float*)bias, (float*)c, M, N, K,
+                                                           sab, sam, sak, sbb, sbk, sbn, scb, scm, scn);
+      break;
+    case 1:
+      gemm_generic_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+          (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)bias, (bf16_t*)c, M, N, K, sab, sam,
+          sak, sbb, sbk, sbn, scb, scm, scn);
+      break;
+    case 2:
+      gemm_generic_kernel<_Float16><<<grid, 256, 0, stream>>>(
+          (const _Float16*)a, (const _Float16*)b, (const _Float16*)bias, (_Float16*)c, M, N, K, sab,
+          sam, sak, sbb, sbk, sbn, scb, scm, scn);
+      break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+int vx_transpose_bf16(const void* in, void* out, int64_t K, int64_t N, int64_t ld_in, int64_t ld_out,
+                      hipStream_t stream) {
+  if (!in || !out || K < 0 || N < 0) return VX_ERR_ARG;
+  if (K == 0 || N == 0) return VX_OK;
+  const int64_t gx = (N + 63) / 64, gy = (K + 63) / 64;
+  if (gx > 0x7fffffffLL || gy > 65535) return VX_ERR_UNSUPPORTED;
+  transpose_bf16_kernel<<<dim3((unsigned)gx, (unsigned)gy), 256, 0, stream>>>(
+      (const bf16_t*)in, (bf16_t*)out, K, N, ld_in, ld_out);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,178 @@
+// Glue between the hot-path kernels of a Qwen3-style decoder layer, fused so that a decode
+// step is a short, capture-safe launch sequence:
+//   * vx_qk_norm_rope_store : per-head RMSNorm of q and k (two-rounding HuggingFace form), rotary
+//     embedding in bf16, q written out, k and v scattered into the paged cache at slot_mapping
+//     (the scatter is what store_kvcache does, vexact/batch_invariant_ops/kv_cache_context.py:294-314)
+//   * vx_embedding          : row gather
+//   * vx_fill_i32           : small fill kernel (graph-safe replacement for a memset node)
+// The per-head sum of squares uses the same lane ownership and butterfly as the 64-thread
+// variant of vx_rms_norm, so fused and unfused paths give the same bits.
+#include "common.h"
+#include <math.h>
+
+namespace vx {
+
+// grid = (ceil(T*(Hq+2Hkv)/4)); one wavefront per (token, head). Lane l < D/4 owns elements
+// 4l .. 4l+3. qkv row layout: [q heads | k heads | v heads], each head D wide.
+template <int D, typename PosT>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
+    const bf16_t* __restrict__ qkv, int64_t ld, const bf16_t* __restrict__ qw,
+    const bf16_t* __restrict__ kw, const bf16_t* __restrict__ cos_t, const bf16_t* __restrict__ sin_t,
+    const PosT* __restrict__ positions, const int* __restrict__ slots, bf16_t* __restrict__ q_out,
+    bf16_t* __restrict__ k_out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int64_t T,
+    int Hq, int Hkv, float eps, int64_t max_pos) {
+  const int HT = Hq + 2 * Hkv;
+  const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (wid >= T * HT) return;
+  const int64_t t = wid / HT;
+  const int h = (int)(wid % HT);
+  const int lane = threadIdx.x & 63;
+  const bool own = lane < D / 4;
+  const bf16_t* src = qkv + t * ld + (int64_t)h * D;
+  uint2 raw = make_uint2(0, 0);
+  if (own) raw = *(const uint2*)(src + 4 * lane);
+  const int slot = slots ? slots[t] : -1;
+  if (h >= Hq + Hkv) {  // value head: plain copy into the cache
+    if (own && slot >= 0 && v_cache)
+      *(uint2*)(v_cache + ((int64_t)slot * Hkv + (h - Hq - Hkv)) * D + 4 * lane) = raw;
+    return;
+  }
+  float x[4] = {bf16lo(raw.x), bf16hi(raw.x), bf16lo(raw.y), bf16hi(raw.y)};
+  float acc = 0.f;
+  if (own) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc += x[c] * x[c];
+  }
+  const float tot = wave_sum(acc);
+  const float inv = 1.0f / sqrtf(tot / (float)D + eps);
+  const bf16_t* w = (h < Hq) ? qw : kw;
+  int64_t pos = (int64_t)positions[t];
+  pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+  float y[4], cs[4], sn[4];
+  if (own) {
+    const uint2 wr = *(const uint2*)(w + 4 * lane);
+    const float wf[4] = {bf16lo(wr.x), bf16hi(wr.x), bf16lo(wr.y), bf16hi(wr.y)};
+    const uint2 cr = *(const uint2*)(cos_t + pos * D + 4 * lane);
+    const uint2 sr = *(const uint2*)(sin_t + pos * D + 4 * lane);
+    cs[0] = bf16lo(cr.x); cs[1] = bf16hi(cr.x); cs[2] = bf16lo(cr.y); cs[3] = bf16hi(cr.y);
+    sn[0] = bf16lo(sr.x); sn[1] = bf16hi(sr.x); sn[2] = bf16lo(sr.y); sn[3] = bf16hi(sr.y);
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const float tn = bf16_to_f32(f32_to_bf16(x[c] * inv));
+      y[c] = bf16_to_f32(f32_to_bf16(wf[c] * tn));
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < 4; c++) { y[c] = 0.f; cs[c] = 0.f; sn[c] = 0.f; }
+  }
+  // rotate_half partner: element j pairs with j + D/2 (first half gets -partner)
+  constexpr int HL = D / 8;  // lanes per half
+  const bool first = lane < HL;
+  float o[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    const float partner = __shfl(y[c], first ? lane + HL : lane - HL, 64);
+    const float rot = first ? -partner : partner;
+    const float a = bf16_to_f32(f32_to_bf16(y[c] * cs[c]));
+    const float b = bf16_to_f32(f32_to_bf16(rot * sn[c]));
+    o[c] = a + b;
+  }
+  if (!own) return;
+  uint2 pk;
+  pk.x = pack_bf16x2(o[0], o[1]);
+  pk.y = pack_bf16x2(o[2], o[3]);
+  if (h < Hq) {
+    *(uint2*)(q_out + (t * Hq + h) * D + 4 * lane) = pk;
+  } else {
+    const int kh = h - Hq;
+    if (k_out) *(uint2*)(k_out + (t * Hkv + kh) * D + 4 * lane) = pk;
+    if (slot >= 0 && k_cache) *(uint2*)(k_cache + ((int64_t)slot * Hkv + kh) * D + 4 * lane) = pk;
+  }
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void embedding_kernel(const bf16_t* __restrict__ table,
+                                                        const IdT* __restrict__ ids,
+                                                        bf16_t* __restrict__ out, int64_t T, int H,
+                                                        int64_t vocab) {
+  const int64_t t = blockIdx.x;
+  int64_t id = (int64_t)ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const uint4* src = (const uint4*)(table + id * H);
+  uint4* dst = (uint4*)(out + t * H);
+  for (int c = threadIdx.x; c < H / 8; c += 256) dst[c] = src[c];
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int* p, int v, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+}  // namespace vx
+
+using namespace vx;
+
+extern "C" {
+
+int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, const void* k_norm_w,
+                          const void* cos_table, const void* sin_table, const void* positions,
+                          int pos_i64, const int* slot_mapping, void* q_out, void* k_out,
+                          void* k_cache, void* v_cache, int64_t T, int Hq, int Hkv, int D, float eps,
+                          int64_t max_pos, hipStream_t stream) {
+  if (!qkv || !q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || !q_out) return VX_ERR_ARG;
+  if (T < 0 || Hq <= 0 || Hkv <= 0 || max_pos <= 0) return VX_ERR_ARG;
+  if (D != 128 && D != 64) return VX_ERR_UNSUPPORTED;
+  if (ld % 4 != 0) return VX_ERR_UNSUPPORTED;
+  if (T == 0) return VX_OK;
+  const int64_t waves = T * (Hq + 2 * Hkv);
+  const int64_t blocks = (waves + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+#define VX_QK(DD, PT)                                                                          \
+  qk_norm_rope_store_kernel<DD, PT><<<(unsigned)blocks, 256, 0, stream>>>(                     \
+      (const bf16_t*)qkv, ld, (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w,                \
+      (const bf16_t*)cos_table, (const bf16_t*)sin_table, (const PT*)positions, slot_mapping,  \
+      (bf16_t*)q_out, (bf16_t*)k_out, (bf16_t*)k_cache, (bf16_t*)v_cache, T, Hq, Hkv, eps, max_pos)
+  if (D == 128) { if (pos_i64) VX_QK(128, int64_t); else VX_QK(128, int); }
+  else { if (pos_i64) VX_QK(64, int64_t); else VX_QK(64, int); }
+#undef VX_QK
+  return launch_status();
+}
+
+int vx_embedding(const void* table, const void* ids, int ids_i64, void* out, int64_t T, int64_t H,
+                 int64_t vocab, hipStream_t stream) {
+  if (!table || !ids || !out || T < 0 || H <= 0 || vocab <= 0) return VX_ERR_ARG;
+  if (H % 8 != 0 || H > 0x7fffffff) return VX_ERR_UNSUPPORTED;
+  if (T == 0) return VX_OK;
+  if (T > 0x7fffffffLL) return VX_ERR_ARG;
+  if (ids_i64)
+    embedding_kernel<int64_t><<<(unsigned)T, 256, 0, stream>>>((const bf16_t*)table, (const int64_t*)ids,
+                                                               (bf16_t*)out, T, (int)H, vocab);
+  else
+    embedding_kernel<int><<<(unsigned)T, 256, 0, stream>>>((const bf16_t*)table, (const int*)ids,
+                                                           (bf16_t*)out, T, (int)H, vocab);
+  return launch_status();
+}
+
+int vx_fill_i32(int* p, int value, int64_t n, hipStream_t stream) {
+  if (!p || n < 0) return VX_ERR_ARG;
+  if (n == 0) return VX_OK;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  fill_i32_kernel<<<(unsigned)blocks, 256, 0, stream>>>(p, value, n);
+  return launch_status();
+}
+
+const char* vx_status_string(int code) {
+  switch (code) {
+    case VX_OK: return "ok";
+    case VX_ERR_ARG: return "invalid argument (null pointer, negative size or bad stride)";
+    case VX_ERR_UNSUPPORTED: return "unsupported shape, dtype, alignment or layout";
+    case VX_ERR_WORKSPACE: return "workspace too small";
+    case VX_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+int vx_abi_version() { return 1; }
+
+}  // extern "C"

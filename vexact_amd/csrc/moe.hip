@@ -1,0 +1,391 @@
+// Fused MoE block: router top-k, routing integers (histogram, stable expert-major ranks, tile
+// table), grouped expert GEMMs and the slot-ordered combine.
+// Replaces, for the forward pass:
+//   router            vexact/models/qwen3_moe/modeling_qwen3_moe.py:128-134
+//   expert_histogram  vexact/batch_invariant_ops/group_gemm/kernel/moe.py:26-81
+//   argsort().argsort() ranks / _build_moe_indices   vexact/batch_invariant_ops/fused_moe.py:43, 268-292
+//   moe_scatter / moe_gather                          group_gemm/kernel/moe.py:84-161, 253-335
+//   group_gemm_same_nk                                group_gemm/kernel/group_gemm.py:65-237
+//   silu * up * routing-weight glue                   fused_moe.py:75-88
+#include "gemm_core.h"
+
+namespace vx {
+
+// ---------------------------------------------------------------------------------------
+// Router: softmax over E experts in fp32, top-k (ties: lower expert index first), optional
+// renormalisation, cast. One wavefront per token, lane owns experts lane, lane+64, ...
+// ---------------------------------------------------------------------------------------
+constexpr int RT_PER = 8;  // E <= 512
+
+template <bool LOGITS_BF16, bool OUT_BF16, bool IDX64>
+__global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict__ logits,
+                                                          void* __restrict__ weights_out,
+                                                          void* __restrict__ idx_out, int64_t T,
+                                                          int E, int k, int64_t ld, int renorm) {
+  const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tok >= T) return;
+  const int lane = threadIdx.x & 63;
+  float x[RT_PER];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < RT_PER; i++) {
+    const int e = lane + 64 * i;
+    if (e < E) {
+      if constexpr (LOGITS_BF16) x[i] = bf16_to_f32(((const bf16_t*)logits)[tok * ld + e]);
+      else x[i] = ((const float*)logits)[tok * ld + e];
+    } else {
+      x[i] = -INFINITY;
+    }
+    mx = fmaxf(mx, x[i]);
+  }
+  mx = wave_max(mx);
+  float pr[RT_PER];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < RT_PER; i++) {
+    pr[i] = (lane + 64 * i < E) ? expf(x[i] - mx) : 0.f;
+    s += pr[i];
+  }
+  s = wave_sum(s);
+  // k rounds of wave-wide argmax on the logits (same order as on the probabilities)
+  float wsel = 0.f;   // lane j < k keeps the j-th selected probability
+  int isel = 0;
+  float tot = 0.f;
+  for (int j = 0; j < k; j++) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    float bp = 0.f;
+#pragma unroll
+    for (int i = 0; i < RT_PER; i++) {
+      const int e = lane + 64 * i;
+      if (e < E && (x[i] > bv || (x[i] == bv && e < bi))) { bv = x[i]; bi = e; bp = pr[i]; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      const float op = __shfl_xor(bp, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; bp = op; }
+    }
+    // retire the winner
+#pragma unroll
+    for (int i = 0; i < RT_PER; i++)
+      if (lane + 64 * i == bi) x[i] = -INFINITY;
+    const float p = bp / s;
+    tot += p;
+    if (lane == j) { wsel = p; isel = bi; }
+  }
+  if (lane < k) {
+    const float w = renorm ? wsel / tot : wsel;
+    if constexpr (OUT_BF16) ((bf16_t*)weights_out)[tok * k + lane] = f32_to_bf16(w);
+    else ((float*)weights_out)[tok * k + lane] = w;
+    if constexpr (IDX64) ((int64_t*)idx_out)[tok * k + lane] = isel;
+    else ((int*)idx_out)[tok * k + lane] = isel;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Routing integers, one 1024-thread block. For n = T*k flat entries (token-major, slot-minor):
+//   splits[e]         = number of entries routed to expert e
+//   cu[e]             = exclusive prefix of splits (cu[E] = n)
+//   scatter_index[f]  = position of flat entry f in the stable expert-major order
+//   sorted_flat[p]    = f at position p ; sorted_token[p] = f / k
+//   tile table        = for each expert, ceil(splits/bm) row tiles of at most bm rows
+// All integer, order-independent or explicitly ordered: results are exact.
+// ---------------------------------------------------------------------------------------
+constexpr int RB_THREADS = 1024;
+
+template <bool IDX64>
+__global__ __launch_bounds__(RB_THREADS) void moe_route_kernel(
+    const void* __restrict__ idx, int64_t n, int k, int E, int bm, int* __restrict__ splits,
+    int* __restrict__ cu, int* __restrict__ scatter_index, int* __restrict__ sorted_token,
+    int* __restrict__ sorted_flat, int* __restrict__ tile_group, int* __restrict__ tile_row0,
+    int* __restrict__ tile_rows, int max_tiles) {
+  extern __shared__ int sm[];
+  int* hist = sm;             // [E]
+  int* running = sm + E;      // [E]  next free position per expert
+  int* tstart = sm + 2 * E;   // [E]  first tile of expert
+  int* wavecnt = sm + 3 * E;  // [16][E]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  auto expert_of = [&](int64_t f) {
+    int e;
+    if constexpr (IDX64) e = (int)((const int64_t*)idx)[f];
+    else e = ((const int*)idx)[f];
+    return min(max(e, 0), E - 1);  // keeps later address arithmetic in range
+  };
+  for (int e = tid; e < E; e += RB_THREADS) hist[e] = 0;
+  for (int t = tid; t < max_tiles; t += RB_THREADS) { tile_group[t] = -1; tile_row0[t] = 0; tile_rows[t] = 0; }
+  __syncthreads();
+  for (int64_t f = tid; f < n; f += RB_THREADS) atomicAdd(&hist[expert_of(f)], 1);
+  __syncthreads();
+  // exclusive scans by wave 0: lane owns experts [lane*per, lane*per+per)
+  if (wave == 0) {
+    const int per = (E + 63) / 64;
+    int c = 0, tl = 0;
+    for (int i = 0; i < per; i++) {
+      const int e = lane * per + i;
+      if (e < E) { c += hist[e]; tl += (hist[e] + bm - 1) / bm; }
+    }
+    int ci = c, ti = tl;  // inclusive scans across lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int a = __shfl_up(ci, o, 64), b = __shfl_up(ti, o, 64);
+      if (lane >= o) { ci += a; ti += b; }
+    }
+    int cbase = ci - c, tbase = ti - tl;
+    for (int i = 0; i < per; i++) {
+      const int e = lane * per + i;
+      if (e < E) {
+        running[e] = cbase;
+        tstart[e] = tbase;
+        splits[e] = hist[e];
+        cu[e] = cbase;
+        cbase += hist[e];
+        tbase += (hist[e] + bm - 1) / bm;
+      }
+    }
+    if (lane == 63) cu[E] = ci;
+  }
+  __syncthreads();
+  // tile table
+  for (int e = tid; e < E; e += RB_THREADS) {
+    const int cnt = hist[e], r0 = running[e];
+    int t = tstart[e];
+    for (int off = 0; off < cnt; off += bm, t++) {
+      if (t < max_tiles) {
+        tile_group[t] = e;
+        tile_row0[t] = r0 + off;
+        tile_rows[t] = min(bm, cnt - off);
+      }
+    }
+  }
+  // stable ranks, 1024 entries at a time
+  int ebits = 0;
+  while ((1 << ebits) < E) ebits++;
+  for (int64_t base = 0; base < n; base += RB_THREADS) {
+    for (int i = tid; i < 16 * E; i += RB_THREADS) wavecnt[i] = 0;
+    __syncthreads();
+    const int64_t f = base + tid;
+    const bool live = f < n;
+    const int e = live ? expert_of(f) : 0;
+    // lanes of this wave with the same expert
+    uint64_t same = __ballot(live);
+    for (int b = 0; b < ebits; b++) {
+      const uint64_t bal = __ballot((e >> b) & 1);
+      same &= ((e >> b) & 1) ? bal : ~bal;
+    }
+    if (!live) same = 0;
+    const int rank_in_wave = __popcll(same & ((1ull << lane) - 1ull));
+    if (live && rank_in_wave == 0) wavecnt[wave * E + e] = __popcll(same);
+    __syncthreads();
+    for (int ee = tid; ee < E; ee += RB_THREADS) {
+      int r = running[ee];
+      for (int w = 0; w < 16; w++) {
+        const int c = wavecnt[w * E + ee];
+        wavecnt[w * E + ee] = r;
+        r += c;
+      }
+      running[ee] = r;
+    }
+    __syncthreads();
+    if (live) {
+      const int pos = wavecnt[wave * E + e] + rank_in_wave;
+      scatter_index[f] = pos;
+      sorted_flat[pos] = (int)f;
+      sorted_token[pos] = (int)(f / k);
+    }
+    __syncthreads();
+  }
+}
+
+template <bool IDX64>
+__global__ __launch_bounds__(256) void expert_histogram_kernel(const void* __restrict__ idx, int64_t n,
+                                                               int E, int* __restrict__ out) {
+  const int64_t f = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (f >= n) return;
+  int64_t e;
+  if constexpr (IDX64) e = ((const int64_t*)idx)[f];
+  else e = ((const int*)idx)[f];
+  if (e >= 0 && e < E) atomicAdd(&out[e], 1);
+}
+
+__global__ __launch_bounds__(256) void zero_i32_kernel(int* p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// out[index[t, i], :] = x[t, :]; one wavefront per (t, i)
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const bf16_t* __restrict__ x,
+                                                          bf16_t* __restrict__ out,
+                                                          const int* __restrict__ index, int64_t n,
+                                                          int k, int H, int64_t ldx, int64_t ldo) {
+  const int64_t f = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (f >= n) return;
+  const int lane = threadIdx.x & 63;
+  const bf16_t* src = x + (f / k) * ldx;
+  bf16_t* dst = out + (int64_t)index[f] * ldo;
+  for (int c = lane; c < H; c += 64) dst[c] = src[c];
+}
+
+// y[t, :] = r16( sum_{i<k, ascending} f32(x[index[t, i], :]) ); optional residual:
+// y = r16(f32(res[t]) + f32(r16(sum))). One 256-thread block per token.
+__global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restrict__ x,
+                                                         const int* __restrict__ index,
+                                                         const bf16_t* res, bf16_t* y, int k, int H,
+                                                         int64_t ldx, int64_t ldr, int64_t ldy) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += 256) {
+    float acc = 0.f;
+    for (int i = 0; i < k; i++) acc += bf16_to_f32(x[(int64_t)index[t * k + i] * ldx + c]);
+    bf16_t o = f32_to_bf16(acc);
+    if (res) o = f32_to_bf16(bf16_to_f32(res[t * ldr + c]) + bf16_to_f32(o));
+    y[t * ldy + c] = o;
+  }
+}
+
+}  // namespace vx
+
+using namespace vx;
+
+extern "C" {
+
+int vx_router_topk(const void* logits, void* weights_out, void* idx_out, int64_t T, int E, int k,
+                   int64_t ld, int logits_bf16, int out_bf16, int idx_i64, int renorm,
+                   hipStream_t stream) {
+  if (!logits || !weights_out || !idx_out || T < 0 || E <= 0 || k <= 0) return VX_ERR_ARG;
+  if (E > 64 * RT_PER || k > 64 || k > E) return VX_ERR_UNSUPPORTED;
+  if (T == 0) return VX_OK;
+  const int64_t blocks = (T + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+#define VX_RT(LB, OB, I64)                                                                   \
+  router_topk_kernel<LB, OB, I64><<<(unsigned)blocks, 256, 0, stream>>>(logits, weights_out, \
+                                                                        idx_out, T, E, k, ld, renorm)
+  const int sel = (logits_bf16 ? 4 : 0) | (out_bf16 ? 2 : 0) | (idx_i64 ? 1 : 0);
+  switch (sel) {
+    case 0: VX_RT(false, false, false); break;
+    case 1: VX_RT(false, false, true); break;
+    case 2: VX_RT(false, true, false); break;
+    case 3: VX_RT(false, true, true); break;
+    case 4: VX_RT(true, false, false); break;
+    case 5: VX_RT(true, false, true); break;
+    case 6: VX_RT(true, true, false); break;
+    default: VX_RT(true, true, true); break;
+  }
+#undef VX_RT
+  return launch_status();
+}
+
+// upper bound on row tiles: every expert with rows wastes at most one partial tile
+int64_t vx_moe_max_tiles(int64_t n_entries, int E, int bm) {
+  if (n_entries <= 0 || E <= 0 || bm <= 0) return 0;
+  const int64_t a = n_entries < E ? n_entries : E;
+  return a + n_entries / bm;
+}
+
+int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,
+                 int* cu, int* scatter_index, int* sorted_token, int* sorted_flat, int* tile_group,
+                 int* tile_row0, int* tile_rows, int64_t max_tiles, hipStream_t stream) {
+  if (!expert_idx || !splits || !cu || !scatter_index || !sorted_token || !sorted_flat ||
+      !tile_group || !tile_row0 || !tile_rows)
+    return VX_ERR_ARG;
+  if (T < 0 || k <= 0 || E <= 0 || bm <= 0) return VX_ERR_ARG;
+  if (E > 512) return VX_ERR_UNSUPPORTED;
+  const int64_t n = T * k;
+  if (n > 0x7fffffffLL) return VX_ERR_ARG;
+  if (max_tiles < vx_moe_max_tiles(n, E, bm) || max_tiles > 0x7fffffffLL) return VX_ERR_WORKSPACE;
+  const size_t lds = (size_t)(3 + 16) * E * sizeof(int);
+  if (idx_i64)
+    moe_route_kernel<true><<<1, RB_THREADS, lds, stream>>>(expert_idx, n, k, E, bm, splits, cu,
+                                                           scatter_index, sorted_token, sorted_flat,
+                                                           tile_group, tile_row0, tile_rows,
+                                                           (int)max_tiles);
+  else
+    moe_route_kernel<false><<<1, RB_THREADS, lds, stream>>>(expert_idx, n, k, E, bm, splits, cu,
+                                                            scatter_index, sorted_token, sorted_flat,
+                                                            tile_group, tile_row0, tile_rows,
+                                                            (int)max_tiles);
+  return launch_status();
+}
+
+// Grouped GEMM over a tile table: C[rows of tile] = X[row_src[rows]] * W[group]^T.
+// epi 0: plain bf16 store. epi 1: SwiGLU with w = gate rows, w2 = up rows, scaled per row by
+// row_scale[row_scale_idx[row]].  bm in {16, 32, 64} selects the streaming kernel, 128 the tiled one.
+int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64_t ldw,
+                int64_t w_gstride, void* c, int64_t ldc, int64_t N, int64_t K, const int* tile_group,
+                const int* tile_row0, const int* tile_rows, int64_t max_tiles, int bm,
+                const int* row_src, const void* row_scale, const int* row_scale_idx, int epi,
+                hipStream_t stream) {
+  if (!x || !w || !c || !tile_group || !tile_row0 || !tile_rows) return VX_ERR_ARG;
+  if (N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff || max_tiles < 0) return VX_ERR_ARG;
+  if (epi != EPI_PLAIN && epi != EPI_SWIGLU) return VX_ERR_ARG;
+  if (epi == EPI_SWIGLU && (!w2 || !row_scale)) return VX_ERR_ARG;
+  if (!gemm_fast_ok(x, w, K, ldx, ldw) || (w_gstride % 8) != 0) return VX_ERR_UNSUPPORTED;
+  if (epi == EPI_SWIGLU && ((uintptr_t)w2 % 16) != 0) return VX_ERR_UNSUPPORTED;
+  if (max_tiles == 0) return VX_OK;
+  if (max_tiles > 65535) return VX_ERR_UNSUPPORTED;
+  GemmParams p = {};
+  p.x = (const bf16_t*)x; p.ldx = ldx;
+  p.w = (const bf16_t*)w; p.w2 = (const bf16_t*)w2; p.ldw = ldw; p.w_gstride = w_gstride;
+  p.c = (bf16_t*)c; p.ldc = ldc;
+  p.M = 0; p.N = (int)N; p.K = (int)K;
+  p.tile_group = tile_group; p.tile_row0 = tile_row0; p.tile_rows = tile_rows;
+  p.row_src = row_src;
+  p.row_scale = (const bf16_t*)row_scale; p.row_scale_idx = row_scale_idx;
+  const unsigned my = (unsigned)max_tiles;
+#define VX_GG(MT)                                                                                  \
+  do {                                                                                             \
+    const dim3 grid((unsigned)((N + 63) / 64), my);                                                \
+    if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true><<<grid, 256, 0, stream>>>(p);  \
+    else gemm_stream_kernel<MT, EPI_PLAIN, true><<<grid, 256, 0, stream>>>(p);                     \
+  } while (0)
+  switch (bm) {
+    case 16: VX_GG(1); break;
+    case 32: VX_GG(2); break;
+    case 64: VX_GG(4); break;
+    case 128: {
+      if (epi == EPI_SWIGLU)
+        gemm_tiled_kernel<EPI_SWIGLU, true><<<dim3((unsigned)((N + 63) / 64), my), 256, 0, stream>>>(p);
+      else
+        gemm_tiled_kernel<EPI_PLAIN, true><<<dim3((unsigned)((N + 127) / 128), my), 256, 0, stream>>>(p);
+      break;
+    }
+    default: return VX_ERR_ARG;
+  }
+#undef VX_GG
+  return launch_status();
+}
+
+int vx_expert_histogram(const void* idx, int idx_i64, int64_t n, int E, int* out, hipStream_t stream) {
+  if (!idx || !out || n < 0 || E <= 0) return VX_ERR_ARG;
+  zero_i32_kernel<<<(unsigned)((E + 255) / 256), 256, 0, stream>>>(out, E);  // no memset node: stays graph-safe
+  if (n == 0) return VX_OK;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  if (idx_i64) expert_histogram_kernel<true><<<(unsigned)blocks, 256, 0, stream>>>(idx, n, E, out);
+  else expert_histogram_kernel<false><<<(unsigned)blocks, 256, 0, stream>>>(idx, n, E, out);
+  return launch_status();
+}
+
+int vx_moe_scatter(const void* x, void* out, const int* index, int64_t T, int k, int64_t H,
+                   int64_t ldx, int64_t ldo, hipStream_t stream) {
+  if (!x || !out || !index || T < 0 || k <= 0 || H <= 0 || H > 0x7fffffff) return VX_ERR_ARG;
+  const int64_t n = T * k;
+  if (n == 0) return VX_OK;
+  const int64_t blocks = (n + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  moe_scatter_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, index, n,
+                                                           k, (int)H, ldx, ldo);
+  return launch_status();
+}
+
+int vx_moe_gather(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                  int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, hipStream_t stream) {
+  if (!x || !y || !index || T < 0 || k <= 0 || H <= 0 || H > 0x7fffffff) return VX_ERR_ARG;
+  if (T == 0) return VX_OK;
+  if (T > 0x7fffffffLL) return VX_ERR_ARG;
+  moe_gather_kernel<<<(unsigned)T, 256, 0, stream>>>((const bf16_t*)x, index, (const bf16_t*)residual,
+                                                     (bf16_t*)y, k, (int)H, ldx, ldr, ldy);
+  return launch_status();
+}
+
+}  // extern "C"

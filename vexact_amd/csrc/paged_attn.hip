@@ -1,0 +1,570 @@
+// Causal GQA attention over a paged (or packed) KV cache for decode and chunked prefill, plus
+// the KV-cache row scatter.
+// Replaces _paged_attn_fwd_block_kernel / _PagedFlashAttentionVarlen
+// (vexact/batch_invariant_ops/triton_invariant_attention.py:433-692), the forward of the packed
+// twin _varlen_attn_fwd_block_kernel (:47-190, :700-784) and _store_cache_kernel / store_kvcache
+// (vexact/batch_invariant_ops/kv_cache_context.py:259-314).
+//
+// Arithmetic per query row at absolute position p (keys 0..p visible), c = scale * log2(e):
+//   keys are cut into chunks of 256 (absolute positions), each chunk into blocks of 64.
+//   chunk state (m, l, acc) starts at (-inf, 0, 0); for each block, ascending:
+//     t_i = fl(s_i * c), masked keys -> -inf ; m' = max(m, max_i t_i) ; a = exp2(m - m')
+//     pb_i = r16(exp2(t_i - m')) ; acc = acc * a + sum_i pb_i * V_i (bf16 MFMA) ; l = l * a + sum_i pb_i
+//   running state (M, L, ACC) folds the chunks in ascending order:
+//     M' = max(M, m) ; A = exp2(M - M') ; B = exp2(m - M') ; L = L*A + l*B ; ACC = ACC*A + acc*B
+//   out = r16(ACC / L)
+// The decode kernel gives every (sequence, kv head, chunk) to one wavefront, writes the chunk
+// states to a workspace and a second kernel folds them; the prefill kernel does the same fold in
+// registers. Both run the same block routine, so a token's output has the same bits whether it
+// is computed as the last row of a prefill chunk, as a decode step, alone or inside a batch.
+//
+// Layout trick: S is computed transposed (keys on MFMA rows, query rows on MFMA columns), so a
+// lane's 4 results belong to one query row and softmax statistics stay in-lane; the bf16 P
+// values are then already in MFMA B-operand order if the contraction slot (g, idx) of a 32-key
+// chunk is mapped to key 16*(idx/4) + 4*g + idx%4. V rows are fetched in that key order with
+// 16 lanes covering one 256-byte row, and an in-register 8x8 transpose turns 8 rows x 8 dims
+// into 8 A-operand fragments, each feeding the MFMA for dims {8 i + t}.
+#include "common.h"
+
+namespace vx {
+
+constexpr int ATT_CHUNK = 256;  // keys per split chunk (absolute positions)
+constexpr int ATT_BLOCK = 64;   // keys per online-softmax block
+
+struct AttnParams {
+  const bf16_t* q;  // [T, Hq, DK]
+  int64_t sqt, sqh;
+  const bf16_t* k;  // paged: [blocks, page, Hkv, DK]; packed: [Tk, Hkv, DK]
+  int64_t skb, skp, skh;  // packed: skp = row stride, skb unused
+  const bf16_t* v;
+  int64_t svb, svp, svh;
+  bf16_t* o;  // [T, Hq, DV]
+  int64_t sot, soh;
+  const int* cu_q;       // [B+1]
+  const int* seqused_k;  // paged: [B] kv lengths
+  const int* cu_k;       // packed: [B+1]
+  const int* block_table;  // [B, bt_stride]
+  int64_t bt_stride;
+  int page_size, page_shift;  // shift = -1 if not a power of two
+  int Hq, Hkv, num_seqs;
+  float qk_scale;  // scale * log2(e)
+  int causal;
+  // decode split workspace
+  float* part_acc;  // [B, Hq, max_chunks, DV]
+  float* part_ml;   // [B, Hq, max_chunks, 2]
+  int max_chunks;
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+template <int DK, int DV, int QT>
+struct AttnWave {
+  static constexpr int KS = DK / 32;           // MFMA k-steps for S
+  static constexpr int NDV = (DV + 127) / 128;  // sets of 8 PV MFMAs
+  static constexpr int NACC = NDV * 8;
+
+  // per q-tile, per lane (column j = lane % 16)
+  uint4 qf[QT][KS];
+  int qpos[QT];  // last visible key of this lane's query row; -1 = row not valid
+  float m[QT], l[QT];
+  f32x4 acc[QT][NACC];
+
+  __device__ __forceinline__ void reset_chunk() {
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+      m[t] = -INFINITY;
+      l[t] = 0.f;
+#pragma unroll
+      for (int i = 0; i < NACC; i++) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  // One 64-key block at absolute key offset kb. ksrc / vsrc resolve (16-key tile, key within
+  // tile) to the address of that key's row for this kv head.
+  template <typename Rows>
+  __device__ __forceinline__ void block(int kb, int kv_len, float c, Rows& ksrc, Rows& vsrc) {
+    const int lane = threadIdx.x & 63;
+    const int r16 = lane & 15, g = lane >> 4;
+    ksrc.prepare(kb, kv_len);
+    vsrc.prepare(kb, kv_len);
+
+    // ---- issue all K and V loads of the block
+    uint4 kf[4][KS];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++) {
+      const bool ok = kb + 16 * tt + r16 < kv_len;
+      const bf16_t* kp = ksrc.ptr(tt, ok ? r16 : 0) + 8 * g;
+#pragma unroll
+      for (int s = 0; s < KS; s++) kf[tt][s] = ldg16(kp + 32 * s, ok);
+    }
+    uint4 vr[2][NDV][8];  // [32-key chunk][dim set][slot]
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++)
+#pragma unroll
+      for (int idx = 0; idx < 8; idx++) {
+        const int tt = 2 * ch + (idx >> 2), within = 4 * g + (idx & 3);
+        const bool ok = kb + 16 * tt + within < kv_len;
+        const bf16_t* vp = vsrc.ptr(tt, ok ? within : 0);
+#pragma unroll
+        for (int ds = 0; ds < NDV; ds++) {
+          const bool dok = 128 * ds + 8 * r16 < DV;
+          vr[ch][ds][idx] = ldg16(vp + (dok ? 128 * ds + 8 * r16 : 0), ok && dok);
+        }
+      }
+
+    // ---- scores and softmax statistics per query tile
+    uint4 pf[QT][2];
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+      // S^T tiles: lane holds keys kb + 16 tt + 4 g + r for query column r16
+      f32x4 st[4];
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) {
+        st[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; s++) st[tt] = mfma16(kf[tt][s], qf[t][s], st[tt]);
+      }
+      float bm = -INFINITY;
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int key = kb + 16 * tt + 4 * g + r;
+          float tv = st[tt][r] * c;
+          tv = (key <= qpos[t]) ? tv : -INFINITY;
+          st[tt][r] = tv;
+          bm = fmaxf(bm, tv);
+        }
+      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float mn = fmaxf(m[t], bm);
+      const float ms = (mn == -INFINITY) ? 0.f : mn;  // fully masked so far: everything stays 0
+      const float alpha = fast_exp2(m[t] - ms);
+      float rs = 0.f;
+      uint32_t pw[4][2];
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) {
+        float pv[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const bf16_t pb = f32_to_bf16(fast_exp2(st[tt][r] - ms));
+          pv[r] = bf16_to_f32(pb);
+          rs += pv[r];
+        }
+        pw[tt][0] = pack_bf16x2(pv[0], pv[1]);
+        pw[tt][1] = pack_bf16x2(pv[2], pv[3]);
+      }
+      rs += __shfl_xor(rs, 16, 64);
+      rs += __shfl_xor(rs, 32, 64);
+      l[t] = l[t] * alpha + rs;
+      m[t] = mn;
+#pragma unroll
+      for (int i = 0; i < NACC; i++) {
+        acc[t][i][0] *= alpha; acc[t][i][1] *= alpha; acc[t][i][2] *= alpha; acc[t][i][3] *= alpha;
+      }
+      pf[t][0] = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
+      pf[t][1] = make_uint4(pw[2][0], pw[2][1], pw[3][0], pw[3][1]);
+    }
+
+    // ---- P V : out^T[dim 8 i + td][query r16]
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++)
+#pragma unroll
+      for (int ds = 0; ds < NDV; ds++)
+#pragma unroll
+        for (int td = 0; td < 8; td++) {
+          // 8x8 bf16 transpose: fragment td takes dim 8 r16 + td of the 8 key slots
+          uint32_t w[4];
+#pragma unroll
+          for (int qd = 0; qd < 4; qd++) {
+            const uint4 ra = vr[ch][ds][2 * qd], rb = vr[ch][ds][2 * qd + 1];
+            const uint32_t a = (td < 2) ? ra.x : (td < 4) ? ra.y : (td < 6) ? ra.z : ra.w;
+            const uint32_t b = (td < 2) ? rb.x : (td < 4) ? rb.y : (td < 6) ? rb.z : rb.w;
+            w[qd] = (td & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
+          }
+          const uint4 vf = make_uint4(w[0], w[1], w[2], w[3]);
+#pragma unroll
+          for (int t = 0; t < QT; t++) acc[t][ds * 8 + td] = mfma16(vf, pf[t][ch], acc[t][ds * 8 + td]);
+        }
+  }
+};
+
+// fold a chunk state into the running state; exact no-op for an all-masked chunk
+__device__ __forceinline__ void fold_scales(float M, float mc, float& Mn, float& A, float& B) {
+  Mn = fmaxf(M, mc);
+  const float ms = (Mn == -INFINITY) ? 0.f : Mn;
+  A = fast_exp2(M - ms);
+  B = fast_exp2(mc - ms);
+}
+
+// Row sources. prepare() is called once per 64-key block; ptr(tt, within) is the row of key
+// kb + 16 tt + within.
+struct PagedRows {
+  const bf16_t* base;  // cache + kv_head offset
+  const int* bt;       // this sequence's block-table row
+  int64_t sb, sp;
+  int ps, shift;
+  int kb_;
+  int64_t t0, t1, t2, t3;  // fast path (page size a power of two >= 16): a tile lies in one page
+  __device__ __forceinline__ int64_t tile_base(int key, int kv_len) const {
+    const int kk = key < kv_len ? key : 0;  // tiles past the end are never dereferenced
+    return (int64_t)bt[kk >> shift] * sb + (int64_t)(kk & (ps - 1)) * sp;
+  }
+  __device__ __forceinline__ void prepare(int kb, int kv_len) {
+    kb_ = kb;
+    if (shift >= 4) {
+      t0 = tile_base(kb, kv_len);
+      t1 = tile_base(kb + 16, kv_len);
+      t2 = tile_base(kb + 32, kv_len);
+      t3 = tile_base(kb + 48, kv_len);
+    }
+  }
+  __device__ __forceinline__ const bf16_t* ptr(int tt, int within) const {
+    if (shift >= 4) return base + (tt == 0 ? t0 : tt == 1 ? t1 : tt == 2 ? t2 : t3) + (int64_t)within * sp;
+    const int key = kb_ + 16 * tt + within;
+    int pg, off;
+    if (shift >= 0) { pg = key >> shift; off = key & (ps - 1); }
+    else { pg = key / ps; off = key - pg * ps; }
+    return base + (int64_t)bt[pg] * sb + (int64_t)off * sp;
+  }
+};
+struct PackedRows {
+  const bf16_t* base;  // already offset to the sequence's first key and the kv head
+  int64_t sp;
+  int kb_;
+  __device__ __forceinline__ void prepare(int kb, int) { kb_ = kb; }
+  __device__ __forceinline__ const bf16_t* ptr(int tt, int within) const {
+    return base + (int64_t)(kb_ + 16 * tt + within) * sp;
+  }
+};
+
+// ---------------------------------------------------------------------------------------
+// Decode: every sequence has at most one query token. grid = (max_chunks, Hkv, B), one
+// wavefront per block; query heads of the kv head are the MFMA columns (G <= 16 * QT).
+// ---------------------------------------------------------------------------------------
+template <int DK, int DV, int QT>
+__global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
+  const int chunk = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int q0 = p.cu_q[seq];
+  const int qlen = p.cu_q[seq + 1] - q0;
+  const int kv_len = p.seqused_k[seq];
+  if (qlen <= 0 || kv_len <= 0) return;
+  const int kstart = chunk * ATT_CHUNK;
+  if (kstart >= kv_len) return;
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int G = p.Hq / p.Hkv;
+  const int64_t tok = q0 + qlen - 1;  // the (only) query token
+  const int pos = p.causal ? kv_len - 1 : kv_len - 1;
+
+  AttnWave<DK, DV, QT> w;
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int hl = 16 * t + r16;  // head within the group
+    const bool ok = hl < G;
+    w.qpos[t] = ok ? pos : -1;
+    const bf16_t* qp = p.q + tok * p.sqt + (int64_t)(kvh * G + (ok ? hl : 0)) * p.sqh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DK / 32; s++) w.qf[t][s] = ldg16(qp + 32 * s, ok);
+  }
+  w.reset_chunk();
+  PagedRows kr{p.k + (int64_t)kvh * p.skh, p.block_table + (int64_t)seq * p.bt_stride, p.skb, p.skp,
+               p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+  PagedRows vr{p.v + (int64_t)kvh * p.svh, p.block_table + (int64_t)seq * p.bt_stride, p.svb, p.svp,
+               p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+  const int kend = min(kstart + ATT_CHUNK, kv_len);
+  for (int kb = kstart; kb < kend; kb += ATT_BLOCK) w.block(kb, kv_len, p.qk_scale, kr, vr);
+
+  // write the chunk state: lane holds dims 128 ds + 32 g + 8 r + td for head column r16
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int hl = 16 * t + r16;
+    if (hl >= G) continue;
+    const int64_t slot = ((int64_t)seq * p.Hq + kvh * G + hl) * p.max_chunks + chunk;
+    if (g == 0) {
+      p.part_ml[slot * 2] = w.m[t];
+      p.part_ml[slot * 2 + 1] = w.l[t];
+    }
+    float* pa = p.part_acc + slot * DV;
+#pragma unroll
+    for (int ds = 0; ds < (DV + 127) / 128; ds++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int d0 = 128 * ds + 32 * g + 8 * r;
+        if (d0 < DV) {
+          float4 a = make_float4(w.acc[t][ds * 8 + 0][r], w.acc[t][ds * 8 + 1][r],
+                                 w.acc[t][ds * 8 + 2][r], w.acc[t][ds * 8 + 3][r]);
+          float4 b = make_float4(w.acc[t][ds * 8 + 4][r], w.acc[t][ds * 8 + 5][r],
+                                 w.acc[t][ds * 8 + 6][r], w.acc[t][ds * 8 + 7][r]);
+          *(float4*)(pa + d0) = a;
+          *(float4*)(pa + d0 + 4) = b;
+        }
+      }
+  }
+}
+
+// grid = (Hq, B); 64 threads, lane handles dims lane, lane + 64, ...
+template <int DV>
+__global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
+  const int head = blockIdx.x, seq = blockIdx.y;
+  const int q0 = p.cu_q[seq];
+  const int qlen = p.cu_q[seq + 1] - q0;
+  const int kv_len = p.seqused_k[seq];
+  if (qlen <= 0 || kv_len <= 0) return;
+  const int nch = (kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
+  const int64_t slot0 = ((int64_t)seq * p.Hq + head) * p.max_chunks;
+  constexpr int PER = (DV + 63) / 64;
+  float M = -INFINITY, L = 0.f, ACC[PER];
+#pragma unroll
+  for (int i = 0; i < PER; i++) ACC[i] = 0.f;
+  for (int c = 0; c < nch; c++) {
+    const float mc = p.part_ml[(slot0 + c) * 2], lc = p.part_ml[(slot0 + c) * 2 + 1];
+    float Mn, A, B;
+    fold_scales(M, mc, Mn, A, B);
+    L = L * A + lc * B;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int d = threadIdx.x + 64 * i;
+      const float a = (d < DV) ? p.part_acc[(slot0 + c) * DV + d] : 0.f;
+      ACC[i] = ACC[i] * A + a * B;
+    }
+    M = Mn;
+  }
+  const int64_t tok = q0 + qlen - 1;
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    const int d = threadIdx.x + 64 * i;
+    if (d < DV) p.o[tok * p.sot + (int64_t)head * p.soh + d] = f32_to_bf16(ACC[i] / L);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// General (prefill / mixed / packed) kernel. grid = (q tiles, Hq, B); 4 wavefronts per block,
+// wavefront v owns query rows [64 QT bx + 16 QT v, +16 QT) of the sequence (local indices).
+// ---------------------------------------------------------------------------------------
+template <int DK, int DV, int QT, bool PAGED>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
+  const int head = blockIdx.y, seq = blockIdx.z;
+  const int q0 = p.cu_q[seq];
+  const int qlen = p.cu_q[seq + 1] - q0;
+  int kv_len, k0 = 0;
+  if constexpr (PAGED) kv_len = p.seqused_k[seq];
+  else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int i0 = (blockIdx.x * 4 + wave) * 16 * QT;
+  if (qlen <= 0 || kv_len <= 0 || i0 >= qlen) return;
+  const int kvh = head / (p.Hq / p.Hkv);
+  const int shift = kv_len - qlen;  // absolute position of local row 0
+
+  AttnWave<DK, DV, QT> w;
+  int maxpos = -1;
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int i = i0 + 16 * t + r16;
+    const bool ok = i < qlen;
+    const int pos = p.causal ? shift + i : kv_len - 1;
+    w.qpos[t] = (ok && pos >= 0) ? pos : -1;
+    const bf16_t* qp = p.q + (int64_t)(q0 + (ok ? i : 0)) * p.sqt + (int64_t)head * p.sqh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DK / 32; s++) w.qf[t][s] = ldg16(qp + 32 * s, ok);
+    maxpos = max(maxpos, w.qpos[t]);
+  }
+  // wave-uniform last visible key
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) maxpos = max(maxpos, __shfl_xor(maxpos, o, 64));
+
+  float M[QT], L[QT];
+  f32x4 ACC[QT][AttnWave<DK, DV, QT>::NACC];
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    M[t] = -INFINITY; L[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < AttnWave<DK, DV, QT>::NACC; i++) ACC[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  auto run = [&](auto& kr, auto& vr) {
+    for (int cs = 0; cs <= maxpos; cs += ATT_CHUNK) {
+      w.reset_chunk();
+      const int kend = min(cs + ATT_CHUNK, maxpos + 1);
+      for (int kb = cs; kb < kend; kb += ATT_BLOCK) w.block(kb, kv_len, p.qk_scale, kr, vr);
+#pragma unroll
+      for (int t = 0; t < QT; t++) {
+        float Mn, A, B;
+        fold_scales(M[t], w.m[t], Mn, A, B);
+        L[t] = L[t] * A + w.l[t] * B;
+#pragma unroll
+        for (int i = 0; i < AttnWave<DK, DV, QT>::NACC; i++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) ACC[t][i][r] = ACC[t][i][r] * A + w.acc[t][i][r] * B;
+        M[t] = Mn;
+      }
+    }
+  };
+  if constexpr (PAGED) {
+    PagedRows kr{p.k + (int64_t)kvh * p.skh, p.block_table + (int64_t)seq * p.bt_stride, p.skb,
+                 p.skp, p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+    PagedRows vr{p.v + (int64_t)kvh * p.svh, p.block_table + (int64_t)seq * p.bt_stride, p.svb,
+                 p.svp, p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+    run(kr, vr);
+  } else {
+    PackedRows kr{p.k + (int64_t)k0 * p.skp + (int64_t)kvh * p.skh, p.skp, 0};
+    PackedRows vr{p.v + (int64_t)k0 * p.svp + (int64_t)kvh * p.svh, p.svp, 0};
+    run(kr, vr);
+  }
+
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int i = i0 + 16 * t + r16;
+    if (i >= qlen) continue;
+    bf16_t* op = p.o + (int64_t)(q0 + i) * p.sot + (int64_t)head * p.soh;
+    const bool dead = w.qpos[t] < 0;  // no visible key: define the output as 0
+#pragma unroll
+    for (int ds = 0; ds < (DV + 127) / 128; ds++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int d0 = 128 * ds + 32 * g + 8 * r;
+        if (d0 < DV) {
+          uint32_t pk[4];
+#pragma unroll
+          for (int h = 0; h < 4; h++) {
+            const float a = dead ? 0.f : ACC[t][ds * 8 + 2 * h][r] / L[t];
+            const float b = dead ? 0.f : ACC[t][ds * 8 + 2 * h + 1][r] / L[t];
+            pk[h] = pack_bf16x2(a, b);
+          }
+          *(uint4*)(op + d0) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// KV-cache scatter: cache.view(-1, row)[slot[t]] = src[t] for slot != -1. One wavefront per token
+// copies row_bytes (multiple of 16) with 16-byte accesses.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void store_kv_kernel(const uint8_t* __restrict__ ksrc,
+                                                       const uint8_t* __restrict__ vsrc,
+                                                       uint8_t* __restrict__ kc, uint8_t* __restrict__ vc,
+                                                       const int* __restrict__ slots, int64_t ntok,
+                                                       int64_t ks_stride, int64_t vs_stride,
+                                                       int k_row_bytes, int v_row_bytes) {
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= ntok) return;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const int lane = threadIdx.x & 63;
+  for (int b = lane * 16; b < k_row_bytes; b += 64 * 16)
+    *(uint4*)(kc + (int64_t)slot * k_row_bytes + b) = *(const uint4*)(ksrc + t * ks_stride + b);
+  if (vsrc)
+    for (int b = lane * 16; b < v_row_bytes; b += 64 * 16)
+      *(uint4*)(vc + (int64_t)slot * v_row_bytes + b) = *(const uint4*)(vsrc + t * vs_stride + b);
+}
+
+template <int DK, int DV>
+static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hipStream_t stream) {
+  if (mode == 0) {  // decode split + combine
+    const int G = p.Hq / p.Hkv;
+    dim3 grid(p.max_chunks, p.Hkv, p.num_seqs);
+    if (G <= 16) attn_decode_split_kernel<DK, DV, 1><<<grid, 64, 0, stream>>>(p);
+    else if (G <= 32) attn_decode_split_kernel<DK, DV, 2><<<grid, 64, 0, stream>>>(p);
+    else return VX_ERR_UNSUPPORTED;
+    attn_decode_combine_kernel<DV><<<dim3(p.Hq, p.num_seqs), 64, 0, stream>>>(p);
+  } else {
+    constexpr int QT = (DK > 192) ? 1 : 2;
+    const int rows = max_q > 0 ? max_q : total_q;
+    dim3 grid((rows + 64 * QT - 1) / (64 * QT), p.Hq, p.num_seqs);
+    if (mode == 1) attn_prefill_kernel<DK, DV, QT, true><<<grid, 256, 0, stream>>>(p);
+    else attn_prefill_kernel<DK, DV, QT, false><<<grid, 256, 0, stream>>>(p);
+  }
+  return launch_status();
+}
+
+}  // namespace vx
+
+using namespace vx;
+
+extern "C" {
+
+int vx_attn_chunk_size() { return ATT_CHUNK; }
+
+// bytes of workspace the decode path needs
+int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Dv,
+                                             int64_t max_kv_len) {
+  const int64_t nch = (max_kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
+  return num_seqs * Hq * nch * (Dv + 2) * 4;
+}
+
+// mode: 0 = paged decode (every sequence has <= 1 query token; needs workspace),
+//       1 = paged general (prefill / mixed), 2 = packed K/V (cu_seqlens_k, no page table).
+int vx_attention(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens_q,
+                 const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                 int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                 int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
+                 int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
+                 int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
+                 int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  if (!q || !k || !v || !out || !cu_seqlens_q) return VX_ERR_ARG;
+  if (total_q < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return VX_ERR_ARG;
+  if (mode < 0 || mode > 2) return VX_ERR_ARG;
+  if (mode != 2 && (!seqused_k || !block_table || page_size <= 0 || max_pages <= 0)) return VX_ERR_ARG;
+  if (mode == 2 && !cu_seqlens_k) return VX_ERR_ARG;
+  if (mode == 0 && !causal) return VX_ERR_UNSUPPORTED;
+  if (total_q == 0 || num_seqs == 0) return VX_OK;
+  if (num_seqs > 65535 || Hq > 65535) return VX_ERR_UNSUPPORTED;
+  // 16-byte row accesses
+  if ((sqt | sqh | skb | skp | skh | svb | svp | svh | sot | soh) % 8 != 0) return VX_ERR_UNSUPPORTED;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16 != 0) return VX_ERR_UNSUPPORTED;
+  AttnParams p = {};
+  p.q = (const bf16_t*)q; p.sqt = sqt; p.sqh = sqh;
+  p.k = (const bf16_t*)k; p.skb = skb; p.skp = skp; p.skh = skh;
+  p.v = (const bf16_t*)v; p.svb = svb; p.svp = svp; p.svh = svh;
+  p.o = (bf16_t*)out; p.sot = sot; p.soh = soh;
+  p.cu_q = cu_seqlens_q; p.seqused_k = seqused_k; p.cu_k = cu_seqlens_k;
+  p.block_table = block_table; p.bt_stride = bt_stride;
+  p.page_size = page_size;
+  p.page_shift = -1;
+  if (page_size > 0 && (page_size & (page_size - 1)) == 0) {
+    int s = 0;
+    while ((1 << s) < page_size) s++;
+    p.page_shift = s;
+  }
+  p.Hq = Hq; p.Hkv = Hkv; p.num_seqs = (int)num_seqs;
+  p.qk_scale = softmax_scale * 1.44269504f;
+  p.causal = causal;
+  if (mode == 0) {
+    const int64_t max_kv = max_pages * (int64_t)page_size;
+    const int64_t nch = (max_kv + ATT_CHUNK - 1) / ATT_CHUNK;
+    if (nch > 0x7fffffff) return VX_ERR_ARG;
+    const int64_t need = num_seqs * Hq * nch * (Dv + 2) * 4;
+    if (!workspace || workspace_bytes < need) return VX_ERR_WORKSPACE;
+    p.max_chunks = (int)nch;
+    p.part_acc = (float*)workspace;
+    p.part_ml = (float*)workspace + num_seqs * Hq * nch * Dv;
+  }
+  const int tq = (int)total_q;
+  if (Dk == 128 && Dv == 128) return launch_attn<128, 128>(p, mode, max_seqlen_q, tq, stream);
+  if (Dk == 64 && Dv == 64) return launch_attn<64, 64>(p, mode, max_seqlen_q, tq, stream);
+  if (Dk == 32 && Dv == 32) return launch_attn<32, 32>(p, mode, max_seqlen_q, tq, stream);
+  if (Dk == 192 && Dv == 128) return launch_attn<192, 128>(p, mode, max_seqlen_q, tq, stream);
+  if (Dk == 256 && Dv == 256) return launch_attn<256, 256>(p, mode, max_seqlen_q, tq, stream);
+  return VX_ERR_UNSUPPORTED;
+}
+
+// cache.view(-1, Hkv*D)[slot] = src[t]; value may be null (store one tensor only)
+int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_cache,
+                     const int* slot_mapping, int64_t num_tokens, int64_t k_src_stride_bytes,
+                     int64_t v_src_stride_bytes, int64_t k_row_bytes, int64_t v_row_bytes,
+                     hipStream_t stream) {
+  if (!key || !k_cache || !slot_mapping || num_tokens < 0) return VX_ERR_ARG;
+  if (value && !v_cache) return VX_ERR_ARG;
+  if (num_tokens == 0) return VX_OK;
+  if (k_row_bytes % 16 != 0 || k_src_stride_bytes % 16 != 0 || k_row_bytes > 0x7fffffff) return VX_ERR_UNSUPPORTED;
+  if (value && (v_row_bytes % 16 != 0 || v_src_stride_bytes % 16 != 0 || v_row_bytes > 0x7fffffff)) return VX_ERR_UNSUPPORTED;
+  if (((uintptr_t)key | (uintptr_t)k_cache | (uintptr_t)value | (uintptr_t)v_cache) % 16 != 0) return VX_ERR_UNSUPPORTED;
+  const int64_t blocks = (num_tokens + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  store_kv_kernel<<<(unsigned)blocks, 256, 0, stream>>>(
+      (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping,
+      num_tokens, k_src_stride_bytes, v_src_stride_bytes, (int)k_row_bytes, (int)v_row_bytes);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,424 @@
+// Row-wise reductions: mean over one dim, RMSNorm (two rounding variants, optional fused
+// residual add), log_softmax, per-token logprob and greedy argmax.
+//
+// All of them are HBM-bound. One row is always reduced by one fixed-size thread group whose
+// size depends on the row length only; a thread owns the 4-element vectors t, t+G, t+2G, ...
+// and adds their elements in ascending order, then a lane butterfly and an ascending
+// wave-order pass finish the sum. The schedule never looks at the number of rows.
+#include "common.h"
+#include <math.h>
+
+namespace vx {
+
+enum : int { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
+
+template <int DT> struct Elem;
+template <> struct Elem<DT_F32> {
+  using T = float;
+  static __device__ __forceinline__ float ld(const T* p) { return *p; }
+  static __device__ __forceinline__ void st(T* p, float v) { *p = v; }
+};
+template <> struct Elem<DT_BF16> {
+  using T = bf16_t;
+  static __device__ __forceinline__ float ld(const T* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void st(T* p, float v) { *p = f32_to_bf16(v); }
+};
+template <> struct Elem<DT_F16> {
+  using T = _Float16;
+  static __device__ __forceinline__ float ld(const T* p) { return (float)*p; }
+  static __device__ __forceinline__ void st(T* p, float v) { *p = (_Float16)v; }
+};
+
+// ---------------------------------------------------------------------------------------
+// mean over the middle dim of an (M, N, K) strided view.
+// Replaces mean_kernel / mean_dim (vexact/batch_invariant_ops/batch_invariant_ops.py:336-473).
+// G threads per output element: 64 when N <= 512, else 256.
+// ---------------------------------------------------------------------------------------
+template <int DT, int G>
+__global__ __launch_bounds__(256) void mean_dim_kernel(const typename Elem<DT>::T* __restrict__ in,
+                                                       typename Elem<DT>::T* __restrict__ out,
+                                                       int64_t s0, int64_t s1, int64_t s2,
+                                                       int64_t o0, int64_t o1, int64_t M, int64_t N,
+                                                       int64_t K) {
+  __shared__ float red[4];
+  constexpr int RPB = 256 / G;  // output elements per block
+  const int sub = threadIdx.x / G;
+  const int t = threadIdx.x % G;
+  const int64_t oid = (int64_t)blockIdx.x * RPB + sub;
+  const bool live = oid < M * K;
+  float acc = 0.f;
+  if (live) {
+    const int64_t m = oid / K, k = oid % K;
+    const typename Elem<DT>::T* base = in + m * s0 + k * s2;
+    for (int64_t v = t; v * 4 < N; v += G) {
+      const int64_t n0 = v * 4;
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+        if (n0 + c < N) acc += Elem<DT>::ld(base + (n0 + c) * s1);
+    }
+  }
+  float tot;
+  if constexpr (G == 64) tot = wave_sum(acc);
+  else tot = block_sum<4>(acc, red);
+  if (live && t == 0) {
+    const int64_t m = oid / K, k = oid % K;
+    Elem<DT>::st(out + m * o0 + k * o1, tot / (float)N);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// RMSNorm over the last dim of [rows, n].
+// mode 0: y = r16(f32(x) * inv * f32(w)), inv = 1/sqrt(ss/n + eps)  -- one rounding;
+//         replaces _rms_norm_kernel (batch_invariant_ops.py:637-669).
+// mode 1: y = r16(f32(w) * f32(r16(f32(x) * inv)))                  -- the two-rounding form a
+//         HuggingFace Qwen3 RMSNorm produces when its .mean(-1) runs through mean_dim.
+// If res != nullptr the row is first replaced by r16(x + res) (a bf16 residual add) and that
+// sum is also written to sum_out.
+// ---------------------------------------------------------------------------------------
+template <int DT, int G>
+__global__ __launch_bounds__(256) void rms_norm_kernel(
+    const typename Elem<DT>::T* x, const typename Elem<DT>::T* res,
+    const typename Elem<DT>::T* __restrict__ w, typename Elem<DT>::T* y,
+    typename Elem<DT>::T* sum_out, int64_t rows, int n, int64_t xs, int64_t rs,
+    int64_t ys, int64_t ss, float eps, int mode) {
+  using E = Elem<DT>;
+  __shared__ float red[4];
+  constexpr int RPB = 256 / G;
+  const int sub = threadIdx.x / G;
+  const int t = threadIdx.x % G;
+  const int64_t row = (int64_t)blockIdx.x * RPB + sub;
+  const bool live = row < rows;
+  const typename E::T* xr = x + row * xs;
+  const typename E::T* rr = res ? res + row * rs : nullptr;
+  typename E::T* so = sum_out ? sum_out + row * ss : nullptr;
+  float acc = 0.f;
+  if (live) {
+    for (int v = t; v * 4 < n; v += G) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int j = v * 4 + c;
+        if (j < n) {
+          float f = E::ld(xr + j);
+          if (rr) {
+            // round the residual sum to the storage type before it is used
+            typename E::T tmp;
+            E::st(&tmp, f + E::ld(rr + j));
+            f = E::ld(&tmp);
+            if (so) so[j] = tmp;
+          }
+          acc += f * f;
+        }
+      }
+    }
+  }
+  float tot;
+  if constexpr (G == 64) tot = wave_sum(acc);
+  else tot = block_sum<4>(acc, red);
+  if (!live) return;
+  const float inv = 1.0f / sqrtf(tot / (float)n + eps);
+  typename E::T* yr = y + row * ys;
+  for (int v = t; v * 4 < n; v += G) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const int j = v * 4 + c;
+      if (j < n) {
+        float f;
+        if (rr && so) {
+          f = E::ld(so + j);  // written by this thread above; safe when sum_out aliases x or res
+        } else {
+          f = E::ld(xr + j);
+          if (rr) {
+            typename E::T tmp;
+            E::st(&tmp, f + E::ld(rr + j));
+            f = E::ld(&tmp);
+          }
+        }
+        const float wf = E::ld(w + j);
+        if (mode == 0) {
+          E::st(yr + j, f * inv * wf);
+        } else {
+          typename E::T tmp;
+          E::st(&tmp, f * inv);
+          E::st(yr + j, wf * E::ld(&tmp));
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// log_softmax / logprob / argmax over rows of [rows, n], split into fixed chunks of
+// LS_CHUNK columns so that few rows still fill the chip. The chunk count depends on n only.
+// Pass 1 writes per (row, chunk): max m_c, s_c = sum exp(x - m_c), and the first index of
+// the max. Pass 2 folds the partials in ascending chunk order:
+//   m = max_c m_c ; S = sum_c s_c * exp(m_c - m) ; y = (x - m) - log(S).
+// Replaces _log_softmax_kernel / log_softmax (batch_invariant_ops.py:231-333) and the
+// cross-entropy call behind logprobs_from_logits_flash_attn (standalone_logprobs.py:28-55).
+// ---------------------------------------------------------------------------------------
+constexpr int LS_CHUNK = 4096;
+constexpr int LS_THREADS = 256;
+constexpr int LS_PER = LS_CHUNK / LS_THREADS;  // 16 values per thread
+
+struct LsPartial {
+  float m;
+  float s;
+  int idx;
+  int pad;
+};
+
+template <int DT>
+__device__ __forceinline__ void ls_load(const typename Elem<DT>::T* row, int n, int c0, float* v) {
+  // thread t owns vectors t, t+256, t+512, t+768 of the chunk (4 elements each)
+#pragma unroll
+  for (int j = 0; j < LS_PER / 4; j++) {
+    const int e0 = c0 + 4 * (threadIdx.x + LS_THREADS * j);
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[4 * j + c] = (e0 + c < n) ? Elem<DT>::ld(row + e0 + c) : -INFINITY;
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(LS_THREADS) void ls_partial_kernel(
+    const typename Elem<DT>::T* __restrict__ x, LsPartial* __restrict__ part, int n, int64_t xs,
+    int nchunk) {
+  __shared__ float red[4];
+  __shared__ int redi[4];
+  const int64_t row = blockIdx.y;
+  const int ch = blockIdx.x;
+  const int c0 = ch * LS_CHUNK;
+  float v[LS_PER];
+  ls_load<DT>(x + row * xs, n, c0, v);
+  float m = v[0];
+  int mi = 0;
+#pragma unroll
+  for (int i = 1; i < LS_PER; i++)
+    if (v[i] > m) { m = v[i]; mi = i; }
+  // element index of this thread's local max
+  int idx = c0 + 4 * (threadIdx.x + LS_THREADS * (mi / 4)) + (mi % 4);
+  const float bm = block_max<4>(m, red);
+  // first index holding the block max
+  int cand = (m == bm) ? idx : 0x7fffffff;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o, 64));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) redi[threadIdx.x >> 6] = cand;
+  __syncthreads();
+  cand = min(min(redi[0], redi[1]), min(redi[2], redi[3]));
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < LS_PER; i++) s += (v[i] == -INFINITY) ? 0.f : expf(v[i] - bm);  // padded tail adds 0
+  const float bs = block_sum<4>(s, red);
+  if (threadIdx.x == 0) {
+    LsPartial p;
+    p.m = bm; p.s = bs; p.idx = cand; p.pad = 0;
+    part[row * nchunk + ch] = p;
+  }
+}
+
+__device__ __forceinline__ void ls_fold(const LsPartial* __restrict__ p, int nchunk, float& m,
+                                        float& logS, int& amax) {
+  m = p[0].m;
+  amax = p[0].idx;
+  for (int c = 1; c < nchunk; c++)
+    if (p[c].m > m) { m = p[c].m; amax = p[c].idx; }
+  float S = 0.f;
+  for (int c = 0; c < nchunk; c++) S += p[c].s * expf(p[c].m - m);
+  logS = logf(S);
+}
+
+template <int DT>
+__global__ __launch_bounds__(LS_THREADS) void ls_final_kernel(
+    const typename Elem<DT>::T* __restrict__ x, typename Elem<DT>::T* __restrict__ y,
+    const LsPartial* __restrict__ part, int n, int64_t xs, int64_t ys, int nchunk) {
+  const int64_t row = blockIdx.y;
+  const int c0 = blockIdx.x * LS_CHUNK;
+  float m, logS;
+  int amax;
+  ls_fold(part + row * nchunk, nchunk, m, logS, amax);
+  const typename Elem<DT>::T* xr = x + row * xs;
+  typename Elem<DT>::T* yr = y + row * ys;
+#pragma unroll
+  for (int j = 0; j < LS_PER / 4; j++) {
+    const int e0 = c0 + 4 * (threadIdx.x + LS_THREADS * j);
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+      if (e0 + c < n) Elem<DT>::st(yr + e0 + c, (Elem<DT>::ld(xr + e0 + c) - m) - logS);
+  }
+}
+
+// out[row] = (x[row, label] - m) - log S ; when labels == nullptr the greedy token (first
+// argmax) is used and also written to tok_out.
+template <int DT>
+__global__ __launch_bounds__(64) void logprob_final_kernel(
+    const typename Elem<DT>::T* __restrict__ x, const int64_t* __restrict__ labels,
+    const LsPartial* __restrict__ part, float* __restrict__ out, int64_t* __restrict__ tok_out,
+    int64_t rows, int n, int64_t xs, int nchunk) {
+  const int64_t row = (int64_t)blockIdx.x * 64 + threadIdx.x;
+  if (row >= rows) return;
+  float m, logS;
+  int amax;
+  ls_fold(part + row * nchunk, nchunk, m, logS, amax);
+  int64_t lab = labels ? labels[row] : (int64_t)amax;
+  if (tok_out) tok_out[row] = lab;
+  float r = NAN;
+  if (lab >= 0 && lab < n) r = (Elem<DT>::ld(x + row * xs + lab) - m) - logS;
+  out[row] = r;
+}
+
+}  // namespace vx
+
+using namespace vx;
+
+extern "C" {
+
+int vx_mean_dim(const void* in, void* out, int dtype, int64_t M, int64_t N, int64_t K, int64_t s0,
+                int64_t s1, int64_t s2, int64_t o0, int64_t o1, hipStream_t stream) {
+  if (!in || !out || M < 0 || N <= 0 || K < 0) return VX_ERR_ARG;
+  const int64_t outs = M * K;
+  if (outs == 0) return VX_OK;
+  const bool small = N <= 512;
+  const int64_t rpb = small ? 4 : 1;
+  const int64_t blocks = (outs + rpb - 1) / rpb;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+#define VX_LAUNCH_MEAN(DT)                                                                      \
+  do {                                                                                          \
+    using T = Elem<DT>::T;                                                                      \
+    if (small)                                                                                  \
+      mean_dim_kernel<DT, 64><<<dim3((unsigned)blocks), 256, 0, stream>>>(                      \
+          (const T*)in, (T*)out, s0, s1, s2, o0, o1, M, N, K);                                  \
+    else                                                                                        \
+      mean_dim_kernel<DT, 256><<<dim3((unsigned)blocks), 256, 0, stream>>>(                     \
+          (const T*)in, (T*)out, s0, s1, s2, o0, o1, M, N, K);                                  \
+  } while (0)
+  switch (dtype) {
+    case DT_F32: VX_LAUNCH_MEAN(DT_F32); break;
+    case DT_BF16: VX_LAUNCH_MEAN(DT_BF16); break;
+    case DT_F16: VX_LAUNCH_MEAN(DT_F16); break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+#undef VX_LAUNCH_MEAN
+  return launch_status();
+}
+
+int vx_rms_norm(const void* x, const void* residual, const void* weight, void* y, void* sum_out,
+                int dtype, int64_t rows, int64_t n, int64_t x_stride, int64_t res_stride,
+                int64_t y_stride, int64_t sum_stride, float eps, int mode, hipStream_t stream) {
+  if (!x || !weight || !y || rows < 0 || n <= 0 || n > 0x7fffffff) return VX_ERR_ARG;
+  if (mode != 0 && mode != 1) return VX_ERR_ARG;
+  if (rows == 0) return VX_OK;
+  const bool small = n <= 512;
+  const int64_t rpb = small ? 4 : 1;
+  const int64_t blocks = (rows + rpb - 1) / rpb;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+#define VX_LAUNCH_RMS(DT)                                                                       \
+  do {                                                                                          \
+    using T = Elem<DT>::T;                                                                      \
+    if (small)                                                                                  \
+      rms_norm_kernel<DT, 64><<<dim3((unsigned)blocks), 256, 0, stream>>>(                      \
+          (const T*)x, (const T*)residual, (const T*)weight, (T*)y, (T*)sum_out, rows, (int)n,  \
+          x_stride, res_stride, y_stride, sum_stride, eps, mode);                               \
+    else                                                                                        \
+      rms_norm_kernel<DT, 256><<<dim3((unsigned)blocks), 256, 0, stream>>>(                     \
+          (const T*)x, (const T*)residual, (const T*)weight, (T*)y, (T*)sum_out, rows, (int)n,  \
+          x_stride, res_stride, y_stride, sum_stride, eps, mode);                               \
+  } while (0)
+  switch (dtype) {
+    case DT_F32: VX_LAUNCH_RMS(DT_F32); break;
+    case DT_BF16: VX_LAUNCH_RMS(DT_BF16); break;
+    case DT_F16: VX_LAUNCH_RMS(DT_F16); break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+#undef VX_LAUNCH_RMS
+  return launch_status();
+}
+
+int64_t vx_log_softmax_workspace_bytes(int64_t rows, int64_t n) {
+  if (rows < 0 || n <= 0) return 0;
+  const int64_t nchunk = (n + LS_CHUNK - 1) / LS_CHUNK;
+  return rows * nchunk * (int64_t)sizeof(LsPartial);
+}
+
+static int ls_partials(const void* x, int dtype, int64_t rows, int64_t n, int64_t xs, void* ws,
+                       int64_t ws_bytes, hipStream_t stream, int* nchunk_out) {
+  if (!x || !ws || rows < 0 || n <= 0 || n > 0x7fffffff - LS_CHUNK) return VX_ERR_ARG;
+  if (rows > 65535) return VX_ERR_UNSUPPORTED;  // grid.y limit; callers split larger batches
+  const int nchunk = (int)((n + LS_CHUNK - 1) / LS_CHUNK);
+  if (ws_bytes < rows * nchunk * (int64_t)sizeof(LsPartial)) return VX_ERR_WORKSPACE;
+  *nchunk_out = nchunk;
+  if (rows == 0) return VX_OK;
+  dim3 grid(nchunk, (unsigned)rows);
+  switch (dtype) {
+    case DT_F32:
+      ls_partial_kernel<DT_F32><<<grid, LS_THREADS, 0, stream>>>((const float*)x, (LsPartial*)ws,
+                                                                 (int)n, xs, nchunk);
+      break;
+    case DT_BF16:
+      ls_partial_kernel<DT_BF16><<<grid, LS_THREADS, 0, stream>>>((const bf16_t*)x, (LsPartial*)ws,
+                                                                  (int)n, xs, nchunk);
+      break;
+    case DT_F16:
+      ls_partial_kernel<DT_F16><<<grid, LS_THREADS, 0, stream>>>((const _Float16*)x,
+                                                                 (LsPartial*)ws, (int)n, xs, nchunk);
+      break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+int vx_log_softmax(const void* x, void* y, int dtype, int64_t rows, int64_t n, int64_t x_stride,
+                   int64_t y_stride, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  if (!y) return VX_ERR_ARG;
+  int nchunk = 0;
+  int rc = ls_partials(x, dtype, rows, n, x_stride, workspace, workspace_bytes, stream, &nchunk);
+  if (rc != VX_OK || rows == 0) return rc;
+  dim3 grid(nchunk, (unsigned)rows);
+  const LsPartial* part = (const LsPartial*)workspace;
+  switch (dtype) {
+    case DT_F32:
+      ls_final_kernel<DT_F32><<<grid, LS_THREADS, 0, stream>>>((const float*)x, (float*)y, part,
+                                                               (int)n, x_stride, y_stride, nchunk);
+      break;
+    case DT_BF16:
+      ls_final_kernel<DT_BF16><<<grid, LS_THREADS, 0, stream>>>(
+          (const bf16_t*)x, (bf16_t*)y, part, (int)n, x_stride, y_stride, nchunk);
+      break;
+    case DT_F16:
+      ls_final_kernel<DT_F16><<<grid, LS_THREADS, 0, stream>>>(
+          (const _Float16*)x, (_Float16*)y, part, (int)n, x_stride, y_stride, nchunk);
+      break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* tokens_out,
+                int dtype, int64_t rows, int64_t n, int64_t x_stride, void* workspace,
+                int64_t workspace_bytes, hipStream_t stream) {
+  if (!out) return VX_ERR_ARG;
+  int nchunk = 0;
+  int rc = ls_partials(logits, dtype, rows, n, x_stride, workspace, workspace_bytes, stream, &nchunk);
+  if (rc != VX_OK || rows == 0) return rc;
+  const unsigned blocks = (unsigned)((rows + 63) / 64);
+  const LsPartial* part = (const LsPartial*)workspace;
+  switch (dtype) {
+    case DT_F32:
+      logprob_final_kernel<DT_F32><<<blocks, 64, 0, stream>>>((const float*)logits, labels, part, out,
+                                                              tokens_out, rows, (int)n, x_stride,
+                                                              nchunk);
+      break;
+    case DT_BF16:
+      logprob_final_kernel<DT_BF16><<<blocks, 64, 0, stream>>>((const bf16_t*)logits, labels, part,
+                                                               out, tokens_out, rows, (int)n,
+                                                               x_stride, nchunk);
+      break;
+    case DT_F16:
+      logprob_final_kernel<DT_F16><<<blocks, 64, 0, stream>>>((const _Float16*)logits, labels, part,
+                                                              out, tokens_out, rows, (int)n,
+                                                              x_stride, nchunk);
+      break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,630 @@
+"""Torch-tensor front end of the C ABI: argument validation, output allocation, launches.
+
+Every function here takes and returns ``torch`` tensors that live on the GPU and launches on
+``torch.cuda.current_stream()``. Nothing falls back to PyTorch arithmetic: if the HIP library is
+missing the call raises.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need_gpu(name: str, t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a CUDA tensor")
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+# ----------------------------------------------------------------------------- row ops
+
+
+def mean_dim(x: torch.Tensor, dim: int, keepdim: bool = False, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    _need_gpu("input", x)
+    assert -x.ndim <= dim < x.ndim, f"Invalid dimension {dim} for tensor with {x.ndim} dimensions"
+    if dim < 0:
+        dim += x.ndim
+    if dtype is None:
+        dtype = torch.float32 if x.dtype in (torch.int8, torch.int16, torch.int32, torch.int64) else x.dtype
+    if x.dtype != dtype:
+        x = x.to(dtype)
+    if dtype not in _DT:
+        raise ValueError(f"mean_dim: unsupported dtype {dtype}")
+    shape = list(x.shape)
+    M = 1
+    for s in shape[:dim]:
+        M *= s
+    N = shape[dim]
+    K = 1
+    for s in shape[dim + 1 :]:
+        K *= s
+    out_shape = shape.copy()
+    if keepdim:
+        out_shape[dim] = 1
+    else:
+        out_shape = shape[:dim] + shape[dim + 1 :]
+    out = torch.empty(out_shape, dtype=dtype, device=x.device)
+    if M * K == 0:
+        return out
+    if N == 0:
+        return out.fill_(float("nan"))
+    x3 = x.reshape(M, N, K)
+    _lib.check(
+        _lib.load().vx_mean_dim(
+            x3.data_ptr(), out.data_ptr(), _DT[dtype], M, N, K, x3.stride(0), x3.stride(1), x3.stride(2), K, 1, _stream()
+        ),
+        "vx_mean_dim",
+    )
+    return out
+
+
+def rms_norm(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    eps: float = 1e-6,
+    *,
+    hf_two_rounding: bool = False,
+    residual: Optional[torch.Tensor] = None,
+    sum_out: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """RMSNorm over the last dim. With ``residual`` the row becomes ``x + residual`` first (rounded
+    to the storage dtype) and that sum is written to ``sum_out`` when given."""
+    _need_gpu("input", x)
+    if x.dtype not in _DT:
+        raise ValueError(f"rms_norm: unsupported dtype {x.dtype}")
+    n = x.shape[-1]
+    x2 = x.reshape(-1, n)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    w = weight.contiguous()
+    if w.dtype != x.dtype:
+        w = w.to(x.dtype)
+    assert w.numel() == n, "weight must have the size of the last dim"
+    y = out if out is not None else torch.empty((x2.shape[0], n), dtype=x.dtype, device=x.device)
+    y2 = y.reshape(-1, n)
+    r2 = s2 = None
+    if residual is not None:
+        r2 = residual.reshape(-1, n)
+        assert r2.dtype == x.dtype and r2.stride(-1) == 1 and r2.shape == x2.shape
+        if sum_out is not None:
+            s2 = sum_out.reshape(-1, n)
+            assert s2.dtype == x.dtype and s2.stride(-1) == 1 and s2.shape == x2.shape
+    _lib.check(
+        _lib.load().vx_rms_norm(
+            x2.data_ptr(), _ptr(r2), w.data_ptr(), y2.data_ptr(), _ptr(s2), _DT[x.dtype], x2.shape[0], n,
+            x2.stride(0), r2.stride(0) if r2 is not None else 0, y2.stride(0),
+            s2.stride(0) if s2 is not None else 0, float(eps), 1 if hf_two_rounding else 0, _stream(),
+        ),
+        "vx_rms_norm",
+    )
+    return y.reshape(x.shape) if out is None else out
+
+
+def log_softmax(x: torch.Tensor, dim: int = -1) -> torch.Tensor:
+    if dim != -1 and dim != x.ndim - 1:
+        raise ValueError("This implementation only supports log_softmax along the last dimension")
+    _need_gpu("input", x)
+    if x.dtype not in _DT:
+        raise ValueError(f"log_softmax: unsupported dtype {x.dtype}")
+    shape = x.shape
+    x2 = x.reshape(-1, shape[-1]).contiguous()
+    rows, n = x2.shape
+    y = torch.empty_like(x2)
+    if rows == 0 or n == 0:
+        return y.reshape(shape)
+    lib = _lib.load()
+    step = 65535  # grid.y limit
+    for r0 in range(0, rows, step):
+        r = min(step, rows - r0)
+        ws = _workspace(lib.vx_log_softmax_workspace_bytes(r, n), x.device)
+        _lib.check(
+            lib.vx_log_softmax(
+                x2[r0:].data_ptr(), y[r0:].data_ptr(), _DT[x.dtype], r, n, x2.stride(0), y.stride(0),
+                ws.data_ptr(), ws.numel(), _stream(),
+            ),
+            "vx_log_softmax",
+        )
+    return y.reshape(shape)
+
+
+def logprobs(
+    logits: torch.Tensor, labels: Optional[torch.Tensor], *, return_tokens: bool = False
+):
+    """Per-row ``logits[i, labels[i]] - logsumexp(logits[i])`` in fp32. ``labels=None`` scores the
+    greedy (first-argmax) token and can return it."""
+    _need_gpu("logits", logits)
+    if logits.dtype not in _DT:
+        raise ValueError(f"logprobs: unsupported dtype {logits.dtype}")
+    x2 = logits.reshape(-1, logits.shape[-1])
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    rows, n = x2.shape
+    out = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    toks = torch.empty(rows, dtype=torch.int64, device=logits.device) if (return_tokens or labels is None) else None
+    lab = None
+    if labels is not None:
+        lab = labels.reshape(-1)
+        if lab.dtype != torch.int64:
+            lab = lab.to(torch.int64)
+        lab = lab.contiguous()
+        assert lab.numel() == rows, "labels must have one entry per row"
+    if rows == 0:
+        return (out, toks) if return_tokens else out
+    lib = _lib.load()
+    step = 65535
+    for r0 in range(0, rows, step):
+        r = min(step, rows - r0)
+        ws = _workspace(lib.vx_log_softmax_workspace_bytes(r, n), logits.device)
+        _lib.check(
+            lib.vx_logprobs(
+                x2[r0:].data_ptr(), _ptr(lab[r0:]) if lab is not None else None, out[r0:].data_ptr(),
+                _ptr(toks[r0:]) if toks is not None else None, _DT[logits.dtype], r, n, x2.stride(0),
+                ws.data_ptr(), ws.numel(), _stream(),
+            ),
+            "vx_logprobs",
+        )
+    return (out, toks) if return_tokens else out
+
+
+# ----------------------------------------------------------------------------- GEMM
+
+
+def _fast_ok(x: torch.Tensor, w_nk: torch.Tensor) -> bool:
+    K = x.shape[1]
+    return (
+        x.dtype == torch.bfloat16
+        and w_nk.dtype == torch.bfloat16
+        and x.stride(1) == 1
+        and w_nk.stride(1) == 1
+        and K % 8 == 0
+        and x.stride(0) % 8 == 0
+        and w_nk.stride(0) % 8 == 0
+        and x.data_ptr() % 16 == 0
+        and w_nk.data_ptr() % 16 == 0
+    )
+
+
+def gemm_nt(
+    x: torch.Tensor, w_nk: torch.Tensor, bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None
+) -> torch.Tensor:
+    """``x[M,K] @ w_nk[N,K].T (+ bias)`` in bf16 on the MFMA path (raises if the layout does not fit)."""
+    M, K = x.shape
+    N = w_nk.shape[0]
+    c = out if out is not None else torch.empty((M, N), dtype=x.dtype, device=x.device)
+    assert c.stride(1) == 1
+    _lib.check(
+        _lib.load().vx_gemm_bf16_nt(
+            x.data_ptr(), w_nk.data_ptr(), _ptr(bias), c.data_ptr(), M, N, K, x.stride(0), w_nk.stride(0),
+            c.stride(0), _stream(),
+        ),
+        "vx_gemm_bf16_nt",
+    )
+    return c
+
+
+def gemm_nt_variant(x: torch.Tensor, w_nk: torch.Tensor, kind: int, mt: int = 1, bias=None) -> torch.Tensor:
+    M, K = x.shape
+    N = w_nk.shape[0]
+    c = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    _lib.check(
+        _lib.load().vx_gemm_bf16_nt_variant(
+            x.data_ptr(), w_nk.data_ptr(), _ptr(bias), c.data_ptr(), M, N, K, x.stride(0), w_nk.stride(0),
+            c.stride(0), kind, mt, _stream(),
+        ),
+        "vx_gemm_bf16_nt_variant",
+    )
+    return c
+
+
+def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``a[M,K] @ b[K,N] (+ bias[N])`` with the dtype of ``a``; any strides.
+
+    bf16 operands go through the MFMA kernels: directly when ``b`` is a transposed view of an
+    ``[N, K]`` row-major weight (the ``nn.Linear`` case), after packing ``b`` otherwise. Other dtypes
+    and unaligned layouts use the generic one-thread-per-output kernel. The choice depends on dtype
+    and layout only, never on M.
+    """
+    assert a.ndim == 2 and b.ndim == 2, "matmul expects 2-D operands"
+    assert a.shape[1] == b.shape[0], "Incompatible dimensions"
+    assert a.dtype == b.dtype, "Incompatible dtypes"
+    assert bias is None or bias.dim() == 1, "Currently assuming bias is 1D, let Horace know if you run into this"
+    _need_gpu("a", a)
+    if a.dtype not in _DT:
+        raise ValueError(f"matmul: unsupported dtype {a.dtype}")
+    M, K = a.shape
+    N = b.shape[1]
+    if bias is not None:
+        bias = bias.to(a.dtype).contiguous()
+    c = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    if M == 0 or N == 0:
+        return c
+    if K == 0:
+        c.zero_()
+        if bias is not None:
+            c += bias
+        return c
+    lib = _lib.load()
+    if a.dtype == torch.bfloat16 and K % 8 == 0:
+        w_nk = b.t()  # [N, K] view
+        x = a
+        if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+            x = a.contiguous()
+        if w_nk.stride(1) != 1 or w_nk.stride(0) % 8 != 0 or w_nk.data_ptr() % 16 != 0:
+            # pack b[K, N] (any strides) into an [N, K] row-major buffer
+            bc = b if b.stride(1) == 1 else b.contiguous()
+            packed = torch.empty((N, K), dtype=b.dtype, device=b.device)
+            _lib.check(
+                lib.vx_transpose_bf16(bc.data_ptr(), packed.data_ptr(), K, N, bc.stride(0), K, _stream()),
+                "vx_transpose_bf16",
+            )
+            w_nk = packed
+        if _fast_ok(x, w_nk):
+            return gemm_nt(x, w_nk, bias, out=c)
+    _lib.check(
+        lib.vx_gemm_generic(
+            a.data_ptr(), b.data_ptr(), _ptr(bias), c.data_ptr(), _DT[a.dtype], 1, M, N, K,
+            0, a.stride(0), a.stride(1), 0, b.stride(0), b.stride(1), 0, c.stride(0), c.stride(1), _stream(),
+        ),
+        "vx_gemm_generic",
+    )
+    return c
+
+
+def bmm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    assert a.ndim == 3 and b.ndim == 3, f"Expected 3D tensors, got {a.ndim}D and {b.ndim}D"
+    B, M, K = a.shape
+    _, K2, N = b.shape
+    assert K == K2 and a.shape[0] == b.shape[0]
+    _need_gpu("a", a)
+    if a.dtype not in _DT or a.dtype != b.dtype:
+        raise ValueError(f"bmm: unsupported dtypes {a.dtype}, {b.dtype}")
+    c = torch.empty((B, M, N), dtype=a.dtype, device=a.device)
+    if c.numel() == 0:
+        return c
+    lib = _lib.load()
+    step = 65535
+    for b0 in range(0, B, step):
+        nb = min(step, B - b0)
+        _lib.check(
+            lib.vx_gemm_generic(
+                a[b0:].data_ptr(), b[b0:].data_ptr(), None, c[b0:].data_ptr(), _DT[a.dtype], nb, M, N, K,
+                a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
+                c.stride(0), c.stride(1), c.stride(2), _stream(),
+            ),
+            "vx_gemm_generic",
+        )
+    return c
+
+
+# ----------------------------------------------------------------------------- KV cache + attention
+
+
+def store_kvcache(key, value, k_cache, v_cache, slot_mapping) -> None:
+    assert slot_mapping.numel() == key.shape[0]
+    for name, t, cache in (("key", key, k_cache), ("value", value, v_cache)):
+        N, H, D = t.shape
+        assert t.stride(-1) == 1
+        assert t.stride(1) == D
+        assert cache.stride(1) == H * D, f"Cache stride mismatch: expected stride(1)={H * D}, got {cache.stride(1)}"
+        assert cache.dtype == t.dtype, f"{name} and its cache must share a dtype"
+    if slot_mapping.dtype != torch.int32:
+        raise ValueError(f"slot_mapping must have dtype torch.int32, got {slot_mapping.dtype}")
+    es = key.element_size()
+    _lib.check(
+        _lib.load().vx_store_kvcache(
+            key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
+            key.shape[0], key.stride(0) * es, value.stride(0) * es, key.shape[1] * key.shape[2] * es,
+            value.shape[1] * value.shape[2] * es, _stream(),
+        ),
+        "vx_store_kvcache",
+    )
+
+
+def paged_attention(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    seqused_k: torch.Tensor,
+    page_table: torch.Tensor,
+    softmax_scale: float,
+    max_seqlen_q: int = 0,
+    out: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Causal paged attention. ``max_seqlen_q == 1`` selects the split-KV decode kernels; any other
+    value the general kernel (identical bits per row)."""
+    T, Hq, Dk = q.shape
+    Hkv, Dv = k_cache.shape[2], v_cache.shape[-1]
+    o = out if out is not None else torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
+    if T == 0:
+        return o
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise ValueError("paged attention supports bfloat16 q/k/v only")
+    if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1:
+        raise ValueError("q, k and v must be contiguous in the head dimension")
+    lib = _lib.load()
+    B = seqused_k.numel()
+    page = k_cache.shape[1]
+    max_pages = page_table.shape[1]
+    mode = 0 if max_seqlen_q == 1 else 1
+    ws = None
+    if mode == 0:
+        need = lib.vx_paged_attn_decode_workspace_bytes(B, Hq, Dv, max_pages * page)
+        ws = workspace if workspace is not None and workspace.numel() * workspace.element_size() >= need else _workspace(need, q.device)
+    _lib.check(
+        lib.vx_attention(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr(), cu_seqlens_q.data_ptr(),
+            seqused_k.data_ptr(), None, page_table.data_ptr(), T, B, Hq, Hkv, Dk, Dv,
+            q.stride(0), q.stride(1), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+            v_cache.stride(0), v_cache.stride(1), v_cache.stride(2), o.stride(0), o.stride(1),
+            page_table.stride(0), max_pages, page, float(softmax_scale), 1, mode, int(max_seqlen_q),
+            _ptr(ws), ws.numel() * ws.element_size() if ws is not None else 0, _stream(),
+        ),
+        "vx_attention",
+    )
+    return o
+
+
+def packed_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    softmax_scale: float,
+    causal: bool,
+    max_seqlen_q: int = 0,
+) -> torch.Tensor:
+    """Varlen attention on packed (non-paged) K/V ``[Tk, Hkv, D]``; same arithmetic as the paged path."""
+    T, Hq, Dk = q.shape
+    Hkv, Dv = k.shape[1], v.shape[-1]
+    o = torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
+    if T == 0:
+        return o
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise ValueError("attention supports bfloat16 q/k/v only")
+    B = cu_seqlens_q.numel() - 1
+    _lib.check(
+        _lib.load().vx_attention(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), cu_seqlens_q.data_ptr(), None,
+            cu_seqlens_k.data_ptr(), None, T, B, Hq, Hkv, Dk, Dv, q.stride(0), q.stride(1),
+            0, k.stride(0), k.stride(1), 0, v.stride(0), v.stride(1), o.stride(0), o.stride(1),
+            0, 0, 0, float(softmax_scale), 1 if causal else 0, 2, int(max_seqlen_q), None, 0, _stream(),
+        ),
+        "vx_attention",
+    )
+    return o
+
+
+# ----------------------------------------------------------------------------- MoE
+
+
+def router_topk(
+    logits: torch.Tensor, top_k: int, renorm: bool = True, out_dtype: torch.dtype = torch.bfloat16,
+    index_dtype: torch.dtype = torch.int64,
+):
+    """softmax(fp32) -> top-k (ties: lower expert index first) -> renorm -> cast."""
+    _need_gpu("logits", logits)
+    T, E = logits.shape
+    if logits.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("router logits must be float32 or bfloat16")
+    if out_dtype not in (torch.float32, torch.bfloat16) or index_dtype not in (torch.int32, torch.int64):
+        raise ValueError("unsupported router output dtypes")
+    lg = logits if logits.stride(1) == 1 else logits.contiguous()
+    w = torch.empty((T, top_k), dtype=out_dtype, device=logits.device)
+    idx = torch.empty((T, top_k), dtype=index_dtype, device=logits.device)
+    _lib.check(
+        _lib.load().vx_router_topk(
+            lg.data_ptr(), w.data_ptr(), idx.data_ptr(), T, E, top_k, lg.stride(0),
+            int(lg.dtype == torch.bfloat16), int(out_dtype == torch.bfloat16), int(index_dtype == torch.int64),
+            int(renorm), _stream(),
+        ),
+        "vx_router_topk",
+    )
+    return w, idx
+
+
+def moe_tile_rows(num_tokens: int) -> int:
+    """Rows per expert tile, chosen from the token count only (any choice gives the same bits)."""
+    if num_tokens <= 256:
+        return 32
+    if num_tokens <= 1024:
+        return 64
+    return 128
+
+
+class MoeRouting:
+    """Device-side routing integers produced by ``vx_moe_route``."""
+
+    __slots__ = ("splits", "cu", "scatter_index", "sorted_token", "sorted_flat", "tile_group", "tile_row0",
+                 "tile_rows", "max_tiles", "bm", "T", "k", "E")
+
+
+def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int] = None, buffers=None) -> MoeRouting:
+    _need_gpu("selected_experts", selected_experts)
+    assert selected_experts.dtype in (torch.int32, torch.int64)
+    idx = selected_experts.contiguous()
+    T, k = idx.shape
+    bm = bm or moe_tile_rows(T)
+    lib = _lib.load()
+    max_tiles = lib.vx_moe_max_tiles(T * k, num_experts, bm)
+    dev = idx.device
+    r = MoeRouting()
+    r.T, r.k, r.E, r.bm, r.max_tiles = T, k, num_experts, bm, max_tiles
+    n = T * k
+    if buffers is None:
+        ints = torch.empty(num_experts + (num_experts + 1) + 3 * n + 3 * max_tiles, dtype=torch.int32, device=dev)
+    else:
+        ints = buffers
+    o = 0
+    r.splits = ints[o : o + num_experts]; o += num_experts
+    r.cu = ints[o : o + num_experts + 1]; o += num_experts + 1
+    r.scatter_index = ints[o : o + n].view(T, k); o += n
+    r.sorted_token = ints[o : o + n]; o += n
+    r.sorted_flat = ints[o : o + n]; o += n
+    r.tile_group = ints[o : o + max_tiles]; o += max_tiles
+    r.tile_row0 = ints[o : o + max_tiles]; o += max_tiles
+    r.tile_rows = ints[o : o + max_tiles]; o += max_tiles
+    _lib.check(
+        lib.vx_moe_route(
+            idx.data_ptr(), int(idx.dtype == torch.int64), T, k, num_experts, bm, r.splits.data_ptr(),
+            r.cu.data_ptr(), r.scatter_index.data_ptr(), r.sorted_token.data_ptr(), r.sorted_flat.data_ptr(),
+            r.tile_group.data_ptr(), r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), max_tiles, _stream(),
+        ),
+        "vx_moe_route",
+    )
+    return r
+
+
+def moe_gemm(
+    x: torch.Tensor, w: torch.Tensor, routing: MoeRouting, *, w2: Optional[torch.Tensor] = None,
+    row_src: Optional[torch.Tensor] = None, row_scale: Optional[torch.Tensor] = None,
+    row_scale_idx: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Grouped GEMM over ``routing``'s tile table. ``w`` is ``[E, N, K]`` (a view with contiguous K is
+    fine). With ``w2`` the SwiGLU epilogue is fused and ``row_scale`` is required."""
+    E, N, K = w.shape
+    n_rows = routing.T * routing.k
+    assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert x.stride(1) == 1 and w.stride(2) == 1
+    if w2 is not None:
+        assert w2.shape == w.shape and w2.stride() == w.stride() and row_scale is not None
+    c = out if out is not None else torch.empty((n_rows, N), dtype=torch.bfloat16, device=x.device)
+    _lib.check(
+        _lib.load().vx_moe_gemm(
+            x.data_ptr(), x.stride(0), w.data_ptr(), _ptr(w2), w.stride(1), w.stride(0), c.data_ptr(), c.stride(0),
+            N, K, routing.tile_group.data_ptr(), routing.tile_row0.data_ptr(), routing.tile_rows.data_ptr(),
+            routing.max_tiles, routing.bm, _ptr(row_src), _ptr(row_scale), _ptr(row_scale_idx),
+            1 if w2 is not None else 0, _stream(),
+        ),
+        "vx_moe_gemm",
+    )
+    return c
+
+
+def expert_histogram(idx: torch.Tensor, num_bins: int) -> torch.Tensor:
+    assert idx.is_cuda
+    assert idx.dtype == torch.int32 or idx.dtype == torch.int64
+    assert idx.numel() < (1 << 31) - 1, "Too many elements."
+    flat = idx.flatten().contiguous()
+    out = torch.empty(num_bins, dtype=torch.int32, device=idx.device)
+    _lib.check(
+        _lib.load().vx_expert_histogram(flat.data_ptr(), int(flat.dtype == torch.int64), flat.numel(), num_bins,
+                                        out.data_ptr(), _stream()),
+        "vx_expert_histogram",
+    )
+    return out
+
+
+def moe_scatter(x: torch.Tensor, index: torch.Tensor, out_dtype=None) -> torch.Tensor:
+    assert x.is_cuda and index.is_cuda
+    assert x.shape[0] == index.shape[0]
+    assert x.device == index.device, f"x.device = {x.device}, index.device = {index.device}"
+    if x.dtype != torch.bfloat16 or (out_dtype or x.dtype) != torch.bfloat16:
+        raise ValueError("moe_scatter supports bfloat16 only")
+    M, N = x.shape
+    topk = index.shape[1]
+    idx = index.to(torch.int32).contiguous()
+    xs = x if x.stride(1) == 1 else x.contiguous()
+    out = torch.empty(M * topk, N, dtype=x.dtype, device=x.device)
+    _lib.check(
+        _lib.load().vx_moe_scatter(xs.data_ptr(), out.data_ptr(), idx.data_ptr(), M, topk, N, xs.stride(0),
+                                   out.stride(0), _stream()),
+        "vx_moe_scatter",
+    )
+    return out
+
+
+def moe_gather(x: torch.Tensor, index: torch.Tensor, out_dtype=None, residual: Optional[torch.Tensor] = None,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    assert x.is_cuda and index.is_cuda
+    M, topk = index.shape
+    assert x.shape[0] == M * topk
+    assert x.device == index.device, f"x.device = {x.device}, index.device = {index.device}"
+    if x.dtype != torch.bfloat16 or (out_dtype or x.dtype) != torch.bfloat16:
+        raise ValueError("moe_gather supports bfloat16 only")
+    N = x.shape[1]
+    idx = index if (index.dtype == torch.int32 and index.is_contiguous()) else index.to(torch.int32).contiguous()
+    xs = x if x.stride(1) == 1 else x.contiguous()
+    y = out if out is not None else torch.empty(M, N, dtype=x.dtype, device=x.device)
+    _lib.check(
+        _lib.load().vx_moe_gather(xs.data_ptr(), idx.data_ptr(), _ptr(residual), y.data_ptr(), M, topk, N,
+                                  xs.stride(0), residual.stride(0) if residual is not None else 0, y.stride(0),
+                                  _stream()),
+        "vx_moe_gather",
+    )
+    return y
+
+
+def fused_moe(
+    hidden_states: torch.Tensor,
+    routing_weights: torch.Tensor,
+    selected_experts: torch.Tensor,
+    gate_w: torch.Tensor,
+    up_w: torch.Tensor,
+    down_w: torch.Tensor,
+    num_experts: int,
+    residual: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Router outputs -> expert SwiGLU MLPs -> slot-ordered combine, four launches:
+    routing integers, gate/up grouped GEMM with gather-on-load and fused SiLU*up*weight,
+    down grouped GEMM, fp32 slot-order sum."""
+    T, H = hidden_states.shape
+    k = selected_experts.shape[1]
+    x = hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous()
+    rw = routing_weights.contiguous()
+    r = moe_route(selected_experts, num_experts)
+    hw = moe_gemm(x, gate_w, r, w2=up_w, row_src=r.sorted_token, row_scale=rw, row_scale_idx=r.sorted_flat)
+    o = moe_gemm(hw, down_w, r)
+    return moe_gather(o, r.scatter_index, residual=residual, out=out)
+
+
+# ----------------------------------------------------------------------------- decoder glue
+
+
+def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, cos_table, sin_table, positions, slot_mapping, q_out,
+                       k_cache, v_cache, Hq: int, Hkv: int, D: int, eps: float, k_out=None) -> None:
+    T = qkv.shape[0]
+    assert qkv.stride(1) == 1 and qkv.shape[1] == (Hq + 2 * Hkv) * D
+    assert positions.dtype in (torch.int32, torch.int64)
+    _lib.check(
+        _lib.load().vx_qk_norm_rope_store(
+            qkv.data_ptr(), qkv.stride(0), q_norm_w.data_ptr(), k_norm_w.data_ptr(), cos_table.data_ptr(),
+            sin_table.data_ptr(), positions.data_ptr(), int(positions.dtype == torch.int64), _ptr(slot_mapping),
+            q_out.data_ptr(), _ptr(k_out), _ptr(k_cache), _ptr(v_cache), T, Hq, Hkv, D, float(eps),
+            cos_table.shape[0], _stream(),
+        ),
+        "vx_qk_norm_rope_store",
+    )
+
+
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    T = ids.numel()
+    vocab, H = table.shape
+    o = out if out is not None else torch.empty((T, H), dtype=table.dtype, device=table.device)
+    _lib.check(
+        _lib.load().vx_embedding(table.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64), o.data_ptr(), T, H,
+                                 vocab, _stream()),
+        "vx_embedding",
+    )
+    return o
