@@ -204,7 +204,7 @@ struct PagedRows {
   const int* bt;       // this sequence's block-table row
   int64_t sb, sp;
   int ps, shift;
-  int kb_;
+  int kb_, last_;  // block start; last existing key (addresses are clamped to it)
   int64_t t0, t1, t2, t3;  // fast path (page size a power of two >= 16): a tile lies in one page
   __device__ __forceinline__ int64_t tile_base(int key, int kv_len) const {
     const int kk = key < kv_len ? key : 0;  // tiles past the end are never dereferenced
@@ -212,6 +212,7 @@ struct PagedRows {
   }
   __device__ __forceinline__ void prepare(int kb, int kv_len) {
     kb_ = kb;
+    last_ = kv_len - 1;
     if (shift >= 4) {
       t0 = tile_base(kb, kv_len);
       t1 = tile_base(kb + 16, kv_len);
@@ -221,7 +222,7 @@ struct PagedRows {
   }
   __device__ __forceinline__ const bf16_t* ptr(int tt, int within) const {
     if (shift >= 4) return base + (tt == 0 ? t0 : tt == 1 ? t1 : tt == 2 ? t2 : t3) + (int64_t)within * sp;
-    const int key = kb_ + 16 * tt + within;
+    const int key = min(kb_ + 16 * tt + within, last_);  // never index the table past the sequence
     int pg, off;
     if (shift >= 0) { pg = key >> shift; off = key & (ps - 1); }
     else { pg = key / ps; off = key - pg * ps; }
@@ -231,10 +232,11 @@ struct PagedRows {
 struct PackedRows {
   const bf16_t* base;  // already offset to the sequence's first key and the kv head
   int64_t sp;
-  int kb_;
-  __device__ __forceinline__ void prepare(int kb, int) { kb_ = kb; }
+  int kb_, last_;
+  __device__ __forceinline__ void prepare(int kb, int kv_len) { kb_ = kb; last_ = kv_len - 1; }
   __device__ __forceinline__ const bf16_t* ptr(int tt, int within) const {
-    return base + (int64_t)(kb_ + 16 * tt + within) * sp;
+    // clamp: a tile past the sequence's last key must not point past the packed tensor
+    return base + (int64_t)min(kb_ + 16 * tt + within, last_) * sp;
   }
 };
 
@@ -268,9 +270,9 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
   }
   w.reset_chunk();
   PagedRows kr{p.k + (int64_t)kvh * p.skh, p.block_table + (int64_t)seq * p.bt_stride, p.skb, p.skp,
-               p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+               p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
   PagedRows vr{p.v + (int64_t)kvh * p.svh, p.block_table + (int64_t)seq * p.bt_stride, p.svb, p.svp,
-               p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+               p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
   const int kend = min(kstart + ATT_CHUNK, kv_len);
   for (int kb = kstart; kb < kend; kb += ATT_BLOCK) w.block(kb, kv_len, p.qk_scale, kr, vr);
 
@@ -401,13 +403,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
   };
   if constexpr (PAGED) {
     PagedRows kr{p.k + (int64_t)kvh * p.skh, p.block_table + (int64_t)seq * p.bt_stride, p.skb,
-                 p.skp, p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+                 p.skp, p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
     PagedRows vr{p.v + (int64_t)kvh * p.svh, p.block_table + (int64_t)seq * p.bt_stride, p.svb,
-                 p.svp, p.page_size, p.page_shift, 0, 0, 0, 0, 0};
+                 p.svp, p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
     run(kr, vr);
   } else {
-    PackedRows kr{p.k + (int64_t)k0 * p.skp + (int64_t)kvh * p.skh, p.skp, 0};
-    PackedRows vr{p.v + (int64_t)k0 * p.svp + (int64_t)kvh * p.svh, p.svp, 0};
+    PackedRows kr{p.k + (int64_t)k0 * p.skp + (int64_t)kvh * p.skh, p.skp, 0, 0};
+    PackedRows vr{p.v + (int64_t)k0 * p.svp + (int64_t)kvh * p.svh, p.svp, 0, 0};
     run(kr, vr);
   }
 
