@@ -49,8 +49,8 @@ def test_router_topk_indices_exact(T, E, k, logit_dtype):
         assert idx.dtype == idt and w.dtype == torch.bfloat16
         # rows where the oracle's fp32 probabilities collide for distinct logits are excluded
         p = torch.softmax(logits.float(), -1)
-        srt = torch.sort(p, -1, descending=True, stable=True).values
-        lsrt = torch.sort(logits.float(), -1, descending=True, stable=True).values
+        srt = torch.sort(p, dim=-1, descending=True, stable=True).values
+        lsrt = torch.sort(logits.float(), dim=-1, descending=True, stable=True).values
         clean = ~(((srt[:, : k + 1][:, 1:] == srt[:, :k]) & (lsrt[:, : k + 1][:, 1:] != lsrt[:, :k])).any(-1))
         assert clean.float().mean() > 0.99
         assert torch.equal(idx.cpu().long()[clean], i_ref[clean]), "top-k indices"
