@@ -19,6 +19,16 @@ def router_ref(router_logits: torch.Tensor, top_k: int, renorm: bool = True, out
     return w.to(out_dtype), order
 
 
+def router_weights_for(router_logits: torch.Tensor, idx: torch.Tensor, renorm: bool = True, out_dtype=torch.bfloat16):
+    """Routing weights for a GIVEN expert choice (same softmax / renormalise / cast as router_ref).
+    Used when a test forces the oracle onto the routing another implementation chose at a near-tie."""
+    probs = F.softmax(router_logits, dim=1, dtype=torch.float32)
+    w = probs.gather(-1, idx.to(torch.int64))
+    if renorm:
+        w = w / w.sum(dim=-1, keepdim=True)
+    return w.to(out_dtype)
+
+
 def routing_integers_ref(selected_experts, num_experts: int):
     """splits, cumulative offsets, stable expert-major rank of every (token, slot), and the inverse
     order (vexact/batch_invariant_ops/group_gemm/kernel/moe.py:26-49 histogram;

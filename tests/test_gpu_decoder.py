@@ -1,0 +1,169 @@
+"""GPU parity of the whole decoder step: a tiny Qwen3-MoE-shaped model against the CPU oracle,
+batch-1 vs batch-N logprob bits, prefill vs decode bits, and HIP-graph replay (padded bucket)
+vs eager (the assertions of tests/test_inferencer.py:300-595, atol = 0)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import decoder as OD
+from tests.util import assert_bf16_close, assert_bitwise
+
+pytestmark = pytest.mark.gpu
+
+from vexact_amd.decoder import (  # noqa: E402
+    DecoderWeights,
+    Qwen3MoeDecoder,
+    build_step_metadata,
+    rope_tables,
+    tiny_config,
+)
+
+
+def _setup(num_seqs=5, seed=3, layers=2):
+    cfg = tiny_config(num_layers=layers)
+    w = DecoderWeights(cfg, device="cuda", seed=seed, std=0.05)
+    rng = np.random.default_rng(seed)
+    prompt_lens = rng.integers(5, 300, size=num_seqs)
+    prompts = [rng.integers(0, cfg.vocab_size, size=n) for n in prompt_lens]
+    pages = [(n + 2 + cfg.page_size - 1) // cfg.page_size for n in prompt_lens]
+    perm = rng.permutation(sum(pages) + 7)
+    blocks, o = [], 0
+    for p in pages:
+        blocks.append(perm[o : o + p].tolist())
+        o += p
+    dec = Qwen3MoeDecoder(cfg, w, num_cache_blocks=len(perm))
+    return cfg, w, dec, prompts, blocks
+
+
+def _prefill(dec, cfg, prompts, blocks, which, routing_log=None):
+    reqs = [dict(num_computed_tokens=len(prompts[s]), tokens_this_step=len(prompts[s]), block_ids=blocks[s]) for s in which]
+    meta = build_step_metadata(reqs, cfg.page_size, (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size)
+    ids = np.concatenate([prompts[s] for s in which])
+    b = dec.bucket(len(ids), len(which))
+    b.load(meta, ids)
+    dec.step(b, meta["max_seqlen_q"], routing_log)
+    torch.cuda.synchronize()
+    return b.tokens.cpu().clone(), b.logprobs.cpu().clone(), meta, ids
+
+
+def _decode_meta(cfg, prompts, blocks, which):
+    reqs = [dict(num_computed_tokens=len(prompts[s]) + 1, tokens_this_step=1, block_ids=blocks[s]) for s in which]
+    return build_step_metadata(reqs, cfg.page_size, (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size)
+
+
+def _check_routing_report(report, what):
+    # the oracle may only be forced across near-ties: a few bf16 ulps of the router logits
+    tot = sum(r["tokens"] for r in report)
+    dif = sum(r["differ"] for r in report)
+    print(f"{what}: routing differed on {dif} of {tot} (token, layer) pairs; "
+          f"largest logit gap crossed {max(r['max_gap'] for r in report):.4f}")
+    assert dif <= 0.1 * tot, f"{what}: routing differs on too many tokens"
+    assert max(r["max_gap_rel"] for r in report) <= 0.05 or max(r["max_gap"] for r in report) <= 0.05, (
+        f"{what}: forced routing crossed a logit gap that is not a near-tie")
+
+
+def test_tiny_decoder_matches_cpu_oracle_and_is_batch_invariant():
+    cfg, w, dec, prompts, blocks = _setup()
+    allseq = list(range(len(prompts)))
+    rlog = []
+    tok, lp, meta, ids = _prefill(dec, cfg, prompts, blocks, allseq, rlog)
+
+    # CPU oracle on the same input bits, following the GPU's expert choice at near-ties
+    wc = w.to_cpu()
+    cos, sin = rope_tables(cfg, "cpu")
+    kc = [torch.zeros_like(t, device="cpu") for t in dec.key_cache]
+    vc = [torch.zeros_like(t, device="cpu") for t in dec.value_cache]
+    report = []
+    logits_ref, _, _ = OD.decoder_step_ref(cfg, wc, ids, meta, kc, vc, cos, sin, [r.cpu() for r in rlog], report)
+    _check_routing_report(report, "prefill")
+    lp_at_gpu_tok = torch.log_softmax(logits_ref.float(), -1).gather(-1, tok.view(-1, 1)).squeeze(-1)
+    assert (lp - lp_at_gpu_tok).abs().max() <= 2e-2, "prefill logprob vs CPU oracle"
+    # written caches: layer 0 depends on embedding, norm, projection and rotary only
+    assert_bf16_close(dec.key_cache[0], kc[0], max_ulp=2, what="layer 0 key cache")
+    assert_bf16_close(dec.value_cache[0], vc[0], max_ulp=2, what="layer 0 value cache")
+    for li in range(1, cfg.num_layers):
+        d = (dec.key_cache[li].cpu().float() - kc[li].float()).abs().max()
+        assert d <= 0.06 * max(1.0, float(kc[li].float().abs().max())), f"layer {li} key cache"
+
+    # decode step: batch of 5 vs each request alone, eager; 0 differing bits
+    first = tok.numpy()
+    dmeta = _decode_meta(cfg, prompts, blocks, allseq)
+    b = dec.bucket(len(allseq), len(allseq))
+    b.load(dmeta, first)
+    rlog = []
+    dec.step(b, 1, rlog)
+    torch.cuda.synchronize()
+    lp_batch, tok_batch = b.logprobs.cpu().clone(), b.tokens.cpu().clone()
+    for s in allseq:
+        m1 = _decode_meta(cfg, prompts, blocks, [s])
+        b1 = dec.bucket(1, 1)
+        b1.load(m1, first[s : s + 1])
+        dec.step(b1, 1)
+        torch.cuda.synchronize()
+        assert_bitwise(b1.logprobs.cpu(), lp_batch[s : s + 1], f"decode logprob of request {s}: batch 1 vs batch 5")
+        assert int(b1.tokens[0]) == int(tok_batch[s])
+
+    # oracle decode step
+    report = []
+    logits_ref, _, _ = OD.decoder_step_ref(cfg, wc, first, dmeta, kc, vc, cos, sin, [r.cpu() for r in rlog], report)
+    _check_routing_report(report, "decode")
+    lp_ref = torch.log_softmax(logits_ref.float(), -1).gather(-1, tok_batch.view(-1, 1)).squeeze(-1)
+    assert (lp_batch - lp_ref).abs().max() <= 2e-2, "decode logprob vs CPU oracle"
+
+
+def test_prefill_alone_equals_prefill_in_batch_and_chunked():
+    cfg, w, dec, prompts, blocks = _setup(seed=4)
+    allseq = list(range(len(prompts)))
+    tok, lp, _, _ = _prefill(dec, cfg, prompts, blocks, allseq)
+    for s in (0, 3):
+        t1, l1, _, _ = _prefill(dec, cfg, prompts, blocks, [s])
+        assert_bitwise(l1, lp[s : s + 1], f"prefill logprob of request {s}: alone vs batch")
+        assert int(t1[0]) == int(tok[s])
+    # chunked prefill of request 1: first part, then the rest; last-token logprob must not change
+    s = 1
+    n = len(prompts[s])
+    cut = max(1, n // 2)
+    maxb = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
+    for lo, hi in ((0, cut), (cut, n)):
+        meta = build_step_metadata([dict(num_computed_tokens=hi, tokens_this_step=hi - lo, block_ids=blocks[s])], cfg.page_size, maxb)
+        b = dec.bucket(hi - lo, 1)
+        b.load(meta, prompts[s][lo:hi])
+        dec.step(b, meta["max_seqlen_q"])
+        torch.cuda.synchronize()
+    assert_bitwise(b.logprobs.cpu(), lp[s : s + 1], "chunked prefill vs whole prefill")
+
+
+def test_graph_replay_with_padding_equals_eager():
+    cfg, w, dec, prompts, blocks = _setup(num_seqs=5, seed=5)
+    allseq = list(range(5))
+    tok, _, _, _ = _prefill(dec, cfg, prompts, blocks, allseq)
+    first = tok.numpy()
+    dmeta = _decode_meta(cfg, prompts, blocks, allseq)
+    be = dec.bucket(5, 5)
+    be.load(dmeta, first)
+    dec.step(be, 1)
+    torch.cuda.synchronize()
+    lp_eager, tok_eager = be.logprobs.cpu().clone(), be.tokens.cpu().clone()
+    # bucket of 8 tokens / 8 sequences: 3 padded rows
+    bg = dec.bucket(8, 8)
+    bg.load(dmeta, first)
+    g = dec.capture(bg, 1)
+    for rep in range(3):
+        bg.load(dmeta, first)
+        g.replay()
+        torch.cuda.synchronize()
+        assert_bitwise(bg.logprobs.cpu()[:5], lp_eager, f"graph replay {rep} vs eager")
+        assert torch.equal(bg.tokens.cpu()[:5], tok_eager)
+        # eager work between replays
+        be.load(dmeta, first)
+        dec.step(be, 1)
+        torch.cuda.synchronize()
+        assert_bitwise(be.logprobs.cpu(), lp_eager, "eager repeat")
+    # a different, smaller batch through the same graph
+    sub = [4, 1]
+    m2 = _decode_meta(cfg, prompts, blocks, sub)
+    bg.load(m2, first[sub])
+    g.replay()
+    torch.cuda.synchronize()
+    assert_bitwise(bg.logprobs.cpu()[:2], lp_eager[sub], "graph replay with another batch composition")

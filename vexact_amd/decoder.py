@@ -1,0 +1,332 @@
+"""A Qwen3-MoE-shaped decoder that runs entirely on the HIP kernels, with paged KV, bucketed
+static buffers and HIP-graph capture of the decode step.
+
+It plays the part of the reference's model runner for this architecture:
+``Inferencer._prepare_gen_ctx`` / ``_prepare_input_buffers_from_gen_ctx``
+(vexact/inferencer/inferencer.py:193-349: integer metadata and the padding rules of a captured
+bucket), ``CudaGraphManager`` (vexact/inferencer/cudagraph_utils.py:45-190: power-of-two token
+buckets, capture, padded replay) and ``_select_tokens`` (inferencer.py:391-449: last-token gather,
+greedy token, fp32 logprob). The layer itself follows the HuggingFace Qwen3-MoE decoder layer the
+reference patches (RMSNorm -> q/k/v -> per-head q/k norm -> rotary -> paged attention -> o_proj ->
+residual -> RMSNorm -> router -> fused experts -> residual), all pipeline stages on one device.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import ops
+
+
+@dataclass
+class DecoderConfig:
+    hidden_size: int = 2048
+    num_layers: int = 48
+    num_heads: int = 32
+    num_kv_heads: int = 4
+    head_dim: int = 128
+    num_experts: int = 128
+    top_k: int = 8
+    moe_intermediate: int = 768
+    vocab_size: int = 151936
+    rms_eps: float = 1e-6
+    rope_theta: float = 1.0e6
+    norm_topk_prob: bool = True
+    page_size: int = 16
+    max_model_len: int = 4096
+
+    @property
+    def qkv_dim(self) -> int:
+        return (self.num_heads + 2 * self.num_kv_heads) * self.head_dim
+
+
+def qwen3_30b_a3b() -> DecoderConfig:
+    return DecoderConfig()
+
+
+def tiny_config(**kw) -> DecoderConfig:
+    base = dict(hidden_size=256, num_layers=2, num_heads=4, num_kv_heads=2, head_dim=128, num_experts=8, top_k=2,
+                moe_intermediate=128, vocab_size=1000, max_model_len=512)
+    base.update(kw)
+    return DecoderConfig(**base)
+
+
+class DecoderWeights:
+    """bf16 weights; q/k/v projections are stored fused as one ``[(Hq+2Hkv)*D, H]`` matrix and the
+    expert gate/up projections as ``[E, 2I, H]`` (gate rows first), like the reference's
+    ``Qwen3MoeExperts`` (vexact/models/qwen3_moe/modeling_qwen3_moe.py:42-67)."""
+
+    def __init__(self, cfg: DecoderConfig, device="cuda", seed: int = 5, std: float = 0.02, generator_device="cuda"):
+        self.cfg = cfg
+        g = torch.Generator(device=generator_device).manual_seed(seed)
+        bf = torch.bfloat16
+
+        def rnd(*shape):
+            t = torch.empty(shape, dtype=bf, device=generator_device)
+            t.normal_(0.0, std, generator=g)
+            return t.to(device)
+
+        H, D, E, I = cfg.hidden_size, cfg.head_dim, cfg.num_experts, cfg.moe_intermediate
+        ones = lambda n: torch.ones(n, dtype=bf, device=device)  # noqa: E731
+        self.embed = rnd(cfg.vocab_size, H)
+        self.lm_head = rnd(cfg.vocab_size, H)
+        self.final_norm = ones(H)
+        self.layers = []
+        for _ in range(cfg.num_layers):
+            self.layers.append(
+                dict(
+                    in_norm=ones(H),
+                    qkv=rnd(cfg.qkv_dim, H),
+                    q_norm=ones(D),
+                    k_norm=ones(D),
+                    o=rnd(H, cfg.num_heads * D),
+                    post_norm=ones(H),
+                    router=rnd(E, H),
+                    gate_up=rnd(E, 2 * I, H),
+                    down=rnd(E, H, I),
+                )
+            )
+
+    def nbytes(self) -> int:
+        n = self.embed.numel() + self.lm_head.numel() + self.final_norm.numel()
+        for l in self.layers:
+            n += sum(t.numel() for t in l.values())
+        return 2 * n
+
+    def to_cpu(self) -> "DecoderWeights":
+        c = object.__new__(DecoderWeights)
+        c.cfg = self.cfg
+        c.embed, c.lm_head, c.final_norm = self.embed.cpu(), self.lm_head.cpu(), self.final_norm.cpu()
+        c.layers = [{k: v.cpu() for k, v in l.items()} for l in self.layers]
+        return c
+
+
+def rope_tables(cfg: DecoderConfig, device) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos / sin ``[max_model_len, D]`` in bf16: fp32 ``position * inv_freq`` duplicated over both
+    halves, then cast (what HuggingFace's rotary embedding yields for bf16 activations)."""
+    D = cfg.head_dim
+    inv_freq = 1.0 / (cfg.rope_theta ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    pos = torch.arange(cfg.max_model_len, dtype=torch.float32)
+    freqs = pos[:, None] * inv_freq[None, :]
+    emb = torch.cat([freqs, freqs], dim=-1)
+    return emb.cos().to(torch.bfloat16).to(device), emb.sin().to(torch.bfloat16).to(device)
+
+
+def build_step_metadata(requests: Sequence[dict], page_size: int, max_blocks_per_req: int) -> dict:
+    """Integer metadata of one step, vectorised numpy (exact). ``requests`` hold
+    ``num_computed_tokens`` (after this step), ``tokens_this_step`` and ``block_ids``."""
+    n_tok = np.array([r["tokens_this_step"] for r in requests], dtype=np.int64)
+    done = np.array([r["num_computed_tokens"] for r in requests], dtype=np.int64)
+    B = len(requests)
+    qsl = np.zeros(B + 1, dtype=np.int32)
+    np.cumsum(n_tok, out=qsl[1:])
+    total = int(qsl[-1])
+    seq_of_tok = np.repeat(np.arange(B), n_tok)
+    positions = np.arange(total, dtype=np.int64) - np.repeat(qsl[:-1].astype(np.int64), n_tok) + np.repeat(done - n_tok, n_tok)
+    block_tables = np.full((B, max_blocks_per_req), -1, dtype=np.int32)
+    for s, r in enumerate(requests):
+        ids = r["block_ids"]
+        block_tables[s, : len(ids)] = ids
+    slot = block_tables[seq_of_tok, positions // page_size].astype(np.int64) * page_size + positions % page_size
+    return {
+        "slot_mapping": slot.astype(np.int32),
+        "context_lens": done.astype(np.int32),
+        "block_tables": block_tables,
+        "query_start_loc": qsl,
+        "max_seqlen_q": int(n_tok.max()) if B else 0,
+        "positions": positions,
+    }
+
+
+def capture_sizes(max_size: int) -> list[int]:
+    """1, 2, 4, ... up to the first power of two >= max_size (cudagraph_utils.py:84-94)."""
+    if max_size <= 0:
+        raise ValueError(f"max_size must be positive or None, got {max_size}")
+    sizes, s = [], 1
+    while s < max_size:
+        sizes.append(s)
+        s *= 2
+    sizes.append(s)
+    return sizes
+
+
+class StepBuffers:
+    """Static device buffers of one (num_tokens, num_seqs) bucket."""
+
+    def __init__(self, cfg: DecoderConfig, num_tokens: int, num_seqs: int, device):
+        T, B = num_tokens, num_seqs
+        self.num_tokens, self.num_seqs = T, B
+        self.max_blocks = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
+        i32, i64, bf = torch.int32, torch.int64, torch.bfloat16
+        z = lambda *s, dtype: torch.zeros(s, dtype=dtype, device=device)  # noqa: E731
+        self.input_ids = z(T, dtype=i64)
+        self.positions = z(T, dtype=i64)
+        self.slot_mapping = torch.full((T,), -1, dtype=i32, device=device)
+        self.block_tables = torch.full((B, self.max_blocks), -1, dtype=i32, device=device)
+        self.context_lens = z(B, dtype=i32)
+        self.query_start_loc = z(B + 1, dtype=i32)
+        H, k = cfg.hidden_size, cfg.top_k
+        self.x = z(T, H, dtype=bf)
+        self.h = z(T, H, dtype=bf)
+        self.qkv = z(T, cfg.qkv_dim, dtype=bf)
+        self.q = z(T, cfg.num_heads, cfg.head_dim, dtype=bf)
+        self.attn = z(T, cfg.num_heads, cfg.head_dim, dtype=bf)
+        self.o = z(T, H, dtype=bf)
+        self.router_logits = z(T, cfg.num_experts, dtype=bf)
+        self.topk_w = z(T, k, dtype=bf)
+        self.topk_idx = z(T, k, dtype=i32)
+        self.hw = z(T * k, cfg.moe_intermediate, dtype=bf)
+        self.eo = z(T * k, H, dtype=bf)
+        self.bm = ops.moe_tile_rows(T)
+        from . import _lib
+
+        lib = _lib.load()
+        self.max_tiles = lib.vx_moe_max_tiles(T * k, cfg.num_experts, self.bm)
+        self.route_ints = z(2 * cfg.num_experts + 1 + 3 * T * k + 3 * self.max_tiles, dtype=i32)
+        self.attn_ws = torch.empty(
+            max(16, lib.vx_paged_attn_decode_workspace_bytes(B, cfg.num_heads, cfg.head_dim, self.max_blocks * cfg.page_size)),
+            dtype=torch.uint8, device=device)
+        # sampling: one row per sequence
+        self.last_h = z(B, H, dtype=bf)
+        self.logits = z(B, cfg.vocab_size, dtype=bf)
+        self.logprobs = z(B, dtype=torch.float32)
+        self.tokens = z(B, dtype=i64)
+
+    def load(self, meta: dict, input_ids: np.ndarray) -> tuple[int, int]:
+        """Copy one step's metadata in, applying the bucket padding rules (inferencer.py:306-324):
+        pad tokens get id 0, position 0, slot -1; pad sequences get ``query_start_loc = T_real``,
+        ``context_len = 0`` and an all-zero block-table row."""
+        T, B = len(input_ids), len(meta["context_lens"])
+        if T > self.num_tokens:
+            raise ValueError(f"total_tokens exceeds capture_tokens: {T} > {self.num_tokens}")
+        if B > self.num_seqs:
+            raise ValueError(f"graph_num_seqs cannot be smaller than num_seqs: {self.num_seqs} < {B}")
+        ids = np.zeros(self.num_tokens, np.int64); ids[:T] = input_ids
+        pos = np.zeros(self.num_tokens, np.int64); pos[:T] = meta["positions"]
+        slot = np.full(self.num_tokens, -1, np.int32); slot[:T] = meta["slot_mapping"]
+        bt = np.zeros((self.num_seqs, self.max_blocks), np.int32)
+        bt[:B] = -1
+        w = meta["block_tables"].shape[1]
+        bt[:B, :w] = meta["block_tables"][:, : self.max_blocks]
+        lens = np.zeros(self.num_seqs, np.int32); lens[:B] = meta["context_lens"]
+        qsl = np.full(self.num_seqs + 1, T, np.int32); qsl[: B + 1] = meta["query_start_loc"]
+        for dst, src in ((self.input_ids, ids), (self.positions, pos), (self.slot_mapping, slot), (self.block_tables, bt),
+                         (self.context_lens, lens), (self.query_start_loc, qsl)):
+            dst.copy_(torch.from_numpy(src), non_blocking=False)
+        return T, B
+
+
+class Qwen3MoeDecoder:
+    """Owns weights, the paged KV cache and per-bucket buffers / graphs."""
+
+    def __init__(self, cfg: DecoderConfig, weights: DecoderWeights, num_cache_blocks: int, device="cuda"):
+        self.cfg, self.w, self.device = cfg, weights, device
+        self.cos, self.sin = rope_tables(cfg, device)
+        shape = (num_cache_blocks, cfg.page_size, cfg.num_kv_heads, cfg.head_dim)
+        self.key_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device) for _ in range(cfg.num_layers)]
+        self.value_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device) for _ in range(cfg.num_layers)]
+        self.buffers: dict[tuple[int, int], StepBuffers] = {}
+        self.graphs: dict[tuple[int, int, int], torch.cuda.CUDAGraph] = {}
+
+    def bucket(self, num_tokens: int, num_seqs: int) -> StepBuffers:
+        key = (num_tokens, num_seqs)
+        if key not in self.buffers:
+            self.buffers[key] = StepBuffers(self.cfg, num_tokens, num_seqs, self.device)
+        return self.buffers[key]
+
+    # ---- one forward pass over a bucket's static buffers (capture-safe: no sync, no host reads)
+    def forward(self, b: StepBuffers, max_seqlen_q: int, routing_log: Optional[list] = None) -> None:
+        cfg, w = self.cfg, self.w
+        scale = cfg.head_dim ** -0.5
+        E, k, I = cfg.num_experts, cfg.top_k, cfg.moe_intermediate
+        ops.embedding(w.embed, b.input_ids, out=b.x)
+        for li, lw in enumerate(w.layers):
+            if li == 0:
+                ops.rms_norm(b.x, lw["in_norm"], cfg.rms_eps, hf_two_rounding=True, out=b.h)
+            ops.gemm_nt(b.h, lw["qkv"], out=b.qkv)
+            ops.qk_norm_rope_store(b.qkv, lw["q_norm"], lw["k_norm"], self.cos, self.sin, b.positions, b.slot_mapping,
+                                   b.q, self.key_cache[li], self.value_cache[li], cfg.num_heads, cfg.num_kv_heads,
+                                   cfg.head_dim, cfg.rms_eps)
+            ops.paged_attention(b.q, self.key_cache[li], self.value_cache[li], b.query_start_loc, b.context_lens,
+                                b.block_tables, scale, max_seqlen_q, out=b.attn, workspace=b.attn_ws)
+            ops.gemm_nt(b.attn.view(b.num_tokens, -1), lw["o"], out=b.o)
+            # x <- x + o ; h <- post_norm(x)
+            ops.rms_norm(b.o, lw["post_norm"], cfg.rms_eps, hf_two_rounding=True, residual=b.x, sum_out=b.x, out=b.h)
+            ops.gemm_nt(b.h, lw["router"], out=b.router_logits)
+            self._router(b)
+            if routing_log is not None:  # debugging / tests only (allocates; not for graph capture)
+                routing_log.append(b.topk_idx.clone())
+            r = ops.moe_route(b.topk_idx, E, bm=b.bm, buffers=b.route_ints)
+            gu = lw["gate_up"]
+            ops.moe_gemm(b.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=b.topk_w,
+                         row_scale_idx=r.sorted_flat, out=b.hw)
+            ops.moe_gemm(b.hw, lw["down"], r, out=b.eo)
+            nxt = w.layers[li + 1]["in_norm"] if li + 1 < cfg.num_layers else w.final_norm
+            # x <- x + sum_slots(eo) ; h <- next norm(x)
+            ops.moe_gather(b.eo, r.scatter_index, residual=b.x, out=b.x)
+            ops.rms_norm(b.x, nxt, cfg.rms_eps, hf_two_rounding=True, out=b.h)
+
+    def _router(self, b: StepBuffers) -> None:
+        from . import _lib
+
+        cfg = self.cfg
+        _lib.check(
+            _lib.load().vx_router_topk(
+                b.router_logits.data_ptr(), b.topk_w.data_ptr(), b.topk_idx.data_ptr(), b.num_tokens, cfg.num_experts,
+                cfg.top_k, b.router_logits.stride(0), 1, 1, 0, int(cfg.norm_topk_prob),
+                torch.cuda.current_stream().cuda_stream),
+            "vx_router_topk",
+        )
+
+    def sample(self, b: StepBuffers, decode: bool) -> None:
+        """Last token of each sequence -> lm_head -> greedy token and its fp32 logprob."""
+        if decode and b.num_tokens == b.num_seqs:
+            last = b.h  # every token is a last token
+        else:
+            idx = (b.query_start_loc[1:].long() - 1).clamp_(min=0)
+            torch.index_select(b.h, 0, idx, out=b.last_h)
+            last = b.last_h
+        ops.gemm_nt(last, self.w.lm_head, out=b.logits)
+        lp, tok = ops.logprobs(b.logits, None, return_tokens=True)
+        b.logprobs.copy_(lp)
+        b.tokens.copy_(tok)
+
+    def step(self, b: StepBuffers, max_seqlen_q: int, routing_log: Optional[list] = None) -> None:
+        self.forward(b, max_seqlen_q, routing_log)
+        self.sample(b, decode=(max_seqlen_q == 1))
+
+    def capture(self, b: StepBuffers, max_seqlen_q: int = 1) -> torch.cuda.CUDAGraph:
+        key = (b.num_tokens, b.num_seqs, max_seqlen_q)
+        if key in self.graphs:
+            return self.graphs[key]
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self.step(b, max_seqlen_q)  # warm-up on a side stream
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.step(b, max_seqlen_q)
+        self.graphs[key] = g
+        return g
+
+
+def decode_bytes_per_step(cfg: DecoderConfig, context_lens: Sequence[int], experts_hit_per_layer: Optional[int] = None) -> dict:
+    """Algorithmic HBM bytes of one decode step: every weight touched once plus the KV of every
+    sequence, plus small activation terms."""
+    H, D, E, I, V = cfg.hidden_size, cfg.head_dim, cfg.num_experts, cfg.moe_intermediate, cfg.vocab_size
+    B = len(context_lens)
+    U = E if experts_hit_per_layer is None else experts_hit_per_layer
+    attn_w = (cfg.qkv_dim * H + H * cfg.num_heads * D) * 2
+    router_w = E * H * 2
+    expert_w = U * 3 * H * I * 2
+    kv = int(sum(context_lens)) * 2 * cfg.num_kv_heads * D * 2
+    per_layer = attn_w + router_w + expert_w + kv
+    head = V * H * 2 + B * V * 2
+    return {"weights": cfg.num_layers * (attn_w + router_w + expert_w) + V * H * 2, "kv": cfg.num_layers * kv,
+            "total": cfg.num_layers * per_layer + head, "moe_per_layer": expert_w, "kv_per_layer": kv}
