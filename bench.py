@@ -1,0 +1,288 @@
+#!/usr/bin/env python3
+"""Headline benchmark: decode tok/s of a Qwen3-30B-A3B-shaped decoder at batch 256 on one MI355X.
+
+Workload (synthetic, seeded): 48 layers, hidden 2048, 32 q / 4 kv heads x 128, 128 experts top-8
+(moe_intermediate 768), vocab 151936, random-init bf16 weights ~N(0, 0.02); 256 sequences with prompt
+lengths uniform in [256, 2048] of random token ids, paged KV (page 16, block tables from a random
+permutation of the pool). The prompts are prefilled with this library's own kernels, then ONE decode
+step (256 tokens, 256 sequences, greedy token + fp32 logprob) is captured in a HIP graph and
+replayed: warm-up W times, then exactly K timed replays.
+
+Prints one JSON line: whole-job tok/s, the roofline of the dominant kernel (MoE gate/up grouped
+GEMM, HBM bound) measured with HIP events in an eager pass, per-kernel GB/s of the other
+memory-bound kernels, the logprob bit drift between batch 256 and batch 1, and the CPU oracle timed
+on the host cores for a bounded sample (one decoder layer + lm_head at batch 256, scaled to 48 layers).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=256)
+    ap.add_argument("--layers", type=int, default=48, help="fewer layers = a smoke run, flagged as such in the output")
+    ap.add_argument("--min-prompt", type=int, default=256)
+    ap.add_argument("--max-prompt", type=int, default=2048)
+    ap.add_argument("--drift-requests", type=int, default=8, help="requests re-run at batch 1 for the bit-drift check")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--seed", type=int, default=5)
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (all pipeline stages collapsed onto one MI355X); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from vexact_amd import _build, _lib, ops
+    from vexact_amd.decoder import (DecoderWeights, Qwen3MoeDecoder, build_step_metadata, decode_bytes_per_step,
+                                    qwen3_30b_a3b)
+
+    if not os.path.exists(_build.LIB_PATH):
+        _build.build()
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda"
+    torch.cuda.set_device(0)
+
+    cfg = qwen3_30b_a3b()
+    cfg.num_layers = args.layers
+    B = args.batch
+    rng = np.random.default_rng(args.seed)
+    prompt_lens = rng.integers(args.min_prompt, args.max_prompt + 1, size=B)
+    prompts = [rng.integers(0, cfg.vocab_size, size=int(n)) for n in prompt_lens]
+    pages = [(int(n) + 1 + cfg.page_size - 1) // cfg.page_size for n in prompt_lens]
+    pool = sum(pages) + 64
+    perm = rng.permutation(pool)
+    blocks, o = [], 0
+    for p in pages:
+        blocks.append(perm[o : o + p].tolist())
+        o += p
+    max_blocks = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
+
+    t0 = time.time()
+    w = DecoderWeights(cfg, device=dev, seed=args.seed)
+    dec = Qwen3MoeDecoder(cfg, w, num_cache_blocks=pool, device=dev)
+    torch.cuda.synchronize()
+    print(f"[bench] weights {w.nbytes() / 1e9:.1f} GB, KV pool {pool} pages "
+          f"({2 * cfg.num_layers * dec.key_cache[0].numel() * 2 / 1e9:.1f} GB), init {time.time() - t0:.1f}s",
+          file=sys.stderr, flush=True)
+
+    # ---- prefill with the library's own kernels, several sequences per pass
+    t0 = time.time()
+    PT, PB = 8192, 16
+    pb = dec.bucket(PT, PB)
+    first_tokens = np.zeros(B, dtype=np.int64)
+    s = 0
+    while s < B:
+        grp, tot = [], 0
+        while s < B and len(grp) < PB and tot + len(prompts[s]) <= PT:
+            grp.append(s)
+            tot += len(prompts[s])
+            s += 1
+        reqs = [dict(num_computed_tokens=len(prompts[i]), tokens_this_step=len(prompts[i]), block_ids=blocks[i]) for i in grp]
+        meta = build_step_metadata(reqs, cfg.page_size, max_blocks)
+        pb.load(meta, np.concatenate([prompts[i] for i in grp]))
+        dec.step(pb, meta["max_seqlen_q"])
+        first_tokens[grp] = pb.tokens[: len(grp)].cpu().numpy()
+    torch.cuda.synchronize()
+    print(f"[bench] prefill of {int(prompt_lens.sum())} tokens: {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+    del dec.buffers[(PT, PB)]
+    del pb
+    torch.cuda.empty_cache()
+
+    # ---- the decode step: 256 tokens, 256 sequences, captured in a HIP graph
+    ctx = [int(n) + 1 for n in prompt_lens]
+    reqs = [dict(num_computed_tokens=ctx[i], tokens_this_step=1, block_ids=blocks[i]) for i in range(B)]
+    dmeta = build_step_metadata(reqs, cfg.page_size, max_blocks)
+    db = dec.bucket(B, B)
+    db.load(dmeta, first_tokens)
+    graph = dec.capture(db, 1)
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tok_s = B * args.steps / dt
+    lp_graph = db.logprobs.cpu().clone()
+    tok_graph = db.tokens.cpu().clone()
+
+    # ---- logprob bit drift: the same requests at batch 1 (eager)
+    drift_bits, checked = 0, 0
+    b1 = dec.bucket(1, 1)
+    for i in range(min(args.drift_requests, B)):
+        r = (i * 37) % B
+        m1 = build_step_metadata([reqs[r]], cfg.page_size, max_blocks)
+        b1.load(m1, first_tokens[r : r + 1])
+        dec.step(b1, 1)
+        torch.cuda.synchronize()
+        a = b1.logprobs.cpu().view(torch.int32)
+        bb = lp_graph[r : r + 1].view(torch.int32)
+        drift_bits += bin(int(a[0]) ^ int(bb[0])).count("1") + (0 if int(b1.tokens[0]) == int(tok_graph[r]) else 64)
+        checked += 1
+
+    # ---- per-kernel timing with HIP events on the launch stream (eager pass over all layers)
+    E, k, I, H = cfg.num_experts, cfg.top_k, cfg.moe_intermediate, cfg.hidden_size
+    ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
+    names = ("moe_gate_up", "moe_down", "attn_decode", "qkv_gemm", "o_gemm")
+    times = {n: [] for n in names}
+    reps = 2
+    scale = cfg.head_dim ** -0.5
+    experts_hit = []
+    for rep in range(reps + 1):
+        pend = []
+        db.load(dmeta, first_tokens)
+        ops.embedding(w.embed, db.input_ids, out=db.x)
+        ops.rms_norm(db.x, w.layers[0]["in_norm"], cfg.rms_eps, hf_two_rounding=True, out=db.h)
+        for li, lw in enumerate(w.layers):
+            def timed(name, fn):
+                a, b_ = ev(), ev()
+                a.record()
+                fn()
+                b_.record()
+                pend.append((name, a, b_))
+            timed("qkv_gemm", lambda: ops.gemm_nt(db.h, lw["qkv"], out=db.qkv))
+            ops.qk_norm_rope_store(db.qkv, lw["q_norm"], lw["k_norm"], dec.cos, dec.sin, db.positions, db.slot_mapping,
+                                   db.q, dec.key_cache[li], dec.value_cache[li], cfg.num_heads, cfg.num_kv_heads,
+                                   cfg.head_dim, cfg.rms_eps)
+            timed("attn_decode", lambda: ops.paged_attention(db.q, dec.key_cache[li], dec.value_cache[li], db.query_start_loc,
+                                                             db.context_lens, db.block_tables, scale, 1, out=db.attn,
+                                                             workspace=db.attn_ws))
+            timed("o_gemm", lambda: ops.gemm_nt(db.attn.view(B, -1), lw["o"], out=db.o))
+            ops.rms_norm(db.o, lw["post_norm"], cfg.rms_eps, hf_two_rounding=True, residual=db.x, sum_out=db.x, out=db.h)
+            ops.gemm_nt(db.h, lw["router"], out=db.router_logits)
+            dec._router(db)
+            r = ops.moe_route(db.topk_idx, E, bm=db.bm, buffers=db.route_ints)
+            if rep == 0:
+                experts_hit.append(int((r.splits > 0).sum()))
+            gu = lw["gate_up"]
+            timed("moe_gate_up", lambda: ops.moe_gemm(db.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token,
+                                                      row_scale=db.topk_w, row_scale_idx=r.sorted_flat, out=db.hw))
+            timed("moe_down", lambda: ops.moe_gemm(db.hw, lw["down"], r, out=db.eo))
+            nxt = w.layers[li + 1]["in_norm"] if li + 1 < cfg.num_layers else w.final_norm
+            ops.moe_gather(db.eo, r.scatter_index, residual=db.x, out=db.x)
+            ops.rms_norm(db.x, nxt, cfg.rms_eps, hf_two_rounding=True, out=db.h)
+        torch.cuda.synchronize()
+        if rep > 0:  # first pass is a warm-up
+            for name, a, b_ in pend:
+                times[name].append(a.elapsed_time(b_) * 1e-3)
+    avg = {n: float(np.mean(v)) for n, v in times.items()}
+    U = float(np.mean(experts_hit))
+    sumL = int(sum(ctx))
+    kbytes = {
+        "moe_gate_up": U * 2 * I * H * 2 + B * H * 2 + B * k * I * 2 + B * k * 6,
+        "moe_down": U * H * I * 2 + B * k * I * 2 + B * k * H * 2,
+        "attn_decode": sumL * 2 * cfg.num_kv_heads * cfg.head_dim * 2 + 2 * B * cfg.num_heads * cfg.head_dim * 2
+        + sum((c + cfg.page_size - 1) // cfg.page_size for c in ctx) * 4,
+        "qkv_gemm": 2 * (cfg.qkv_dim * H + B * H + B * cfg.qkv_dim),
+        "o_gemm": 2 * (H * cfg.num_heads * cfg.head_dim + B * cfg.num_heads * cfg.head_dim + B * H),
+    }
+    kernels = {n: {"avg_us": round(avg[n] * 1e6, 1), "bytes": int(kbytes[n]), "GBps": round(kbytes[n] / avg[n] / 1e9, 1),
+                   "frac_hbm": round(kbytes[n] / avg[n] / 1e9 / HBM_PEAK_GBS, 4)} for n in names}
+    dom = "moe_gate_up"
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(dom)
+        except Exception:
+            traffic = None
+    roofline = {"bound": "hbm", "kernel": "gemm_stream_kernel<2, SWIGLU, grouped> (MoE gate/up)",
+                "achieved": kernels[dom]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": kernels[dom]["frac_hbm"], "traffic": traffic}
+
+    step_bytes = decode_bytes_per_step(cfg, ctx, experts_hit_per_layer=U)
+    out = {
+        "metric": "decode tok/s Qwen3-30B-A3B bs=256 on 1 GPU",
+        "value": round(tok_s, 1),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"Qwen3-30B-A3B-shaped decoder ({cfg.num_layers} layers, 128 experts top-8, vocab 151936), "
+                               f"hipGraph decode step, batch {B}, prompts U[{args.min_prompt},{args.max_prompt}], paged KV page 16",
+                   "batch": B, "sum_context": sumL, "full_model": cfg.num_layers == 48 and B == 256},
+        "step_hbm_bytes": int(step_bytes["total"]),
+        "step_frac_of_hbm_roofline": round(step_bytes["total"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "logprob_drift_bits_b256_vs_b1": drift_bits,
+        "drift_requests_checked": checked,
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, args.cpu_seconds)
+    print(json.dumps(out), flush=True)
+
+
+def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
+    """The CPU oracle (torch CPU restatement of the reference's formulas) on this host's cores: one
+    decoder layer + lm_head at the bench batch, scaled to all layers."""
+    import torch
+
+    from oracle import decoder as OD
+    from oracle.row_ops import hf_rms_norm_ref, logprobs_ref, matmul_ref
+    from vexact_amd.decoder import rope_tables
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    torch.set_num_threads(cores)
+    lw = {k_: v.cpu() for k_, v in w.layers[0].items()}
+    kc, vc = dec.key_cache[0].cpu(), dec.value_cache[0].cpu()
+    cos, sin = rope_tables(cfg, "cpu")
+    x = w.embed[torch.as_tensor(first_tokens).to(w.embed.device)].cpu()
+    pos = torch.as_tensor(dmeta["positions"]).long()
+    lm_head, fnorm = w.lm_head.cpu(), w.final_norm.cpu()
+    t_layer, t_head, n = 0.0, 0.0, 0
+    t_start = time.perf_counter()
+    while True:
+        t0 = time.perf_counter()
+        y = OD.layer_ref(cfg, lw, x, pos, dmeta, kc, vc, cos, sin)
+        t1 = time.perf_counter()
+        logits = matmul_ref(hf_rms_norm_ref(y, fnorm, cfg.rms_eps), lm_head.t())
+        tok = logits.float().argmax(-1)
+        logprobs_ref(logits.float(), tok)
+        t2 = time.perf_counter()
+        t_layer += t1 - t0
+        t_head += t2 - t1
+        n += 1
+        if time.perf_counter() - t_start > budget_s or n >= 5:
+            break
+    step = cfg.num_layers * t_layer / n + t_head / n
+    return {"value": round(B / step, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+            "sample": f"1 of {cfg.num_layers} decoder layers + lm_head at batch {B}, {n} repeats "
+                      f"({t_layer / n:.2f}s per layer, {t_head / n:.2f}s head), scaled to {cfg.num_layers} layers"}
+
+
+if __name__ == "__main__":
+    main()
