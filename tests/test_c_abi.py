@@ -1,0 +1,55 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/vexact_hip.h declares."""
+
+import ctypes
+import os
+import re
+
+from vexact_amd import _build, _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "vexact_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_is_built_and_loads():
+    if not os.path.exists(_build.LIB_PATH):
+        _build.build()
+    lib = _lib.load()
+    assert lib.vx_abi_version() == 1
+    assert lib.vx_status_string(0) == b"ok"
+    assert b"workspace" in lib.vx_status_string(-3)
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = _declared()
+    assert len(names) >= 25
+    lib = ctypes.CDLL(_build.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    assert sorted(_lib.PROTOTYPES) == names, "ctypes prototypes and header out of sync"
+
+
+def test_host_only_helpers():
+    lib = _lib.load()
+    assert lib.vx_attn_chunk_size() == 256
+    # partial states: (Dv + 2) floats per (sequence, head, 256-key chunk)
+    assert lib.vx_paged_attn_decode_workspace_bytes(64, 16, 128, 4096) == 64 * 16 * 16 * 130 * 4
+    assert lib.vx_paged_attn_decode_workspace_bytes(1, 1, 128, 1) == 130 * 4
+    # 16 bytes per (row, 4096-column chunk)
+    assert lib.vx_log_softmax_workspace_bytes(7, 151936) == 7 * 38 * 16
+    assert lib.vx_moe_max_tiles(2048, 128, 32) == 128 + 64
+    assert lib.vx_moe_max_tiles(8, 128, 32) == 8
+    assert lib.vx_moe_max_tiles(0, 128, 32) == 0
+
+
+def test_bad_arguments_are_rejected_before_any_launch():
+    lib = _lib.load()
+    assert lib.vx_gemm_bf16_nt(None, None, None, None, 1, 1, 8, 8, 8, 8, None) == -1
+    assert lib.vx_rms_norm(None, None, None, None, None, 1, 1, 8, 8, 0, 8, 0, 1e-6, 0, None) == -1
+    assert lib.vx_moe_route(None, 0, 1, 1, 1, 32, None, None, None, None, None, None, None, None, 8, None) == -1
+    assert lib.vx_attention(None, None, None, None, None, None, None, None, 1, 1, 4, 2, 128, 128,
+                            0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 16, 1.0, 1, 0, 1, None, 0, None) == -1

@@ -1,0 +1,146 @@
+"""Host-side logic that needs no GPU: step metadata, bucket padding, block allocator, contexts."""
+
+import threading
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import metadata as OMeta
+from vexact_amd.batch_invariant_ops import AttentionBlockSize, get_batch_invariant_attention_block_size
+from vexact_amd.batch_invariant_ops import kv_cache_context as KC
+from vexact_amd.decoder import StepBuffers, build_step_metadata, capture_sizes, decode_bytes_per_step, qwen3_30b_a3b, tiny_config
+
+
+def _requests(rng, n, page):
+    reqs, nxt = [], 0
+    for _ in range(n):
+        done = int(rng.integers(1, 200))
+        this = int(rng.integers(1, done + 1)) if rng.random() < 0.5 else 1
+        nb = (done + page - 1) // page
+        ids = list(range(nxt, nxt + nb))
+        rng.shuffle(ids)
+        nxt += nb
+        reqs.append(dict(num_computed_tokens=done, tokens_this_step=this, block_ids=ids))
+    return reqs
+
+
+def test_step_metadata_matches_the_loop_restatement():
+    rng = np.random.default_rng(0)
+    for page in (16, 256, 5):
+        reqs = _requests(rng, 9, page)
+        got = build_step_metadata(reqs, page, 40)
+        ref = OMeta.prepare_gen_ctx_ref(reqs, page, 40)
+        for k in ("slot_mapping", "context_lens", "block_tables", "query_start_loc", "positions"):
+            assert np.array_equal(got[k], ref[k]), k
+            assert got[k].dtype == ref[k].dtype, k
+        assert got["max_seqlen_q"] == ref["max_seqlen_q"]
+
+
+def test_hand_worked_metadata_example():
+    # page 4; request A has 6 tokens cached in blocks [7, 2] and adds 1; request B prefills 3 into block [5]
+    reqs = [dict(num_computed_tokens=7, tokens_this_step=1, block_ids=[7, 2]),
+            dict(num_computed_tokens=3, tokens_this_step=3, block_ids=[5])]
+    m = OMeta.prepare_gen_ctx_ref(reqs, 4, 3)
+    assert m["slot_mapping"].tolist() == [2 * 4 + 2, 20, 21, 22]
+    assert m["positions"].tolist() == [6, 0, 1, 2]
+    assert m["context_lens"].tolist() == [7, 3]
+    assert m["block_tables"].tolist() == [[7, 2, -1], [5, -1, -1]]
+    assert m["query_start_loc"].tolist() == [0, 1, 4] and m["max_seqlen_q"] == 3
+
+
+def test_bucket_padding_rules():
+    cfg = tiny_config()
+    rng = np.random.default_rng(1)
+    reqs = _requests(rng, 3, cfg.page_size)
+    for r in reqs:
+        r["tokens_this_step"] = 1
+    meta = build_step_metadata(reqs, cfg.page_size, cfg.max_model_len // cfg.page_size)
+    b = StepBuffers(cfg, 8, 8, "cpu")
+    T, B = b.load(meta, np.array([11, 12, 13]))
+    ref = OMeta.pad_for_graph_ref(meta, 8, 8)
+    assert (T, B) == (3, 3)
+    assert b.input_ids.tolist() == [11, 12, 13, 0, 0, 0, 0, 0]
+    assert np.array_equal(b.slot_mapping.numpy(), ref["slot_mapping"])
+    assert np.array_equal(b.positions.numpy(), ref["positions"])
+    assert np.array_equal(b.context_lens.numpy(), ref["context_lens"])
+    assert np.array_equal(b.block_tables.numpy(), ref["block_tables"])
+    assert np.array_equal(b.query_start_loc.numpy(), ref["query_start_loc"])
+    with pytest.raises(ValueError, match="total_tokens exceeds capture_tokens"):
+        StepBuffers(cfg, 2, 8, "cpu").load(meta, np.array([1, 2, 3]))
+    with pytest.raises(ValueError, match="graph_num_seqs cannot be smaller than num_seqs"):
+        StepBuffers(cfg, 8, 2, "cpu").load(meta, np.array([1, 2, 3]))
+
+
+def test_capture_sizes_and_byte_model():
+    assert capture_sizes(1) == [1]
+    assert capture_sizes(5) == [1, 2, 4, 8]
+    assert capture_sizes(256) == [1, 2, 4, 8, 16, 32, 64, 128, 256]
+    with pytest.raises(ValueError):
+        capture_sizes(0)
+    cfg = qwen3_30b_a3b()
+    b = decode_bytes_per_step(cfg, [1152] * 256)
+    assert abs(b["moe_per_layer"] - 1.208e9) < 1e7          # 128 experts x 3 x 2048 x 768 x 2 B
+    assert b["kv_per_layer"] == 256 * 1152 * 2048            # 2 x 4 kv heads x 128 x 2 B per token
+    assert 88e9 < b["total"] < 92e9                          # ~60.5 GB weights + ~29 GB KV
+
+
+def test_block_allocator_semantics():
+    cfg = types.SimpleNamespace(max_cache_blocks=6, page_size=4)
+    m = KC.KVCacheManager(cfg)
+    assert m.allocate_blocks(9) == [0, 1, 2]            # lowest ids first
+    assert m.allocate_blocks(9, num_current_blocks=3) == []
+    assert m.allocate_blocks(13, num_current_blocks=3) == [3]
+    assert m.allocate_blocks(100) is None               # out of blocks: nothing allocated
+    assert m.num_free_blocks() == 2 and m.num_allocated_blocks() == 4
+    m.free_blocks([1, 3, 3, 5])                          # 5 was never allocated: ignored
+    assert m.num_free_blocks() == 4
+    assert m.allocate_blocks(8) == [1, 3]               # freed ids are reused, lowest first
+    assert m.allocate_blocks(4) == [4]
+
+
+def test_kv_context_is_thread_local_and_validated():
+    KC.clear_kv_cache_context()
+    assert not KC.has_kv_cache_context() and KC.get_kv_cache_context() is None
+    lens = torch.zeros(2, dtype=torch.int32)
+    KC.set_kv_cache_context(is_paged_attn=False, context_lens=lens, query_start_loc=torch.zeros(3, dtype=torch.int32), max_seqlen_q=4)
+    assert KC.has_kv_cache_context() and KC.get_kv_cache_context().max_seqlen_q == 4
+    seen = []
+    t = threading.Thread(target=lambda: seen.append(KC.get_kv_cache_context()))
+    t.start(); t.join()
+    assert seen == [None]
+    with pytest.raises(AssertionError, match="key_cache required"):
+        KC.set_kv_cache_context(is_paged_attn=True, context_lens=lens)
+    with pytest.raises(AssertionError, match="query_start_loc required"):
+        KC.set_kv_cache_context(is_paged_attn=False, context_lens=lens)
+    KC.clear_kv_cache_context()
+
+
+def test_kv_cache_store_shapes():
+    hf = types.SimpleNamespace(num_key_value_heads=2, head_dim=8, hidden_size=64, num_attention_heads=8, num_hidden_layers=3,
+                               qk_head_dim=12, v_head_dim=8)
+    cc = types.SimpleNamespace(max_cache_blocks=5, page_size=4)
+    st = KC.KVCacheStore(hf, cc, torch.device("cpu"))
+    assert sorted(st.key_cache) == [0, 1, 2]
+    assert st.key_cache[0].shape == (5, 4, 2, 12) and st.value_cache[2].shape == (5, 4, 2, 8)
+    assert st.key_cache[1].dtype == torch.bfloat16 and float(st.key_cache[1].abs().sum()) == 0.0
+
+
+def test_ops_refuse_cpu_tensors_and_bad_arguments():
+    from vexact_amd.batch_invariant_ops import log_softmax, matmul_persistent, mean_dim, triton_bmm
+
+    assert get_batch_invariant_attention_block_size() == AttentionBlockSize(16, 16)
+    x = torch.zeros(2, 8)
+    with pytest.raises(ValueError, match="only supports log_softmax along the last dimension"):
+        log_softmax(x, dim=0)
+    with pytest.raises(ValueError, match="must be a CUDA tensor"):
+        log_softmax(x, dim=-1)
+    with pytest.raises(AssertionError, match="Input must be a CUDA tensor"):
+        mean_dim(x, 1)
+    with pytest.raises(AssertionError, match="Incompatible dimensions"):
+        matmul_persistent(torch.zeros(2, 3), torch.zeros(4, 5))
+    with pytest.raises(AssertionError, match="Incompatible dtypes"):
+        matmul_persistent(torch.zeros(2, 3), torch.zeros(3, 5, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError, match="Expected 3D tensors"):
+        triton_bmm(torch.zeros(2, 3), torch.zeros(3, 5))
