@@ -47,17 +47,18 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
                                                  __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// 16-byte global load that yields zeros when !ok. The address must be dereferenceable even
-// when !ok (callers clamp it); selecting on the loaded value instead of on the address keeps
-// the access a single global_load_dwordx4.
-__device__ __forceinline__ uint4 ldg16(const void* p, bool ok) {
-  uint4 v = *reinterpret_cast<const uint4*>(p);
+// 16-byte global loads. The address must always be dereferenceable (callers clamp it); zeroing
+// is done on the loaded VALUE, and only where the value is consumed, so that a load stays a single
+// global_load_dwordx4 and the wait for it is not pulled up to the issue point.
+__device__ __forceinline__ uint4 ldg16_raw(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint4 mask16(uint4 v, bool ok) {
   v.x = ok ? v.x : 0u;
   v.y = ok ? v.y : 0u;
   v.z = ok ? v.z : 0u;
   v.w = ok ? v.w : 0u;
   return v;
 }
+__device__ __forceinline__ uint4 ldg16(const void* p, bool ok) { return mask16(ldg16_raw(p), ok); }
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -73,15 +73,28 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
   p.bias = (const bf16_t*)bias;
   p.c = (bf16_t*)c; p.ldc = ldc;
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
-  if (M <= 64) {
-    const dim3 grid((unsigned)((N + 63) / 64), 1);
-    if (M <= 16) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
-    else if (M <= 32) gemm_stream_kernel<2, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  // Kernel choice (any choice gives the same bits): up to 512 rows the weight-streaming kernel wins
+  // unless the problem is large enough to fill the chip with 128x128 tiles; its row-tile height is
+  // the largest of 64 / 32 / 16 that still yields >= 256 workgroups.
+  const int64_t nt = (N + 63) / 64;
+  int mt = 0;
+  if (M <= 16) mt = 1;
+  else if (M <= 32) mt = 2;
+  else if (M <= 64) mt = 4;
+  else if (M <= 512 && nt * ((M + 63) / 64) <= 1024) {
+    mt = 1;
+    if (nt * ((M + 63) / 64) >= 256) mt = 4;
+    else if (nt * ((M + 31) / 32) >= 256) mt = 2;
+  }
+  if (mt != 0) {
+    const dim3 grid((unsigned)nt, (unsigned)((M + 16 * mt - 1) / (16 * mt)));
+    if (mt == 1) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+    else if (mt == 2) gemm_stream_kernel<2, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
     else gemm_stream_kernel<4, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
   } else {
-    const int64_t mt = (M + TL_BM - 1) / TL_BM;
-    if (mt > 65535) return VX_ERR_UNSUPPORTED;
-    const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)mt);
+    const int64_t mtl = (M + TL_BM - 1) / TL_BM;
+    if (mtl > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)mtl);
     gemm_tiled_kernel<EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
   }
   return launch_status();

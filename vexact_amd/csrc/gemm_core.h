@@ -100,30 +100,66 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   }
 
   uint4 wa[U], wb[EPI == EPI_SWIGLU ? U : 1];
+  // Weight loads of one group of U k-steps. A group that lies fully inside K is loaded without any
+  // masking so the loads stay in flight across the MFMAs of the previous group; only a ragged last
+  // group (K not a multiple of 32*U) pays for masks, and a group past K is all zeros.
   auto load_w = [&](int kstep0) {
+    if (kstep0 + 32 * U <= K) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      const int k = kstep0 + 32 * u + 8 * g;  // element index of this lane's 8 values
-      const bool ok = k < K;
-      const int ko = ok ? kstep0 + 32 * u : 0;
-      wa[u] = ldg16(wp + ko, ok);
-      if constexpr (EPI == EPI_SWIGLU) wb[u] = ldg16(wp2 + ko, ok);
+      for (int u = 0; u < U; u++) {
+        wa[u] = ldg16_raw(wp + kstep0 + 32 * u);
+        if constexpr (EPI == EPI_SWIGLU) wb[u] = ldg16_raw(wp2 + kstep0 + 32 * u);
+      }
+    } else if (kstep0 < K) {
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const bool ok = kstep0 + 32 * u + 8 * g < K;
+        const int ko = ok ? kstep0 + 32 * u : 0;
+        wa[u] = ldg16(wp + ko, ok);
+        if constexpr (EPI == EPI_SWIGLU) wb[u] = ldg16(wp2 + ko, ok);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        wa[u] = make_uint4(0, 0, 0, 0);
+        if constexpr (EPI == EPI_SWIGLU) wb[u] = make_uint4(0, 0, 0, 0);
+      }
     }
   };
 
+  // Activation staging: thread owns pieces tid + 256 j (j < NP) of the BM x KC tile; piece =
+  // (row pc / PPR, 16-byte column pc % PPR). Row sources are resolved once.
+  constexpr int PPR = KC / 8;            // 16-byte pieces per staged row
+  constexpr int NP = BM * PPR / 256;     // pieces per thread (16)
+  int64_t xoff[NP];                      // element offset of the piece's row in x, -1 = zero row
+#pragma unroll
+  for (int j = 0; j < NP; j++) {
+    const int pc = threadIdx.x + 256 * j;
+    const int r = pc / PPR;
+    int64_t off = -1;
+    if (r < rows) {
+      const int64_t sr = p.row_src ? (int64_t)p.row_src[row0 + r] : (int64_t)(row0 + r);
+      off = sr * p.ldx + (pc % PPR) * 8;
+    }
+    xoff[j] = off;
+  }
+
   load_w(0);
   for (int kc = 0; kc < K; kc += KC) {
+    uint4 stage[NP];
+#pragma unroll
+    for (int j = 0; j < NP; j++) {  // all loads of the fill in flight together
+      const int c8 = (threadIdx.x + 256 * j) % PPR;
+      const bool ok = xoff[j] >= 0 && kc + c8 * 8 < K;
+      stage[j] = ldg16_raw(p.x + (ok ? xoff[j] + kc : 0));
+    }
     __syncthreads();  // everyone is done reading the previous fill
-    constexpr int PPR = KC / 8;  // 16-byte pieces per staged row
-    for (int pc = threadIdx.x; pc < BM * PPR; pc += 256) {
-      const int r = pc / PPR, c8 = pc % PPR;
-      const bool ok = r < rows && kc + c8 * 8 < K;
-      const bf16_t* src = p.x;
-      if (ok) {
-        const int64_t sr = p.row_src ? (int64_t)p.row_src[row0 + r] : (int64_t)(row0 + r);
-        src = p.x + sr * p.ldx + kc + c8 * 8;
-      }
-      *(uint4*)(xs + r * RB + c8 * 16) = ldg16(src, ok);
+#pragma unroll
+    for (int j = 0; j < NP; j++) {
+      const int pc = threadIdx.x + 256 * j;
+      const int c8 = pc % PPR;
+      const bool ok = xoff[j] >= 0 && kc + c8 * 8 < K;
+      *(uint4*)(xs + (pc / PPR) * RB + c8 * 16) = mask16(stage[j], ok);
     }
     __syncthreads();
     const int kend = min(K - kc, KC);
@@ -242,23 +278,23 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p) {
     wrow[j] = wb + wbase + (int64_t)wr * p.ldw + c8 * 8;
   }
   uint4 gx[4], gw[4];
-  auto gload = [&](int k0) {
+  auto gload = [&](int k0) {  // raw loads; zeroing happens in lstore, after the MFMAs of this step
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int c8 = (tid + 256 * j) & 7;
-      const bool kok = k0 + c8 * 8 < K;
-      const int ko = kok ? k0 : 0;
-      gx[j] = ldg16(xrow[j] + ko, xok[j] && kok);
-      gw[j] = ldg16(wrow[j] + ko, kok);
+      const int ko = (k0 + c8 * 8 < K) ? k0 : 0;
+      gx[j] = ldg16_raw(xrow[j] + ko);
+      gw[j] = ldg16_raw(wrow[j] + ko);
     }
   };
-  auto lstore = [&](int buf) {
+  auto lstore = [&](int buf, int k0) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int pc = tid + 256 * j;
       const int r = pc >> 3, c8 = pc & 7;
-      *(uint4*)(&lx[buf][r * TL_RB + c8 * 16]) = gx[j];
-      *(uint4*)(&lw[buf][r * TL_RB + c8 * 16]) = gw[j];
+      const bool kok = k0 + c8 * 8 < K;
+      *(uint4*)(&lx[buf][r * TL_RB + c8 * 16]) = mask16(gx[j], xok[j] && kok);
+      *(uint4*)(&lw[buf][r * TL_RB + c8 * 16]) = mask16(gw[j], kok);
     }
   };
 
@@ -276,7 +312,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p) {
 
   const int nk = (K + TL_BK - 1) / TL_BK;
   gload(0);
-  lstore(0);
+  lstore(0, 0);
   __syncthreads();
   for (int kt = 0; kt < nk; kt++) {
     const int buf = kt & 1;
@@ -295,7 +331,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p) {
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = mfma16(wf[j], xf[i], acc[i][j]);
     }
-    if (kt + 1 < nk) lstore(buf ^ 1);
+    if (kt + 1 < nk) lstore(buf ^ 1, (kt + 1) * TL_BK);
     __syncthreads();
   }
 

@@ -95,7 +95,7 @@ struct AttnWave {
       const bool ok = kb + 16 * tt + r16 < kv_len;
       const bf16_t* kp = ksrc.ptr(tt, ok ? r16 : 0) + 8 * g;
 #pragma unroll
-      for (int s = 0; s < KS; s++) kf[tt][s] = ldg16(kp + 32 * s, ok);
+      for (int s = 0; s < KS; s++) kf[tt][s] = ldg16_raw(kp + 32 * s);  // keys past the end get score -inf below
     }
     uint4 vr[2][NDV][8];  // [32-key chunk][dim set][slot]
 #pragma unroll
@@ -108,7 +108,7 @@ struct AttnWave {
 #pragma unroll
         for (int ds = 0; ds < NDV; ds++) {
           const bool dok = 128 * ds + 8 * r16 < DV;
-          vr[ch][ds][idx] = ldg16(vp + (dok ? 128 * ds + 8 * r16 : 0), ok && dok);
+          vr[ch][ds][idx] = ldg16_raw(vp + (dok ? 128 * ds + 8 * r16 : 0));
         }
       }
 
@@ -165,6 +165,18 @@ struct AttnWave {
       pf[t][0] = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
       pf[t][1] = make_uint4(pw[2][0], pw[2][1], pw[3][0], pw[3][1]);
     }
+
+    // values of keys past the end must be exact zeros (their probability is 0, but 0 * garbage
+    // could be NaN); done here, after the score MFMAs, so the loads stay in flight until now
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++)
+#pragma unroll
+      for (int idx = 0; idx < 8; idx++) {
+        const bool ok = kb + 16 * (2 * ch + (idx >> 2)) + 4 * g + (idx & 3) < kv_len;
+#pragma unroll
+        for (int ds = 0; ds < NDV; ds++)
+          vr[ch][ds][idx] = mask16(vr[ch][ds][idx], ok && (128 * ds + 8 * r16 < DV));
+      }
 
     // ---- P V : out^T[dim 8 i + td][query r16]
 #pragma unroll
