@@ -57,6 +57,58 @@ struct AttnParams {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Where a sequence's keys and values live. SRC_FAST: paged, page size a power of two >= 16, so a
+// 16-key tile lies inside one page and its page id is wave-uniform. SRC_GENERIC: paged, any page
+// size (one table lookup per key). SRC_PACKED: contiguous rows [Tk, Hkv, D].
+enum : int { SRC_FAST = 0, SRC_GENERIC = 1, SRC_PACKED = 2 };
+
+template <int KIND>
+struct KVSource {
+  const bf16_t* kbase;  // + kv head offset (packed: + first key of the sequence)
+  const bf16_t* vbase;
+  const int* bt;        // this sequence's block-table row
+  int64_t skb, skp, svb, svp;
+  int ps, shift, last;  // last = kv_len - 1; every address is clamped to an existing key
+
+  struct Tiles { int64_t k[4], v[4]; };  // element offsets of the four 16-key tiles of a block
+
+  __device__ __forceinline__ Tiles tiles(int kb) const {
+    Tiles t;
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++) {
+      t.k[tt] = 0; t.v[tt] = 0;
+      if constexpr (KIND == SRC_FAST) {
+        const int key = kb + 16 * tt;
+        const int kk = key <= last ? key : 0;  // a tile past the end is never dereferenced for real
+        const int64_t pg = bt[kk >> shift];
+        const int64_t off = kk & (ps - 1);
+        t.k[tt] = pg * skb + off * skp;
+        t.v[tt] = pg * svb + off * svp;
+      }
+    }
+    return t;
+  }
+  // row of key kb + 16 tt + within; `within` must already be 0 for keys past the end (FAST)
+  __device__ __forceinline__ const bf16_t* krow(const Tiles& t, int kb, int tt, int within) const {
+    if constexpr (KIND == SRC_FAST) return kbase + t.k[tt] + (int64_t)within * skp;
+    const int key = min(kb + 16 * tt + within, last);
+    if constexpr (KIND == SRC_PACKED) return kbase + (int64_t)key * skp;
+    int pg, off;
+    if (shift >= 0) { pg = key >> shift; off = key & (ps - 1); }
+    else { pg = key / ps; off = key - pg * ps; }
+    return kbase + (int64_t)bt[pg] * skb + (int64_t)off * skp;
+  }
+  __device__ __forceinline__ const bf16_t* vrow(const Tiles& t, int kb, int tt, int within) const {
+    if constexpr (KIND == SRC_FAST) return vbase + t.v[tt] + (int64_t)within * svp;
+    const int key = min(kb + 16 * tt + within, last);
+    if constexpr (KIND == SRC_PACKED) return vbase + (int64_t)key * svp;
+    int pg, off;
+    if (shift >= 0) { pg = key >> shift; off = key & (ps - 1); }
+    else { pg = key / ps; off = key - pg * ps; }
+    return vbase + (int64_t)bt[pg] * svb + (int64_t)off * svp;
+  }
+};
+
 template <int DK, int DV, int QT>
 struct AttnWave {
   static constexpr int KS = DK / 32;           // MFMA k-steps for S
@@ -68,6 +120,9 @@ struct AttnWave {
   int qpos[QT];  // last visible key of this lane's query row; -1 = row not valid
   float m[QT], l[QT];
   f32x4 acc[QT][NACC];
+  // K and V of the block being worked on / in flight
+  uint4 kf[4][KS];
+  uint4 vr[2][NDV][8];  // [32-key chunk][dim set][slot]
 
   __device__ __forceinline__ void reset_chunk() {
 #pragma unroll
@@ -79,41 +134,42 @@ struct AttnWave {
     }
   }
 
-  // One 64-key block at absolute key offset kb. ksrc / vsrc resolve (16-key tile, key within
-  // tile) to the address of that key's row for this kv head.
-  template <typename Rows>
-  __device__ __forceinline__ void block(int kb, int kv_len, float c, Rows& ksrc, Rows& vsrc) {
-    const int lane = threadIdx.x & 63;
-    const int r16 = lane & 15, g = lane >> 4;
-    ksrc.prepare(kb, kv_len);
-    vsrc.prepare(kb, kv_len);
-
-    // ---- issue all K and V loads of the block
-    uint4 kf[4][KS];
+  // lane (r16, g) fetches key 16 tt + r16, dims 32 s + 8 g .. +8: the MFMA A operand of S^T.
+  // Keys past the end read an existing row instead; their scores are set to -inf later.
+  template <typename Src>
+  __device__ __forceinline__ void issue_k(const Src& src, const typename Src::Tiles& tl, int kb, int kv_len) {
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int tt = 0; tt < 4; tt++) {
       const bool ok = kb + 16 * tt + r16 < kv_len;
-      const bf16_t* kp = ksrc.ptr(tt, ok ? r16 : 0) + 8 * g;
+      const bf16_t* kp = src.krow(tl, kb, tt, ok ? r16 : 0) + 8 * g;
 #pragma unroll
-      for (int s = 0; s < KS; s++) kf[tt][s] = ldg16_raw(kp + 32 * s);  // keys past the end get score -inf below
+      for (int s = 0; s < KS; s++) kf[tt][s] = ldg16_raw(kp + 32 * s);
     }
-    uint4 vr[2][NDV][8];  // [32-key chunk][dim set][slot]
+  }
+  // lane (r16, g) fetches, for slot idx of 32-key chunk ch, key 32 ch + 16 (idx/4) + 4 g + idx%4,
+  // dims 8 r16 .. +8 (16 lanes cover one 256-byte row)
+  template <typename Src>
+  __device__ __forceinline__ void issue_v(const Src& src, const typename Src::Tiles& tl, int kb, int kv_len) {
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int ch = 0; ch < 2; ch++)
 #pragma unroll
       for (int idx = 0; idx < 8; idx++) {
         const int tt = 2 * ch + (idx >> 2), within = 4 * g + (idx & 3);
         const bool ok = kb + 16 * tt + within < kv_len;
-        const bf16_t* vp = vsrc.ptr(tt, ok ? within : 0);
+        const bf16_t* vp = src.vrow(tl, kb, tt, ok ? within : 0);
 #pragma unroll
         for (int ds = 0; ds < NDV; ds++) {
           const bool dok = 128 * ds + 8 * r16 < DV;
           vr[ch][ds][idx] = ldg16_raw(vp + (dok ? 128 * ds + 8 * r16 : 0));
         }
       }
+  }
 
-    // ---- scores and softmax statistics per query tile
-    uint4 pf[QT][2];
+  // scores of the 64-key block at kb from kf, online-softmax update, P packed for the PV MFMAs
+  __device__ __forceinline__ void scores(int kb, float c, uint4 (&pf)[QT][2]) {
+    const int lane = threadIdx.x & 63, g = lane >> 4;
 #pragma unroll
     for (int t = 0; t < QT; t++) {
       // S^T tiles: lane holds keys kb + 16 tt + 4 g + r for query column r16
@@ -165,31 +221,34 @@ struct AttnWave {
       pf[t][0] = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
       pf[t][1] = make_uint4(pw[2][0], pw[2][1], pw[3][0], pw[3][1]);
     }
+  }
 
-    // values of keys past the end must be exact zeros (their probability is 0, but 0 * garbage
-    // could be NaN); done here, after the score MFMAs, so the loads stay in flight until now
+  // acc += P V with the block's values in vr. Values of keys past the end are zeroed first (their
+  // probability is 0, but 0 * garbage could be NaN).
+  __device__ __forceinline__ void pv(int kb, int kv_len, const uint4 (&pf)[QT][2]) {
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+    const bool tail = kb + ATT_BLOCK > kv_len;  // wave-uniform: only a sequence's last block
 #pragma unroll
     for (int ch = 0; ch < 2; ch++)
 #pragma unroll
-      for (int idx = 0; idx < 8; idx++) {
-        const bool ok = kb + 16 * (2 * ch + (idx >> 2)) + 4 * g + (idx & 3) < kv_len;
+      for (int ds = 0; ds < NDV; ds++) {
+        uint4 row[8];
 #pragma unroll
-        for (int ds = 0; ds < NDV; ds++)
-          vr[ch][ds][idx] = mask16(vr[ch][ds][idx], ok && (128 * ds + 8 * r16 < DV));
-      }
-
-    // ---- P V : out^T[dim 8 i + td][query r16]
-#pragma unroll
-    for (int ch = 0; ch < 2; ch++)
-#pragma unroll
-      for (int ds = 0; ds < NDV; ds++)
+        for (int idx = 0; idx < 8; idx++) {
+          row[idx] = vr[ch][ds][idx];
+          const bool dok = 128 * ds + 8 * r16 < DV;
+          if (tail || !dok) {
+            const bool ok = kb + 16 * (2 * ch + (idx >> 2)) + 4 * g + (idx & 3) < kv_len;
+            row[idx] = mask16(row[idx], ok && dok);
+          }
+        }
 #pragma unroll
         for (int td = 0; td < 8; td++) {
           // 8x8 bf16 transpose: fragment td takes dim 8 r16 + td of the 8 key slots
           uint32_t w[4];
 #pragma unroll
           for (int qd = 0; qd < 4; qd++) {
-            const uint4 ra = vr[ch][ds][2 * qd], rb = vr[ch][ds][2 * qd + 1];
+            const uint4 ra = row[2 * qd], rb = row[2 * qd + 1];
             const uint32_t a = (td < 2) ? ra.x : (td < 4) ? ra.y : (td < 6) ? ra.z : ra.w;
             const uint32_t b = (td < 2) ? rb.x : (td < 4) ? rb.y : (td < 6) ? rb.z : rb.w;
             w[qd] = (td & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
@@ -198,6 +257,27 @@ struct AttnWave {
 #pragma unroll
           for (int t = 0; t < QT; t++) acc[t][ds * 8 + td] = mfma16(vf, pf[t][ch], acc[t][ds * 8 + td]);
         }
+      }
+  }
+
+  // One chunk: keys [kb0, kb_end) in 64-key blocks, chunk state reset first. The loads of block
+  // b+1 are issued as soon as block b has consumed the registers they land in (K after the score
+  // MFMAs, V after the PV MFMAs), so a wavefront always has a block of K or V in flight.
+  template <typename Src>
+  __device__ __forceinline__ void run_chunk(const Src& src, int kb0, int kb_end, int kv_len, float c) {
+    reset_chunk();
+    typename Src::Tiles tl = src.tiles(kb0);
+    issue_k(src, tl, kb0, kv_len);
+    issue_v(src, tl, kb0, kv_len);
+    for (int kb = kb0; kb < kb_end; kb += ATT_BLOCK) {
+      const bool more = kb + ATT_BLOCK < kb_end;
+      if (more) tl = src.tiles(kb + ATT_BLOCK);  // page ids of the next block: ready before they are needed
+      uint4 pf[QT][2];
+      scores(kb, c, pf);
+      if (more) issue_k(src, tl, kb + ATT_BLOCK, kv_len);
+      pv(kb, kv_len, pf);
+      if (more) issue_v(src, tl, kb + ATT_BLOCK, kv_len);
+    }
   }
 };
 
@@ -209,56 +289,30 @@ __device__ __forceinline__ void fold_scales(float M, float mc, float& Mn, float&
   B = fast_exp2(mc - ms);
 }
 
-// Row sources. prepare() is called once per 64-key block; ptr(tt, within) is the row of key
-// kb + 16 tt + within.
-struct PagedRows {
-  const bf16_t* base;  // cache + kv_head offset
-  const int* bt;       // this sequence's block-table row
-  int64_t sb, sp;
-  int ps, shift;
-  int kb_, last_;  // block start; last existing key (addresses are clamped to it)
-  int64_t t0, t1, t2, t3;  // fast path (page size a power of two >= 16): a tile lies in one page
-  __device__ __forceinline__ int64_t tile_base(int key, int kv_len) const {
-    const int kk = key < kv_len ? key : 0;  // tiles past the end are never dereferenced
-    return (int64_t)bt[kk >> shift] * sb + (int64_t)(kk & (ps - 1)) * sp;
+template <int KIND>
+__device__ __forceinline__ KVSource<KIND> make_source(const AttnParams& p, int seq, int kvh, int k0, int kv_len) {
+  KVSource<KIND> s;
+  s.skb = p.skb; s.skp = p.skp; s.svb = p.svb; s.svp = p.svp;
+  s.ps = p.page_size; s.shift = p.page_shift; s.last = kv_len - 1;
+  if constexpr (KIND == SRC_PACKED) {
+    s.kbase = p.k + (int64_t)k0 * p.skp + (int64_t)kvh * p.skh;
+    s.vbase = p.v + (int64_t)k0 * p.svp + (int64_t)kvh * p.svh;
+    s.bt = nullptr;
+  } else {
+    s.kbase = p.k + (int64_t)kvh * p.skh;
+    s.vbase = p.v + (int64_t)kvh * p.svh;
+    s.bt = p.block_table + (int64_t)seq * p.bt_stride;
   }
-  __device__ __forceinline__ void prepare(int kb, int kv_len) {
-    kb_ = kb;
-    last_ = kv_len - 1;
-    if (shift >= 4) {
-      t0 = tile_base(kb, kv_len);
-      t1 = tile_base(kb + 16, kv_len);
-      t2 = tile_base(kb + 32, kv_len);
-      t3 = tile_base(kb + 48, kv_len);
-    }
-  }
-  __device__ __forceinline__ const bf16_t* ptr(int tt, int within) const {
-    if (shift >= 4) return base + (tt == 0 ? t0 : tt == 1 ? t1 : tt == 2 ? t2 : t3) + (int64_t)within * sp;
-    const int key = min(kb_ + 16 * tt + within, last_);  // never index the table past the sequence
-    int pg, off;
-    if (shift >= 0) { pg = key >> shift; off = key & (ps - 1); }
-    else { pg = key / ps; off = key - pg * ps; }
-    return base + (int64_t)bt[pg] * sb + (int64_t)off * sp;
-  }
-};
-struct PackedRows {
-  const bf16_t* base;  // already offset to the sequence's first key and the kv head
-  int64_t sp;
-  int kb_, last_;
-  __device__ __forceinline__ void prepare(int kb, int kv_len) { kb_ = kb; last_ = kv_len - 1; }
-  __device__ __forceinline__ const bf16_t* ptr(int tt, int within) const {
-    // clamp: a tile past the sequence's last key must not point past the packed tensor
-    return base + (int64_t)min(kb_ + 16 * tt + within, last_) * sp;
-  }
-};
+  return s;
+}
 
 // ---------------------------------------------------------------------------------------
-// Decode: every sequence has at most one query token. grid = (max_chunks, Hkv, B), one
+// Decode: every sequence has at most one query token. grid = (Hkv, B, max_chunks), one
 // wavefront per block; query heads of the kv head are the MFMA columns (G <= 16 * QT).
 // ---------------------------------------------------------------------------------------
-template <int DK, int DV, int QT>
+template <int DK, int DV, int QT, int KIND>
 __global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
-  const int chunk = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int kvh = blockIdx.x, seq = blockIdx.y, chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
@@ -280,13 +334,8 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
 #pragma unroll
     for (int s = 0; s < DK / 32; s++) w.qf[t][s] = ldg16(qp + 32 * s, ok);
   }
-  w.reset_chunk();
-  PagedRows kr{p.k + (int64_t)kvh * p.skh, p.block_table + (int64_t)seq * p.bt_stride, p.skb, p.skp,
-               p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
-  PagedRows vr{p.v + (int64_t)kvh * p.svh, p.block_table + (int64_t)seq * p.bt_stride, p.svb, p.svp,
-               p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
-  const int kend = min(kstart + ATT_CHUNK, kv_len);
-  for (int kb = kstart; kb < kend; kb += ATT_BLOCK) w.block(kb, kv_len, p.qk_scale, kr, vr);
+  const KVSource<KIND> src = make_source<KIND>(p, seq, kvh, 0, kv_len);
+  w.run_chunk(src, kstart, min(kstart + ATT_CHUNK, kv_len), kv_len, p.qk_scale);
 
   // write the chunk state: lane holds dims 128 ds + 32 g + 8 r + td for head column r16
 #pragma unroll
@@ -355,13 +404,13 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
 // General (prefill / mixed / packed) kernel. grid = (q tiles, Hq, B); 4 wavefronts per block,
 // wavefront v owns query rows [64 QT bx + 16 QT v, +16 QT) of the sequence (local indices).
 // ---------------------------------------------------------------------------------------
-template <int DK, int DV, int QT, bool PAGED>
+template <int DK, int DV, int QT, int KIND>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
   const int head = blockIdx.y, seq = blockIdx.z;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   int kv_len, k0 = 0;
-  if constexpr (PAGED) kv_len = p.seqused_k[seq];
+  if constexpr (KIND != SRC_PACKED) kv_len = p.seqused_k[seq];
   else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int i0 = (blockIdx.x * 4 + wave) * 16 * QT;
@@ -395,34 +444,20 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
     for (int i = 0; i < AttnWave<DK, DV, QT>::NACC; i++) ACC[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  auto run = [&](auto& kr, auto& vr) {
-    for (int cs = 0; cs <= maxpos; cs += ATT_CHUNK) {
-      w.reset_chunk();
-      const int kend = min(cs + ATT_CHUNK, maxpos + 1);
-      for (int kb = cs; kb < kend; kb += ATT_BLOCK) w.block(kb, kv_len, p.qk_scale, kr, vr);
+  const KVSource<KIND> src = make_source<KIND>(p, seq, kvh, k0, kv_len);
+  for (int cs = 0; cs <= maxpos; cs += ATT_CHUNK) {
+    w.run_chunk(src, cs, min(cs + ATT_CHUNK, maxpos + 1), kv_len, p.qk_scale);
 #pragma unroll
-      for (int t = 0; t < QT; t++) {
-        float Mn, A, B;
-        fold_scales(M[t], w.m[t], Mn, A, B);
-        L[t] = L[t] * A + w.l[t] * B;
+    for (int t = 0; t < QT; t++) {
+      float Mn, A, B;
+      fold_scales(M[t], w.m[t], Mn, A, B);
+      L[t] = L[t] * A + w.l[t] * B;
 #pragma unroll
-        for (int i = 0; i < AttnWave<DK, DV, QT>::NACC; i++)
+      for (int i = 0; i < AttnWave<DK, DV, QT>::NACC; i++)
 #pragma unroll
-          for (int r = 0; r < 4; r++) ACC[t][i][r] = ACC[t][i][r] * A + w.acc[t][i][r] * B;
-        M[t] = Mn;
-      }
+        for (int r = 0; r < 4; r++) ACC[t][i][r] = ACC[t][i][r] * A + w.acc[t][i][r] * B;
+      M[t] = Mn;
     }
-  };
-  if constexpr (PAGED) {
-    PagedRows kr{p.k + (int64_t)kvh * p.skh, p.block_table + (int64_t)seq * p.bt_stride, p.skb,
-                 p.skp, p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
-    PagedRows vr{p.v + (int64_t)kvh * p.svh, p.block_table + (int64_t)seq * p.bt_stride, p.svb,
-                 p.svp, p.page_size, p.page_shift, 0, 0, 0, 0, 0, 0};
-    run(kr, vr);
-  } else {
-    PackedRows kr{p.k + (int64_t)k0 * p.skp + (int64_t)kvh * p.skh, p.skp, 0, 0};
-    PackedRows vr{p.v + (int64_t)k0 * p.svp + (int64_t)kvh * p.svh, p.svp, 0, 0};
-    run(kr, vr);
   }
 
 #pragma unroll
@@ -474,19 +509,27 @@ __global__ __launch_bounds__(256) void store_kv_kernel(const uint8_t* __restrict
 
 template <int DK, int DV>
 static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hipStream_t stream) {
+  const bool fast = p.page_shift >= 4;  // page size a power of two >= 16
   if (mode == 0) {  // decode split + combine
     const int G = p.Hq / p.Hkv;
-    dim3 grid(p.max_chunks, p.Hkv, p.num_seqs);
-    if (G <= 16) attn_decode_split_kernel<DK, DV, 1><<<grid, 64, 0, stream>>>(p);
-    else if (G <= 32) attn_decode_split_kernel<DK, DV, 2><<<grid, 64, 0, stream>>>(p);
-    else return VX_ERR_UNSUPPORTED;
+    dim3 grid(p.Hkv, p.num_seqs, p.max_chunks);
+    if (G <= 16) {
+      if (fast) attn_decode_split_kernel<DK, DV, 1, SRC_FAST><<<grid, 64, 0, stream>>>(p);
+      else attn_decode_split_kernel<DK, DV, 1, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
+    } else if (G <= 32) {
+      if (fast) attn_decode_split_kernel<DK, DV, 2, SRC_FAST><<<grid, 64, 0, stream>>>(p);
+      else attn_decode_split_kernel<DK, DV, 2, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
+    } else {
+      return VX_ERR_UNSUPPORTED;
+    }
     attn_decode_combine_kernel<DV><<<dim3(p.Hq, p.num_seqs), 64, 0, stream>>>(p);
   } else {
-    constexpr int QT = (DK > 192) ? 1 : 2;
+    constexpr int QT = (DK > 128) ? 1 : 2;
     const int rows = max_q > 0 ? max_q : total_q;
     dim3 grid((rows + 64 * QT - 1) / (64 * QT), p.Hq, p.num_seqs);
-    if (mode == 1) attn_prefill_kernel<DK, DV, QT, true><<<grid, 256, 0, stream>>>(p);
-    else attn_prefill_kernel<DK, DV, QT, false><<<grid, 256, 0, stream>>>(p);
+    if (mode == 2) attn_prefill_kernel<DK, DV, QT, SRC_PACKED><<<grid, 256, 0, stream>>>(p);
+    else if (fast) attn_prefill_kernel<DK, DV, QT, SRC_FAST><<<grid, 256, 0, stream>>>(p);
+    else attn_prefill_kernel<DK, DV, QT, SRC_GENERIC><<<grid, 256, 0, stream>>>(p);
   }
   return launch_status();
 }
