@@ -157,6 +157,11 @@ int vx_moe_scatter(const void* x, void* out, const int* index, int64_t T, int k,
                    int64_t ldo, hipStream_t stream);
 int vx_moe_gather(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
                   int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, hipStream_t stream);
+/* Same, and additionally h = RMSNorm(y) with norm_weight (mode as vx_rms_norm): the RMSNorm that
+ * follows the MoE block in the decoder layer, fused; bit-identical to vx_moe_gather + vx_rms_norm. */
+int vx_moe_gather_norm(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                       int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
+                       int64_t ldh, float eps, int mode, hipStream_t stream);
 
 /* ---- decoder-layer glue ---------------------------------------------------------------- */
 

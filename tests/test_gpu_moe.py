@@ -160,3 +160,29 @@ def test_fused_moe_rows_do_not_depend_on_token_count():
     assert_bitwise(one, full[3000:3001], "token 3000 alone")
     ref = OM.fused_moe_ref(x[:128], w[:128], sel[:128], gate, up, down)
     assert_bf16_close(full[:128], ref, max_ulp=2, atol_frac=2e-3, what="T=4096 rows vs oracle")
+
+
+def test_gather_with_fused_norm_equals_separate_kernels():
+    g = torch.Generator().manual_seed(21)
+    for T, k, H in ((37, 8, 2048), (5, 2, 256), (9, 4, 4096)):
+        x = torch.randn(T * k, H, generator=g).to(torch.bfloat16).cuda()
+        res = torch.randn(T, H, generator=g).to(torch.bfloat16).cuda()
+        w = (1 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16).cuda()
+        idx = torch.randperm(T * k, generator=g).to(torch.int32).view(T, k).cuda()
+        y_ref = ops.moe_gather(x, idx, residual=res)
+        acc = torch.zeros(T, H)
+        for i in range(k):
+            acc = acc + x.cpu()[idx.cpu()[:, i].long()].float()
+        want = (res.cpu().float() + acc.to(torch.bfloat16).float()).to(torch.bfloat16)
+        assert_bitwise(y_ref, want, "gather + residual")
+        for two in (True, False):
+            h_ref = ops.rms_norm(y_ref, w, 1e-6, hf_two_rounding=two)
+            y = torch.empty_like(y_ref)
+            h = torch.empty_like(y_ref)
+            ops.moe_gather(x, idx, residual=res, out=y, norm_weight=w, norm_out=h, eps=1e-6, hf_two_rounding=two)
+            assert_bitwise(y, y_ref, "fused gather output")
+            assert_bitwise(h, h_ref, "fused norm output")
+        # in place over the residual
+        r2 = res.clone()
+        ops.moe_gather(x, idx, residual=r2, out=r2)
+        assert_bitwise(r2, y_ref, "in-place gather")

@@ -123,6 +123,15 @@ int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void
     if (mt == 1) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
     else if (mt == 2) gemm_stream_kernel<2, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
     else gemm_stream_kernel<4, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  } else if (kind == 2) {  // streaming with 16 k-steps in flight
+    if (mt != 1 && mt != 2 && mt != 4) return VX_ERR_ARG;
+    const int64_t bm = 16 * mt;
+    const int64_t my = (M + bm - 1) / bm;
+    if (my > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)my);
+    if (mt == 1) gemm_stream_kernel<1, EPI_PLAIN, false, 16><<<grid, 256, 0, stream>>>(p);
+    else if (mt == 2) gemm_stream_kernel<2, EPI_PLAIN, false, 16><<<grid, 256, 0, stream>>>(p);
+    else gemm_stream_kernel<4, EPI_PLAIN, false, 16><<<grid, 256, 0, stream>>>(p);
   } else if (kind == 1) {
     const int64_t my = (M + TL_BM - 1) / TL_BM;
     if (my > 65535) return VX_ERR_UNSUPPORTED;

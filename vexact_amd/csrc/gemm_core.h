@@ -60,13 +60,14 @@ struct StreamCfg {
   static constexpr int KC = 32768 / BM;           // K elements staged per LDS fill
   static constexpr int ROW_BYTES = KC * 2 + 16;   // +16: rows land on distinct bank groups
   static constexpr int LDS_BYTES = BM * ROW_BYTES;
-  static constexpr int U = 8;                     // k-steps of weight loads in flight
 };
 
-template <int MT, int EPI, bool GROUPED>
+// U = k-steps of weight loads a wavefront keeps in flight (one group); 32 U must divide KC.
+template <int MT, int EPI, bool GROUPED, int U = 8>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   using Cfg = StreamCfg<MT>;
-  constexpr int BM = Cfg::BM, KC = Cfg::KC, RB = Cfg::ROW_BYTES, U = Cfg::U;
+  constexpr int BM = Cfg::BM, KC = Cfg::KC, RB = Cfg::ROW_BYTES;
+  static_assert(KC % (32 * U) == 0, "a staged chunk must hold whole groups");
   __shared__ __attribute__((aligned(16))) uint8_t xs[Cfg::LDS_BYTES];
 
   int row0, rows;

@@ -228,7 +228,8 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const bf16_t* __restri
 }
 
 // y[t, :] = r16( sum_{i<k, ascending} f32(x[index[t, i], :]) ); optional residual:
-// y = r16(f32(res[t]) + f32(r16(sum))). One 256-thread block per token.
+// y = r16(f32(res[t]) + f32(r16(sum))). One 256-thread block per token. Scalar fallback for
+// layouts the vector kernel cannot take.
 __global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restrict__ x,
                                                          const int* __restrict__ index,
                                                          const bf16_t* res, bf16_t* y, int k, int H,
@@ -240,6 +241,68 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const bf16_t* __restric
     bf16_t o = f32_to_bf16(acc);
     if (res) o = f32_to_bf16(bf16_to_f32(res[t * ldr + c]) + bf16_to_f32(o));
     y[t * ldy + c] = o;
+  }
+}
+
+// Vector version (H % 4 == 0, 8-byte aligned rows) with an optional fused RMSNorm of the result:
+// h[t] = rmsnorm(y[t]) with weight nw (mode 1: round(nw * round(y * inv)); mode 0: round(y * inv * nw)).
+// Thread t owns the 4-element vectors t, t + 256, ... : the same ownership, in-thread order and
+// block reduction as the 256-thread RMSNorm kernel, so fusing does not change a bit.
+template <int MAXV>  // vectors per thread kept in registers (H <= 1024 * MAXV)
+__global__ __launch_bounds__(256) void moe_gather_vec_kernel(const bf16_t* __restrict__ x,
+                                                             const int* __restrict__ index,
+                                                             const bf16_t* res, bf16_t* y, int k, int H,
+                                                             int64_t ldx, int64_t ldr, int64_t ldy,
+                                                             const bf16_t* __restrict__ nw, bf16_t* h,
+                                                             int64_t ldh, float eps, int mode) {
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  float o[MAXV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXV; j++) {
+    const int c = 4 * (tid + 256 * j);
+    if (c < H) {
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      for (int i = 0; i < k; i++) {
+        const uint2 raw = *(const uint2*)(x + (int64_t)index[t * k + i] * ldx + c);
+        a0 += bf16lo(raw.x); a1 += bf16hi(raw.x); a2 += bf16lo(raw.y); a3 += bf16hi(raw.y);
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(a0, a1);
+      pk.y = pack_bf16x2(a2, a3);
+      if (res) {
+        const uint2 rr = *(const uint2*)(res + t * ldr + c);
+        pk.x = pack_bf16x2(bf16lo(rr.x) + bf16lo(pk.x), bf16hi(rr.x) + bf16hi(pk.x));
+        pk.y = pack_bf16x2(bf16lo(rr.y) + bf16lo(pk.y), bf16hi(rr.y) + bf16hi(pk.y));
+      }
+      *(uint2*)(y + t * ldy + c) = pk;
+      o[j][0] = bf16lo(pk.x); o[j][1] = bf16hi(pk.x); o[j][2] = bf16lo(pk.y); o[j][3] = bf16hi(pk.y);
+#pragma unroll
+      for (int e = 0; e < 4; e++) ss += o[j][e] * o[j][e];
+    }
+  }
+  if (!h) return;
+  const float tot = block_sum<4>(ss, red);
+  const float inv = 1.0f / sqrtf(tot / (float)H + eps);
+#pragma unroll
+  for (int j = 0; j < MAXV; j++) {
+    const int c = 4 * (tid + 256 * j);
+    if (c < H) {
+      const uint2 wr = *(const uint2*)(nw + c);
+      const float wf[4] = {bf16lo(wr.x), bf16hi(wr.x), bf16lo(wr.y), bf16hi(wr.y)};
+      float r[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (mode == 0) r[e] = o[j][e] * inv * wf[e];
+        else r[e] = wf[e] * bf16_to_f32(f32_to_bf16(o[j][e] * inv));
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(r[0], r[1]);
+      pk.y = pack_bf16x2(r[2], r[3]);
+      *(uint2*)(h + t * ldh + c) = pk;
+    }
   }
 }
 
@@ -378,14 +441,40 @@ int vx_moe_scatter(const void* x, void* out, const int* index, int64_t T, int k,
   return launch_status();
 }
 
-int vx_moe_gather(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
-                  int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, hipStream_t stream) {
+// y = gather-sum (+ residual); when norm_weight and h are given, also h = RMSNorm(y) (mode as in
+// vx_rms_norm). The fused norm needs H % 4 == 0, H <= 8192 and 8-byte aligned rows.
+int vx_moe_gather_norm(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                       int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
+                       int64_t ldh, float eps, int mode, hipStream_t stream) {
   if (!x || !y || !index || T < 0 || k <= 0 || H <= 0 || H > 0x7fffffff) return VX_ERR_ARG;
+  if ((norm_weight == nullptr) != (h == nullptr)) return VX_ERR_ARG;
+  if (mode != 0 && mode != 1) return VX_ERR_ARG;
   if (T == 0) return VX_OK;
   if (T > 0x7fffffffLL) return VX_ERR_ARG;
-  moe_gather_kernel<<<(unsigned)T, 256, 0, stream>>>((const bf16_t*)x, index, (const bf16_t*)residual,
-                                                     (bf16_t*)y, k, (int)H, ldx, ldr, ldy);
+  const bool vec = (H % 4 == 0) && (ldx % 4 == 0) && (ldy % 4 == 0) && (ldr % 4 == 0) && (ldh % 4 == 0) &&
+                   (((uintptr_t)x | (uintptr_t)y | (uintptr_t)residual | (uintptr_t)h | (uintptr_t)norm_weight) % 8 == 0) &&
+                   H <= 8192;
+  if (!vec) {
+    if (h) return VX_ERR_UNSUPPORTED;
+    moe_gather_kernel<<<(unsigned)T, 256, 0, stream>>>((const bf16_t*)x, index, (const bf16_t*)residual,
+                                                       (bf16_t*)y, k, (int)H, ldx, ldr, ldy);
+    return launch_status();
+  }
+#define VX_GV(MV)                                                                                     \
+  moe_gather_vec_kernel<MV><<<(unsigned)T, 256, 0, stream>>>(                                         \
+      (const bf16_t*)x, index, (const bf16_t*)residual, (bf16_t*)y, k, (int)H, ldx, ldr, ldy,         \
+      (const bf16_t*)norm_weight, (bf16_t*)h, ldh, eps, mode)
+  if (H <= 1024) VX_GV(1);
+  else if (H <= 2048) VX_GV(2);
+  else if (H <= 4096) VX_GV(4);
+  else VX_GV(8);
+#undef VX_GV
   return launch_status();
+}
+
+int vx_moe_gather(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                  int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, hipStream_t stream) {
+  return vx_moe_gather_norm(x, index, residual, y, T, k, H, ldx, ldr, ldy, nullptr, nullptr, 0, 0.f, 1, stream);
 }
 
 }  // extern "C"

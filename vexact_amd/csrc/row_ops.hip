@@ -146,6 +146,66 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
   }
 }
 
+// bf16 fast path of rms_norm_kernel: 8-byte loads/stores, row values kept in registers. Same
+// element ownership, in-thread order and reductions as the generic kernel, hence the same bits.
+// Requirements (checked by the launcher): n % 4 == 0, n <= 1024 * MAXV (G = 256) or n <= 512
+// (G = 64), strides % 4 == 0, 8-byte aligned pointers.
+template <int G, int MAXV>
+__global__ __launch_bounds__(256) void rms_norm_bf16v_kernel(const bf16_t* x, const bf16_t* res,
+                                                             const bf16_t* __restrict__ w, bf16_t* y,
+                                                             bf16_t* sum_out, int64_t rows, int n,
+                                                             int64_t xs, int64_t rs, int64_t ys, int64_t ss,
+                                                             float eps, int mode) {
+  __shared__ float red[4];
+  constexpr int RPB = 256 / G;
+  const int sub = threadIdx.x / G, t = threadIdx.x % G;
+  const int64_t row = (int64_t)blockIdx.x * RPB + sub;
+  const bool live = row < rows;
+  float f[MAXV][4];
+  float acc = 0.f;
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < MAXV; j++) {
+      const int c = 4 * (t + G * j);
+      if (c < n) {
+        uint2 raw = *(const uint2*)(x + row * xs + c);
+        if (res) {
+          const uint2 rr = *(const uint2*)(res + row * rs + c);
+          raw.x = pack_bf16x2(bf16lo(raw.x) + bf16lo(rr.x), bf16hi(raw.x) + bf16hi(rr.x));
+          raw.y = pack_bf16x2(bf16lo(raw.y) + bf16lo(rr.y), bf16hi(raw.y) + bf16hi(rr.y));
+          if (sum_out) *(uint2*)(sum_out + row * ss + c) = raw;
+        }
+        f[j][0] = bf16lo(raw.x); f[j][1] = bf16hi(raw.x); f[j][2] = bf16lo(raw.y); f[j][3] = bf16hi(raw.y);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc += f[j][e] * f[j][e];
+      }
+    }
+  }
+  float tot;
+  if constexpr (G == 64) tot = wave_sum(acc);
+  else tot = block_sum<4>(acc, red);
+  if (!live) return;
+  const float inv = 1.0f / sqrtf(tot / (float)n + eps);
+#pragma unroll
+  for (int j = 0; j < MAXV; j++) {
+    const int c = 4 * (t + G * j);
+    if (c < n) {
+      const uint2 wr = *(const uint2*)(w + c);
+      const float wf[4] = {bf16lo(wr.x), bf16hi(wr.x), bf16lo(wr.y), bf16hi(wr.y)};
+      float r[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (mode == 0) r[e] = f[j][e] * inv * wf[e];
+        else r[e] = wf[e] * bf16_to_f32(f32_to_bf16(f[j][e] * inv));
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(r[0], r[1]);
+      pk.y = pack_bf16x2(r[2], r[3]);
+      *(uint2*)(y + row * ys + c) = pk;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // log_softmax / logprob / argmax over rows of [rows, n], split into fixed chunks of
 // LS_CHUNK columns so that few rows still fill the chip. The chunk count depends on n only.
@@ -310,6 +370,20 @@ int vx_rms_norm(const void* x, const void* residual, const void* weight, void* y
   const int64_t rpb = small ? 4 : 1;
   const int64_t blocks = (rows + rpb - 1) / rpb;
   if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  if (dtype == DT_BF16 && n % 4 == 0 && n <= 8192 && ((x_stride | res_stride | y_stride | sum_stride) % 4 == 0) &&
+      (((uintptr_t)x | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)y | (uintptr_t)sum_out) % 8 == 0)) {
+#define VX_RMSV(GG, MV)                                                                            \
+  rms_norm_bf16v_kernel<GG, MV><<<dim3((unsigned)blocks), 256, 0, stream>>>(                       \
+      (const bf16_t*)x, (const bf16_t*)residual, (const bf16_t*)weight, (bf16_t*)y, (bf16_t*)sum_out, \
+      rows, (int)n, x_stride, res_stride, y_stride, sum_stride, eps, mode)
+    if (small) VX_RMSV(64, 2);
+    else if (n <= 1024) VX_RMSV(256, 1);
+    else if (n <= 2048) VX_RMSV(256, 2);
+    else if (n <= 4096) VX_RMSV(256, 4);
+    else VX_RMSV(256, 8);
+#undef VX_RMSV
+    return launch_status();
+  }
 #define VX_LAUNCH_RMS(DT)                                                                       \
   do {                                                                                          \
     using T = Elem<DT>::T;                                                                      \

@@ -267,8 +267,8 @@ class Qwen3MoeDecoder:
             ops.moe_gemm(b.hw, lw["down"], r, out=b.eo)
             nxt = w.layers[li + 1]["in_norm"] if li + 1 < cfg.num_layers else w.final_norm
             # x <- x + sum_slots(eo) ; h <- next norm(x)
-            ops.moe_gather(b.eo, r.scatter_index, residual=b.x, out=b.x)
-            ops.rms_norm(b.x, nxt, cfg.rms_eps, hf_two_rounding=True, out=b.h)
+            ops.moe_gather(b.eo, r.scatter_index, residual=b.x, out=b.x, norm_weight=nxt, norm_out=b.h,
+                           eps=cfg.rms_eps, hf_two_rounding=True)
 
     def _router(self, b: StepBuffers) -> None:
         from . import _lib
