@@ -54,21 +54,16 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u, float w) {
 // Streaming kernel. 256 threads = 4 wavefronts; wavefront v owns weight rows
 // [n0 + 16 v, n0 + 16 v + 16); the block covers 64 weight rows and BM = 16*MT activation rows.
 // ---------------------------------------------------------------------------------------
-template <int MT>
-struct StreamCfg {
-  static constexpr int BM = 16 * MT;
-  static constexpr int KC = 32768 / BM;           // K elements staged per LDS fill
-  static constexpr int ROW_BYTES = KC * 2 + 16;   // +16: rows land on distinct bank groups
-  static constexpr int LDS_BYTES = BM * ROW_BYTES;
-};
-
-// U = k-steps of weight loads a wavefront keeps in flight (one group); 32 U must divide KC.
-template <int MT, int EPI, bool GROUPED, int U = 8>
+// U  = k-steps of weight loads a wavefront keeps in flight (one group);
+// KD = divisor of the staged K chunk: KC = 32768 / (BM * KD) elements per LDS fill (64 KB / KD of
+//      LDS per block, so KD = 2 lets more blocks share a CU). 32 U must divide KC.
+template <int MT, int EPI, bool GROUPED, int U = 8, int KD = 1>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
-  using Cfg = StreamCfg<MT>;
-  constexpr int BM = Cfg::BM, KC = Cfg::KC, RB = Cfg::ROW_BYTES;
+  constexpr int BM = 16 * MT;
+  constexpr int KC = 32768 / (BM * KD);  // K elements staged per LDS fill
+  constexpr int RB = KC * 2 + 16;        // +16: rows land on distinct bank groups
+  __shared__ __attribute__((aligned(16))) uint8_t xs[BM * RB];
   static_assert(KC % (32 * U) == 0, "a staged chunk must hold whole groups");
-  __shared__ __attribute__((aligned(16))) uint8_t xs[Cfg::LDS_BYTES];
 
   int row0, rows;
   int64_t wbase = 0;

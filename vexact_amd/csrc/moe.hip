@@ -395,11 +395,13 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
   p.row_src = row_src;
   p.row_scale = (const bf16_t*)row_scale; p.row_scale_idx = row_scale_idx;
   const unsigned my = (unsigned)max_tiles;
+  // U = 8 k-steps in flight per wavefront, 32 KB activation chunks (two of these blocks plus
+  // their registers fit a CU; measured marginally ahead of 64 KB chunks and of U = 4)
 #define VX_GG(MT)                                                                                  \
   do {                                                                                             \
     const dim3 grid((unsigned)((N + 63) / 64), my);                                                \
-    if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true><<<grid, 256, 0, stream>>>(p);  \
-    else gemm_stream_kernel<MT, EPI_PLAIN, true><<<grid, 256, 0, stream>>>(p);                     \
+    if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true, 8, 2><<<grid, 256, 0, stream>>>(p); \
+    else gemm_stream_kernel<MT, EPI_PLAIN, true, 8, 2><<<grid, 256, 0, stream>>>(p);               \
   } while (0)
   switch (bm) {
     case 16: VX_GG(1); break;
