@@ -140,16 +140,18 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
     xoff[j] = off;
   }
 
-  load_w(0);
-  for (int kc = 0; kc < K; kc += KC) {
-    uint4 stage[NP];
+  // The activation chunk for step c+1 is requested before the MFMAs of chunk c and written to LDS
+  // after them, so its latency hides behind compute instead of stalling every wavefront at a barrier.
+  uint4 stage[NP];
+  auto stage_load = [&](int kc) {
 #pragma unroll
     for (int j = 0; j < NP; j++) {  // all loads of the fill in flight together
       const int c8 = (threadIdx.x + 256 * j) % PPR;
       const bool ok = xoff[j] >= 0 && kc + c8 * 8 < K;
       stage[j] = ldg16_raw(p.x + (ok ? xoff[j] + kc : 0));
     }
-    __syncthreads();  // everyone is done reading the previous fill
+  };
+  auto stage_store = [&](int kc) {
 #pragma unroll
     for (int j = 0; j < NP; j++) {
       const int pc = threadIdx.x + 256 * j;
@@ -157,7 +159,15 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
       const bool ok = xoff[j] >= 0 && kc + c8 * 8 < K;
       *(uint4*)(xs + (pc / PPR) * RB + c8 * 16) = mask16(stage[j], ok);
     }
-    __syncthreads();
+  };
+
+  load_w(0);
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+  for (int kc = 0; kc < K; kc += KC) {
+    const bool more = kc + KC < K;
+    if (more) stage_load(kc + KC);
     const int kend = min(K - kc, KC);
     for (int s0 = 0; s0 < kend; s0 += 32 * U) {
       uint4 ca[U], cb[EPI == EPI_SWIGLU ? U : 1];
@@ -176,6 +186,11 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
           if constexpr (EPI == EPI_SWIGLU) acc2[i] = mfma16(cb[u], xf, acc2[i]);
         }
       }
+    }
+    if (more) {
+      __syncthreads();  // everyone is done reading this chunk
+      stage_store(kc + KC);
+      __syncthreads();
     }
   }
 

@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Per-kernel micro-benchmarks at the headline shapes (Qwen3-30B-A3B decode, batch 256).
+
+Each kernel is launched once per "layer" on its own copy of the weights / KV cache (so nothing is
+served from the caches), the loop over layers is captured in a HIP graph to keep host launch cost
+out, and the replay is timed with events. Prints time, algorithmic bytes (or flops) and the
+fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
+to run under ``rocprofv3 --pmc``.
+
+    python -m vexact_amd.kernel_bench --what moe,attn,gemm,small,prefill,copy
+"""
+
+from __future__ import annotations
+
+import argparse
+import os
+import sys
+
+import numpy as np
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+from vexact_amd import _lib, ops  # noqa: E402
+
+HBM_PEAK = 8.0e12
+MFMA_PEAK = 2.5e15
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--what", default="moe,attn,gemm,small")
+    ap.add_argument("--batch", type=int, default=256)
+    ap.add_argument("--layers", type=int, default=6, help="independent weight / cache copies to rotate over")
+    ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
+    a = ap.parse_args()
+    dev = "cuda"
+    B, NL = a.batch, a.layers
+    H, I, E, k = 2048, 768, 128, 8
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def rnd(*s, std=0.02):
+        t = torch.empty(s, dtype=torch.bfloat16, device=dev)
+        t.normal_(0, std, generator=g)
+        return t
+
+    def timeit(fn, n_layers=NL):
+        for li in range(n_layers):
+            fn(li)
+        torch.cuda.synchronize()
+        if a.nograph:
+            return None
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for li in range(n_layers):
+                fn(li)
+        graph.replay()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(a.reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e-3 / n_layers)
+        return float(np.mean(ts))
+
+    def report(name, t, nbytes=None, flops=None):
+        if t is None:
+            print(f"{name:34s} launched", flush=True)
+        elif flops is not None:
+            print(f"{name:34s} {t * 1e6:9.1f} us  {flops / t / 1e12:8.1f} TFLOP/s  ({flops / t / MFMA_PEAK * 100:5.1f}% of 2.5 PFLOP/s)", flush=True)
+        else:
+            print(f"{name:34s} {t * 1e6:9.1f} us  {nbytes / t / 1e9:8.1f} GB/s  ({nbytes / t / HBM_PEAK * 100:5.1f}% of 8 TB/s)  {nbytes / 1e6:.1f} MB", flush=True)
+
+    what = a.what.split(",")
+    if "moe" in what:
+        x = rnd(B, H, std=1.0)
+        logits = torch.randn(B, E, generator=g, device=dev)
+        w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
+        r = ops.moe_route(idx, E, bm=ops.moe_tile_rows(B))
+        U = int((r.splits > 0).sum())
+        gu = [rnd(E, 2 * I, H) for _ in range(NL)]
+        dn = [rnd(E, H, I) for _ in range(NL)]
+        hw = torch.empty(B * k, I, dtype=torch.bfloat16, device=dev)
+        eo = torch.empty(B * k, H, dtype=torch.bfloat16, device=dev)
+        y = torch.empty(B, H, dtype=torch.bfloat16, device=dev)
+        report(f"moe gate/up (B={B}, {U} experts)",
+               timeit(lambda li: ops.moe_gemm(x, gu[li][:, :I, :], r, w2=gu[li][:, I:, :], row_src=r.sorted_token,
+                                              row_scale=w, row_scale_idx=r.sorted_flat, out=hw)),
+               U * 2 * I * H * 2 + B * H * 2 + B * k * I * 2 + B * k * 6)
+        report("moe down", timeit(lambda li: ops.moe_gemm(hw, dn[li], r, out=eo)), U * H * I * 2 + B * k * I * 2 + B * k * H * 2)
+        report("moe route", timeit(lambda li: ops.moe_route(idx, E, bm=32)), B * k * 16)
+        report("moe gather + residual", timeit(lambda li: ops.moe_gather(eo, r.scatter_index, residual=x, out=y)),
+               B * k * H * 2 + 2 * B * H * 2)
+        report("router top-k", timeit(lambda li: ops.router_topk(logits, k, index_dtype=torch.int32)), B * E * 4)
+    if "attn" in what:
+        Hq, Hkv, D, page = 32, 4, 128, 16
+        rng = np.random.default_rng(5)
+        L = rng.integers(257, 2050, size=B)
+        pages = [(int(n) + page - 1) // page for n in L]
+        pool = sum(pages) + 64
+        perm = rng.permutation(pool)
+        maxb = 4096 // page
+        bt = np.full((B, maxb), -1, np.int32)
+        o = 0
+        for s, p in enumerate(pages):
+            bt[s, :p] = perm[o : o + p]
+            o += p
+        kc = [rnd(pool, page, Hkv, D, std=1.0) for _ in range(NL)]
+        vc = [rnd(pool, page, Hkv, D, std=1.0) for _ in range(NL)]
+        q = rnd(B, Hq, D, std=1.0)
+        cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
+        used = torch.tensor(L, dtype=torch.int32, device=dev)
+        btd = torch.tensor(bt, device=dev)
+        out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
+        ws = torch.empty(_lib.load().vx_paged_attn_decode_workspace_bytes(B, Hq, D, 4096), dtype=torch.uint8, device=dev)
+        report(f"paged decode attention (sum L={int(L.sum())})",
+               timeit(lambda li: ops.paged_attention(q, kc[li], vc[li], cu, used, btd, D**-0.5, 1, out=out, workspace=ws)),
+               int(L.sum()) * 2 * Hkv * D * 2 + 2 * B * Hq * D * 2 + sum(pages) * 4)
+    if "gemm" in what:
+        for name, N, K in (("qkv", 5120, 2048), ("o", 2048, 4096), ("router", 128, 2048), ("lm_head", 151936, 2048)):
+            nl = 2 if N > 100000 else NL
+            ws_ = [rnd(N, K) for _ in range(nl)]
+            xx = rnd(B, K, std=1.0)
+            c = torch.empty(B, N, dtype=torch.bfloat16, device=dev)
+            report(f"gemm {name} M={B} N={N} K={K}", timeit(lambda li: ops.gemm_nt(xx, ws_[li], out=c), n_layers=nl),
+                   2 * (N * K + B * K + B * N))
+            del ws_
+    if "prefill" in what:
+        for name, M, N, K in (("qkv", 8192, 5120, 2048), ("o", 8192, 2048, 4096), ("lm_head", 4096, 151936, 2048),
+                              ("square", 8192, 8192, 8192)):
+            w_ = rnd(N, K)
+            xx = rnd(M, K, std=1.0)
+            c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            report(f"prefill gemm {name} M={M} N={N} K={K}", timeit(lambda li: ops.gemm_nt(xx, w_, out=c), n_layers=2),
+                   flops=2 * M * N * K)
+            del w_, xx, c
+    if "small" in what:
+        x = rnd(B, H, std=1.0)
+        res = rnd(B, H, std=1.0)
+        wn = rnd(H, std=1.0)
+        y = torch.empty_like(x)
+        report("rms_norm", timeit(lambda li: ops.rms_norm(x, wn, 1e-6, hf_two_rounding=True, out=y)), 2 * B * H * 2)
+        report("rms_norm + residual", timeit(lambda li: ops.rms_norm(x, wn, 1e-6, hf_two_rounding=True, residual=res, sum_out=res, out=y)),
+               4 * B * H * 2)
+        Hq, Hkv, D = 32, 4, 128
+        qkv = rnd(B, (Hq + 2 * Hkv) * D, std=1.0)
+        cos = rnd(4096, D, std=1.0)
+        sin = rnd(4096, D, std=1.0)
+        pos = torch.arange(B, device=dev)
+        slot = torch.arange(B, device=dev, dtype=torch.int32)
+        qo = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
+        kcache = rnd(64, 16, Hkv, D)
+        vcache = rnd(64, 16, Hkv, D)
+        report("q/k norm + rope + cache store",
+               timeit(lambda li: ops.qk_norm_rope_store(qkv, wn[:D], wn[:D], cos, sin, pos, slot, qo, kcache, vcache, Hq, Hkv, D, 1e-6)),
+               2 * B * 5120 * 2)
+        logits = rnd(B, 151936, std=1.0)
+        report("greedy token + logprob", timeit(lambda li: ops.logprobs(logits, None, return_tokens=True)), B * 151936 * 2)
+    if "copy" in what:
+        # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        report("copy 1 GiB", timeit(lambda li: dst.copy_(src), n_layers=2), 2 << 30)
+
+
+if __name__ == "__main__":
+    main()
