@@ -6,6 +6,7 @@
 // Replaces matmul_kernel_persistent / matmul_persistent
 // (vexact/batch_invariant_ops/batch_invariant_ops.py:53-228) and _bmm_kernel / triton_bmm (:484-606).
 #include "gemm_core.h"
+#include "gemm_wide.h"
 
 namespace vx {
 
@@ -137,6 +138,8 @@ int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void
     if (my > 65535) return VX_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)my);
     gemm_tiled_kernel<EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
+  } else if (kind == 3) {  // wide 256x256 tiles
+    if (!gemm_wide_launch(p, stream)) return VX_ERR_UNSUPPORTED;
   } else {
     return VX_ERR_ARG;
   }
