@@ -43,6 +43,29 @@ def test_stream_and_tiled_kernels_agree_bitwise():
     assert_bf16_close(ref, O.matmul_ref(a, w.t(), bias), max_ulp=2, what="biased gemm vs oracle")
 
 
+@pytest.mark.parametrize(
+    "M,N,K,bias",
+    [
+        (256, 256, 64, False),  # one tile, one k-step
+        (300, 520, 128, True),  # ragged rows and columns, two k-steps
+        (513, 1023, 192, False),  # row stride of C not a multiple of 8 -> scalar stores
+        (4352, 4096, 128, False),  # 272 tiles on 256 workgroups: some walk a second tile
+        (2048, 5120, 2048, True),  # qkv-projection shape of a prefill chunk
+    ],
+)
+def test_wide_kernel_agrees_bitwise(M, N, K, bias):
+    a = _gen((M, K), 13)
+    w = _gen((N, K), 14, scale=0.05)
+    ag, wg = a.cuda(), w.cuda()
+    bg = _gen((N,), 15).cuda() if bias else None
+    ref = ops.gemm_nt_variant(ag, wg, kind=1, bias=bg)
+    assert_bitwise(ops.gemm_nt_variant(ag, wg, kind=3, bias=bg), ref, f"wide vs tiled {M}x{N}x{K}")
+    if M * N >= 128 * 65536:  # the default entry point picks the wide kernel here
+        full = ops.gemm_nt(ag, wg, bias=bg)
+        assert_bitwise(full, ref, "dispatch vs tiled")
+        assert_bitwise(ops.gemm_nt(ag[1000:1003], wg, bias=bg), full[1000:1003], "3 rows alone vs inside a chunk")
+
+
 def test_lm_head_shape_rows():
     # config-1 shaped: [M, 2048] x [2048, 151936], rows of one draw
     a = _gen((64, 2048), 6)

@@ -93,6 +93,9 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
     else if (mt == 2) gemm_stream_kernel<2, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
     else gemm_stream_kernel<4, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
   } else {
+    // many rows: 256x256 tiles once they fill at least half the chip, else 128x128 tiles
+    const int64_t wide_tiles = ((M + WD_BM - 1) / WD_BM) * ((N + WD_BN - 1) / WD_BN);
+    if (wide_tiles >= 128 && gemm_wide_launch(p, stream)) return launch_status();
     const int64_t mtl = (M + TL_BM - 1) / TL_BM;
     if (mtl > 65535) return VX_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)mtl);
@@ -101,8 +104,9 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
   return launch_status();
 }
 
-// Forces one of the two kernels regardless of M (kind 0 = streaming with 16*mt rows per tile,
-// mt in {1,2,4}; kind 1 = tiled). For tests that check both kernels give the same bits.
+// Forces one kernel regardless of M (kind 0 = streaming with 16*mt rows per tile, mt in {1,2,4};
+// kind 1 = 128x128 tiled; kind 2 = streaming, 16 k-steps in flight; kind 3 = 256x256 wide tiles,
+// needs K % 64 == 0). For tests that check that all kernels give the same bits.
 int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void* c, int64_t M,
                             int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind,
                             int mt, hipStream_t stream) {
