@@ -169,6 +169,8 @@ int vx_moe_gather_norm(const void* x, const int* index, const void* residual, vo
 
 /* Per-head RMSNorm (mode 1 form) of q and k, bf16 rotary embedding from cos/sin tables
  * [max_pos, D], q -> q_out [T, Hq, D], k -> k_out (optional) and k_cache slot, v -> v_cache slot.
+ * Both caches are [blocks, page_size, Hkv, D] views with the given element strides (block, in-page
+ * row, head; D contiguous), so a head-major physical layout [blocks, Hkv, page_size, D] can be used.
  * qkv rows are [q heads | k heads | v heads]. The scatter is store_kvcache
  * (kv_cache_context.py:294-314); norm + rotary are the HuggingFace Qwen3 attention prologue the
  * reference runs between its q/k/v projections and its attention call. */
@@ -176,7 +178,8 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
                           const void* cos_table, const void* sin_table, const void* positions,
                           int pos_i64, const int* slot_mapping, void* q_out, void* k_out,
                           void* k_cache, void* v_cache, int64_t T, int Hq, int Hkv, int D, float eps,
-                          int64_t max_pos, hipStream_t stream);
+                          int64_t max_pos, int page_size, int64_t cache_block_stride,
+                          int64_t cache_row_stride, int64_t cache_head_stride, hipStream_t stream);
 int vx_embedding(const void* table, const void* ids, int ids_i64, void* out, int64_t T, int64_t H,
                  int64_t vocab, hipStream_t stream);
 int vx_fill_i32(int* p, int value, int64_t n, hipStream_t stream);

@@ -72,8 +72,8 @@ def test_tiny_decoder_matches_cpu_oracle_and_is_batch_invariant():
     # CPU oracle on the same input bits, following the GPU's expert choice at near-ties
     wc = w.to_cpu()
     cos, sin = rope_tables(cfg, "cpu")
-    kc = [torch.zeros_like(t, device="cpu") for t in dec.key_cache]
-    vc = [torch.zeros_like(t, device="cpu") for t in dec.value_cache]
+    kc = [torch.zeros(t.shape, dtype=t.dtype) for t in dec.key_cache]
+    vc = [torch.zeros(t.shape, dtype=t.dtype) for t in dec.value_cache]
     report = []
     logits_ref, _, _ = OD.decoder_step_ref(cfg, wc, ids, meta, kc, vc, cos, sin, [r.cpu() for r in rlog], report)
     _check_routing_report(report, "prefill")

@@ -46,7 +46,7 @@ PROTOTYPES = {
     "vx_moe_gather_norm": (_I, [_P, _P, _P, _P, _L, _I, _L, _L, _L, _L, _P, _P, _L, _F, _I, _P]),
     "vx_qk_norm_rope_store": (
         _I,
-        [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _F, _L, _P],
+        [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _F, _L, _I, _L, _L, _L, _P],
     ),
     "vx_embedding": (_I, [_P, _P, _I, _P, _L, _L, _L, _P]),
     "vx_fill_i32": (_I, [_P, _I, _L, _P]),

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const bf16_t* __restrict__ kw, const bf16_t* __restrict__ cos_t, const bf16_t* __restrict__ sin_t,
     const PosT* __restrict__ positions, const int* __restrict__ slots, bf16_t* __restrict__ q_out,
     bf16_t* __restrict__ k_out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int64_t T,
-    int Hq, int Hkv, float eps, int64_t max_pos) {
+    int Hq, int Hkv, float eps, int64_t max_pos, int page_size, int64_t csb, int64_t csp, int64_t csh) {
   const int HT = Hq + 2 * Hkv;
   const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (wid >= T * HT) return;
@@ -32,9 +32,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   uint2 raw = make_uint2(0, 0);
   if (own) raw = *(const uint2*)(src + 4 * lane);
   const int slot = slots ? slots[t] : -1;
+  // cache element offset of this token's row: block slot / page, in-page row slot % page
+  const int64_t crow = slot >= 0 ? (int64_t)(slot / page_size) * csb + (int64_t)(slot % page_size) * csp : 0;
   if (h >= Hq + Hkv) {  // value head: plain copy into the cache
     if (own && slot >= 0 && v_cache)
-      *(uint2*)(v_cache + ((int64_t)slot * Hkv + (h - Hq - Hkv)) * D + 4 * lane) = raw;
+      *(uint2*)(v_cache + crow + (int64_t)(h - Hq - Hkv) * csh + 4 * lane) = raw;
     return;
   }
   float x[4] = {bf16lo(raw.x), bf16hi(raw.x), bf16lo(raw.y), bf16hi(raw.y)};
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   } else {
     const int kh = h - Hq;
     if (k_out) *(uint2*)(k_out + (t * Hkv + kh) * D + 4 * lane) = pk;
-    if (slot >= 0 && k_cache) *(uint2*)(k_cache + ((int64_t)slot * Hkv + kh) * D + 4 * lane) = pk;
+    if (slot >= 0 && k_cache) *(uint2*)(k_cache + crow + (int64_t)kh * csh + 4 * lane) = pk;
   }
 }
 
@@ -118,11 +120,19 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
                           const void* cos_table, const void* sin_table, const void* positions,
                           int pos_i64, const int* slot_mapping, void* q_out, void* k_out,
                           void* k_cache, void* v_cache, int64_t T, int Hq, int Hkv, int D, float eps,
-                          int64_t max_pos, hipStream_t stream) {
+                          int64_t max_pos, int page_size, int64_t cache_block_stride,
+                          int64_t cache_row_stride, int64_t cache_head_stride, hipStream_t stream) {
   if (!qkv || !q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || !q_out) return VX_ERR_ARG;
   if (T < 0 || Hq <= 0 || Hkv <= 0 || max_pos <= 0) return VX_ERR_ARG;
   if (D != 128 && D != 64) return VX_ERR_UNSUPPORTED;
   if (ld % 4 != 0) return VX_ERR_UNSUPPORTED;
+  if (k_cache || v_cache) {
+    if (page_size <= 0) return VX_ERR_ARG;
+    if (cache_block_stride % 4 != 0 || cache_row_stride % 4 != 0 || cache_head_stride % 4 != 0)
+      return VX_ERR_UNSUPPORTED;
+  } else {
+    page_size = 1;
+  }
   if (T == 0) return VX_OK;
   const int64_t waves = T * (Hq + 2 * Hkv);
   const int64_t blocks = (waves + 3) / 4;
@@ -131,7 +141,8 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
   qk_norm_rope_store_kernel<DD, PT><<<(unsigned)blocks, 256, 0, stream>>>(                     \
       (const bf16_t*)qkv, ld, (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w,                \
       (const bf16_t*)cos_table, (const bf16_t*)sin_table, (const PT*)positions, slot_mapping,  \
-      (bf16_t*)q_out, (bf16_t*)k_out, (bf16_t*)k_cache, (bf16_t*)v_cache, T, Hq, Hkv, eps, max_pos)
+      (bf16_t*)q_out, (bf16_t*)k_out, (bf16_t*)k_cache, (bf16_t*)v_cache, T, Hq, Hkv, eps, max_pos,     \
+      page_size, cache_block_stride, cache_row_stride, cache_head_stride)
   if (D == 128) { if (pos_i64) VX_QK(128, int64_t); else VX_QK(128, int); }
   else { if (pos_i64) VX_QK(64, int64_t); else VX_QK(64, int); }
 #undef VX_QK

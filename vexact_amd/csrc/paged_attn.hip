@@ -70,27 +70,25 @@ struct KVSource {
   int64_t skb, skp, svb, svp;
   int ps, shift, last;  // last = kv_len - 1; every address is clamped to an existing key
 
-  struct Tiles { int64_t k[4], v[4]; };  // element offsets of the four 16-key tiles of a block
+  struct Tiles { int pg[4], off[4]; };  // page id and first in-page row of the four 16-key tiles of a block
 
   __device__ __forceinline__ Tiles tiles(int kb) const {
     Tiles t;
 #pragma unroll
     for (int tt = 0; tt < 4; tt++) {
-      t.k[tt] = 0; t.v[tt] = 0;
+      t.pg[tt] = 0; t.off[tt] = 0;
       if constexpr (KIND == SRC_FAST) {
         const int key = kb + 16 * tt;
         const int kk = key <= last ? key : 0;  // a tile past the end is never dereferenced for real
-        const int64_t pg = bt[kk >> shift];
-        const int64_t off = kk & (ps - 1);
-        t.k[tt] = pg * skb + off * skp;
-        t.v[tt] = pg * svb + off * svp;
+        t.pg[tt] = bt[kk >> shift];
+        t.off[tt] = kk & (ps - 1);
       }
     }
     return t;
   }
   // row of key kb + 16 tt + within; `within` must already be 0 for keys past the end (FAST)
   __device__ __forceinline__ const bf16_t* krow(const Tiles& t, int kb, int tt, int within) const {
-    if constexpr (KIND == SRC_FAST) return kbase + t.k[tt] + (int64_t)within * skp;
+    if constexpr (KIND == SRC_FAST) return kbase + (int64_t)t.pg[tt] * skb + (int64_t)(t.off[tt] + within) * skp;
     const int key = min(kb + 16 * tt + within, last);
     if constexpr (KIND == SRC_PACKED) return kbase + (int64_t)key * skp;
     int pg, off;
@@ -99,7 +97,7 @@ struct KVSource {
     return kbase + (int64_t)bt[pg] * skb + (int64_t)off * skp;
   }
   __device__ __forceinline__ const bf16_t* vrow(const Tiles& t, int kb, int tt, int within) const {
-    if constexpr (KIND == SRC_FAST) return vbase + t.v[tt] + (int64_t)within * svp;
+    if constexpr (KIND == SRC_FAST) return vbase + (int64_t)t.pg[tt] * svb + (int64_t)(t.off[tt] + within) * svp;
     const int key = min(kb + 16 * tt + within, last);
     if constexpr (KIND == SRC_PACKED) return vbase + (int64_t)key * svp;
     int pg, off;
@@ -311,7 +309,7 @@ __device__ __forceinline__ KVSource<KIND> make_source(const AttnParams& p, int s
 // wavefront per block; query heads of the kv head are the MFMA columns (G <= 16 * QT).
 // ---------------------------------------------------------------------------------------
 template <int DK, int DV, int QT, int KIND>
-__global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
+__device__ __forceinline__ void attn_decode_split_body(const AttnParams& p) {
   const int kvh = blockIdx.x, seq = blockIdx.y, chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
@@ -363,6 +361,18 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
         }
       }
   }
+}
+
+// Two wavefronts per SIMD hide one wavefront's set-up and tail behind another's streaming; that
+// needs <= 256 registers, which the one-q-tile variants up to head size 128 meet without spilling.
+// The larger variants keep the full register file (one wavefront per SIMD).
+template <int DK, int DV, int QT, int KIND>
+__global__ __launch_bounds__(64) void attn_decode_split_kernel(AttnParams p) {
+  attn_decode_split_body<DK, DV, QT, KIND>(p);
+}
+template <int DK, int DV, int QT, int KIND>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_split_kernel_occ2(AttnParams p) {
+  attn_decode_split_body<DK, DV, QT, KIND>(p);
 }
 
 // grid = (Hq, B); 64 threads, lane handles dims lane, lane + 64, ...
@@ -514,8 +524,13 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
     const int G = p.Hq / p.Hkv;
     dim3 grid(p.Hkv, p.num_seqs, p.max_chunks);
     if (G <= 16) {
-      if (fast) attn_decode_split_kernel<DK, DV, 1, SRC_FAST><<<grid, 64, 0, stream>>>(p);
-      else attn_decode_split_kernel<DK, DV, 1, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
+      if constexpr (DK <= 128 && DV <= 128) {
+        if (fast) attn_decode_split_kernel_occ2<DK, DV, 1, SRC_FAST><<<grid, 64, 0, stream>>>(p);
+        else attn_decode_split_kernel_occ2<DK, DV, 1, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
+      } else {
+        if (fast) attn_decode_split_kernel<DK, DV, 1, SRC_FAST><<<grid, 64, 0, stream>>>(p);
+        else attn_decode_split_kernel<DK, DV, 1, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
+      }
     } else if (G <= 32) {
       if (fast) attn_decode_split_kernel<DK, DV, 2, SRC_FAST><<<grid, 64, 0, stream>>>(p);
       else attn_decode_split_kernel<DK, DV, 2, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);

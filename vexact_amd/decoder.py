@@ -226,9 +226,13 @@ class Qwen3MoeDecoder:
     def __init__(self, cfg: DecoderConfig, weights: DecoderWeights, num_cache_blocks: int, device="cuda"):
         self.cfg, self.w, self.device = cfg, weights, device
         self.cos, self.sin = rope_tables(cfg, device)
-        shape = (num_cache_blocks, cfg.page_size, cfg.num_kv_heads, cfg.head_dim)
-        self.key_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device) for _ in range(cfg.num_layers)]
-        self.value_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device) for _ in range(cfg.num_layers)]
+        # Physically head-major, [blocks, Hkv, page, D]: one kv head's page is 4 KB of contiguous HBM
+        # for the wavefront that reads it. The kernels see the usual [blocks, page, Hkv, D] view.
+        shape = (num_cache_blocks, cfg.num_kv_heads, cfg.page_size, cfg.head_dim)
+        self.key_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device).permute(0, 2, 1, 3)
+                          for _ in range(cfg.num_layers)]
+        self.value_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device).permute(0, 2, 1, 3)
+                            for _ in range(cfg.num_layers)]
         self.buffers: dict[tuple[int, int], StepBuffers] = {}
         self.graphs: dict[tuple[int, int, int], torch.cuda.CUDAGraph] = {}
 

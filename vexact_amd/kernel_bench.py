@@ -32,6 +32,9 @@ def main() -> None:
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--layers", type=int, default=6, help="independent weight / cache copies to rotate over")
     ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--kv-layout", default="head", choices=("head", "token"),
+                    help="physical KV cache layout: [blocks, Hkv, page, D] (what the decoder allocates) or [blocks, page, Hkv, D]")
+    ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
     ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
     a = ap.parse_args()
     dev = "cuda"
@@ -96,7 +99,7 @@ def main() -> None:
                B * k * H * 2 + 2 * B * H * 2)
         report("router top-k", timeit(lambda li: ops.router_topk(logits, k, index_dtype=torch.int32)), B * E * 4)
     if "attn" in what:
-        Hq, Hkv, D, page = 32, 4, 128, 16
+        Hq, Hkv, D, page = 32, 4, 128, a.page
         rng = np.random.default_rng(5)
         L = rng.integers(257, 2050, size=B)
         pages = [(int(n) + page - 1) // page for n in L]
@@ -108,8 +111,12 @@ def main() -> None:
         for s, p in enumerate(pages):
             bt[s, :p] = perm[o : o + p]
             o += p
-        kc = [rnd(pool, page, Hkv, D, std=1.0) for _ in range(NL)]
-        vc = [rnd(pool, page, Hkv, D, std=1.0) for _ in range(NL)]
+        if a.kv_layout == "head":
+            kc = [rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3) for _ in range(NL)]
+            vc = [rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3) for _ in range(NL)]
+        else:
+            kc = [rnd(pool, page, Hkv, D, std=1.0) for _ in range(NL)]
+            vc = [rnd(pool, page, Hkv, D, std=1.0) for _ in range(NL)]
         q = rnd(B, Hq, D, std=1.0)
         cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
         used = torch.tensor(L, dtype=torch.int32, device=dev)
@@ -138,6 +145,10 @@ def main() -> None:
                    flops=2 * M * N * K)
             del w_, xx, c
     if "small" in what:
+        one = torch.zeros(64, dtype=torch.int32, device=dev)
+        lib = _lib.load()
+        report("one-element fill (node floor)",
+               timeit(lambda li: _lib.check(lib.vx_fill_i32(one.data_ptr(), 1, 1, torch.cuda.current_stream().cuda_stream), "fill")), 4)
         x = rnd(B, H, std=1.0)
         res = rnd(B, H, std=1.0)
         wn = rnd(H, std=1.0)

@@ -609,15 +609,22 @@ def fused_moe(
 
 def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, cos_table, sin_table, positions, slot_mapping, q_out,
                        k_cache, v_cache, Hq: int, Hkv: int, D: int, eps: float, k_out=None) -> None:
+    """Caches are ``[blocks, page, Hkv, D]`` views (any block / row / head strides, D contiguous)."""
     T = qkv.shape[0]
     assert qkv.stride(1) == 1 and qkv.shape[1] == (Hq + 2 * Hkv) * D
     assert positions.dtype in (torch.int32, torch.int64)
+    page, sb, sp, sh = 1, 0, 0, 0
+    if k_cache is not None:
+        assert k_cache.dim() == 4 and k_cache.shape[2] == Hkv and k_cache.shape[3] == D and k_cache.stride(3) == 1
+        page, (sb, sp, sh) = k_cache.shape[1], k_cache.stride()[:3]
+        if v_cache is not None:
+            assert v_cache.shape == k_cache.shape and v_cache.stride() == k_cache.stride()
     _lib.check(
         _lib.load().vx_qk_norm_rope_store(
             qkv.data_ptr(), qkv.stride(0), q_norm_w.data_ptr(), k_norm_w.data_ptr(), cos_table.data_ptr(),
             sin_table.data_ptr(), positions.data_ptr(), int(positions.dtype == torch.int64), _ptr(slot_mapping),
             q_out.data_ptr(), _ptr(k_out), _ptr(k_cache), _ptr(v_cache), T, Hq, Hkv, D, float(eps),
-            cos_table.shape[0], _stream(),
+            cos_table.shape[0], page, sb, sp, sh, _stream(),
         ),
         "vx_qk_norm_rope_store",
     )
