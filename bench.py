@@ -258,7 +258,7 @@ def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
     torch.set_num_threads(cores)
     lw = {k_: v.cpu() for k_, v in w.layers[0].items()}
-    kc, vc = dec.key_cache[0].cpu(), dec.value_cache[0].cpu()
+    kc, vc = dec.key_cache[0].cpu().contiguous(), dec.value_cache[0].cpu().contiguous()
     cos, sin = rope_tables(cfg, "cpu")
     x = w.embed[torch.as_tensor(first_tokens).to(w.embed.device)].cpu()
     pos = torch.as_tensor(dmeta["positions"]).long()
