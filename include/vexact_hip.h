@@ -77,7 +77,8 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
 /* Same, forcing the kernel: kind 0 = weight-streaming with 16*mt-row tiles (mt in 1,2,4),
  * kind 1 = 128x128 LDS-tiled, kind 2 = weight-streaming with 16 k-steps in flight, kind 3 = 256x256
  * persistent tiles with direct-to-LDS loads (needs K % 64 == 0 and operands below 4 GiB, else
- * VX_ERR_UNSUPPORTED). Results are bit-identical across kinds (tested). */
+ * VX_ERR_UNSUPPORTED), kind 4 = LDS ring kernel for 65..512 rows, mt = configuration 0..6 (K % 64,
+ * 128 or 256 == 0 depending on the configuration). Results are bit-identical across kinds (tested). */
 int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void* c, int64_t M,
                             int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind,
                             int mt, hipStream_t stream);

@@ -66,6 +66,23 @@ def test_wide_kernel_agrees_bitwise(M, N, K, bias):
         assert_bitwise(ops.gemm_nt(ag[1000:1003], wg, bias=bg), full[1000:1003], "3 rows alone vs inside a chunk")
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 640, 2048), (100, 200, 64), (77, 333, 192), (130, 70, 320), (512, 128, 768)])
+def test_ring_kernel_agrees_bitwise(M, N, K):
+    a = _gen((M, K), 16)
+    w = _gen((N, K), 17, scale=0.05)
+    bias = _gen((N,), 18)
+    ag, wg, bg = a.cuda(), w.cuda(), bias.cuda()
+    ref = ops.gemm_nt_variant(ag, wg, kind=1, bias=bg)
+    ran = 0
+    for cfg, kdiv in ((0, 64), (1, 128), (2, 128), (3, 128), (4, 256), (5, 64), (6, 64)):
+        if K % kdiv:
+            continue
+        assert_bitwise(ops.gemm_nt_variant(ag, wg, kind=4, mt=cfg, bias=bg), ref, f"ring config {cfg} vs tiled")
+        ran += 1
+    assert ran >= 3
+    assert_bitwise(ops.gemm_nt(ag, wg, bias=bg), ref, "dispatch vs tiled")
+
+
 def test_lm_head_shape_rows():
     # config-1 shaped: [M, 2048] x [2048, 151936], rows of one draw
     a = _gen((64, 2048), 6)

@@ -87,6 +87,8 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
     if (nt * ((M + 63) / 64) >= 256) mt = 4;
     else if (nt * ((M + 31) / 32) >= 256) mt = 2;
   }
+  // 65 .. 512 rows: the LDS ring kernel, whose loads do not wait on one wavefront's MFMA chain
+  if (mt != 0 && M > 64 && gemm_ring_auto(p, stream)) return launch_status();
   if (mt != 0) {
     const dim3 grid((unsigned)nt, (unsigned)((M + 16 * mt - 1) / (16 * mt)));
     if (mt == 1) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
@@ -106,7 +108,8 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
 
 // Forces one kernel regardless of M (kind 0 = streaming with 16*mt rows per tile, mt in {1,2,4};
 // kind 1 = 128x128 tiled; kind 2 = streaming, 16 k-steps in flight; kind 3 = 256x256 wide tiles,
-// needs K % 64 == 0). For tests that check that all kernels give the same bits.
+// needs K % 64 == 0; kind 4 = LDS ring kernel, mt = configuration 0..6). For tests that check
+// that all kernels give the same bits.
 int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void* c, int64_t M,
                             int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind,
                             int mt, hipStream_t stream) {
@@ -144,6 +147,8 @@ int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void
     gemm_tiled_kernel<EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
   } else if (kind == 3) {  // wide 256x256 tiles
     if (!gemm_wide_launch(p, stream)) return VX_ERR_UNSUPPORTED;
+  } else if (kind == 4) {  // LDS ring, mt = tile shape code
+    if (!gemm_ring_launch(p, mt, stream)) return VX_ERR_UNSUPPORTED;
   } else {
     return VX_ERR_ARG;
   }

@@ -243,4 +243,197 @@ static inline bool gemm_wide_launch(const GemmParams& p, hipStream_t stream) {
   return true;
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Ring kernel for a few hundred rows (decode-sized batches against dense weights), where one
+// wavefront's chain of dependent HBM round trips, not bandwidth, bounds the streaming kernel.
+// 4 wavefronts (2 x 2) compute a (32 XF) x (32 WF) tile; both operands go directly to LDS
+// (same swizzled 128-byte rows as the wide kernel) into a ring of S stages of 64 k-elements, so
+// S - 1 steps of loads are in flight per workgroup whatever the compute does. One barrier per step;
+// the loads of step s + S - 1 refill the stage that was read in step s - 1. Past the last step the
+// ring keeps loading (valid addresses, unread stages) so that the outstanding-load count the
+// waits rely on stays constant.
+// ---------------------------------------------------------------------------------------
+template <int XF, int WF, int S, int KSUB>
+__global__ __launch_bounds__(256) void gemm_ring_kernel(GemmParams p) {
+  constexpr int BM = 32 * XF, BN = 32 * WF, BK = 64 * KSUB;
+  constexpr int XB = BM * 128, SUB = (BM + BN) * 128, STAGE = KSUB * SUB;
+  constexpr int NSUB = (BM + BN) / 8;  // wavefront-wide load instructions per 64-wide sub-tile
+  constexpr int NLD = KSUB * NSUB;     // per step
+  constexpr int LPW = NLD / 4;         // per wavefront
+  static_assert(NLD % 4 == 0, "loads must split evenly over the 4 wavefronts");
+  static_assert((S - 2) * LPW <= 63, "vmcnt field");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t rg_lds[];
+
+  const int M = p.M, N = p.N, K = p.K;
+  const int row0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, g = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // load instruction q = wave + 4 t: sub-tile q / NSUB, rows [8 (q % NSUB), +8) of X (first BM / 8) or W
+  const int lrow = lane >> 3, lslot = lane & 7;
+  uint32_t ld_off[LPW];
+#pragma unroll
+  for (int t = 0; t < LPW; t++) {
+    const int q = (wave + 4 * t) % NSUB;
+    if (q < BM / 8) {
+      const int R = 8 * q + lrow;
+      ld_off[t] = (uint32_t)(((int64_t)min(row0 + R, M - 1) * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
+    } else {
+      const int R = 8 * (q - BM / 8) + lrow;
+      const int sw = (((R / (4 * WF)) & 3) << 1) | ((R >> 1) & 1);
+      ld_off[t] = (uint32_t)(((int64_t)min(n0 + R, N - 1) * p.ldw + (lslot ^ sw) * 8) * 2);
+    }
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)rg_lds;
+  const int nk = K / BK;  // K % BK == 0 (host check)
+  auto issue = [&](int step) {  // loads of `step` (wrapped past the end) into stage step % S
+    const int st = step < nk ? step : step % nk;
+    const uint32_t sb = lds0 + (step % S) * STAGE;
+#pragma unroll
+    for (int t = 0; t < LPW; t++) {
+      const int qq = wave + 4 * t;  // wave-uniform
+      const int u = qq / NSUB, q = qq % NSUB;
+      const bool isx = q < BM / 8;
+      const uint32_t dst = sb + u * SUB + (isx ? q * 1024 : XB + (q - BM / 8) * 1024);
+      const bf16_t* base = (isx ? p.x : p.w) + (st * KSUB + u) * 64;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :: "s"(dst), "v"(ld_off[t]), "s"(base) : "memory", "m0");
+    }
+  };
+
+  f32x4 acc[XF][WF];
+#pragma unroll
+  for (int i = 0; i < XF; i++)
+#pragma unroll
+    for (int j = 0; j < WF; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // fragment addresses (k-half 0; k-half 1 flips bit 6). Weight fragment j, MFMA row rho is weight
+  // row 4 WF (rho / 4) + 4 j + rho % 4 of the wavefront's 16 WF: a lane's outputs are contiguous in n.
+  const int xoff = (16 * XF * wm + r16) * 128 + ((g ^ (r16 >> 1)) * 16);
+  const int woff = XB + (16 * WF * wn + 4 * WF * (r16 >> 2) + (r16 & 3)) * 128 +
+                   ((g ^ (((r16 >> 2) << 1) | ((r16 >> 1) & 1))) * 16);
+
+#pragma unroll
+  for (int t = 0; t < S - 1; t++) issue(t);
+  for (int s = 0; s < nk; s++) {
+    // in-order completion: at most the S - 2 youngest steps may still be in flight
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"((S - 2) * LPW) : "memory");
+    __syncthreads();  // step s is in LDS for everyone; everyone is done reading step s - 1
+    issue(s + S - 1);
+    const uint8_t* sb = rg_lds + (s % S) * STAGE;
+    // all fragment reads of the step first, then its MFMAs: one LDS round trip per step
+    uint4 wf[2 * KSUB][WF], xf[2 * KSUB][XF];
+#pragma unroll
+    for (int kk = 0; kk < 2 * KSUB; kk++) {
+      const uint8_t* sk = sb + (kk >> 1) * SUB;
+#pragma unroll
+      for (int j = 0; j < WF; j++) wf[kk][j] = *(const uint4*)(sk + (woff ^ (64 * (kk & 1))) + j * 512);
+#pragma unroll
+      for (int i = 0; i < XF; i++) xf[kk][i] = *(const uint4*)(sk + (xoff ^ (64 * (kk & 1))) + i * 2048);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 2 * KSUB; kk++)
+#pragma unroll
+      for (int i = 0; i < XF; i++)
+#pragma unroll
+        for (int j = 0; j < WF; j++) acc[i][j] = mfma16(wf[kk][j], xf[kk][i], acc[i][j]);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the ring's trailing loads still target our LDS
+
+  // epilogue: lane holds C[row0 + 16 XF wm + 16 i + r16][n0 + 16 WF wn + 4 WF g + 4 j + c]
+  const int nb = n0 + 16 * WF * wn + 4 * WF * g;
+  const bool vec_ok = (p.ldc & 7) == 0 && ((uintptr_t)p.c & 15) == 0;
+#pragma unroll
+  for (int i = 0; i < XF; i++) {
+    const int m = row0 + 16 * XF * wm + 16 * i + r16;
+    if (m >= M) continue;
+    bf16_t o[4 * WF];
+#pragma unroll
+    for (int j = 0; j < WF; j++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        float v = acc[i][j][c];
+        if (p.bias) v += bf16_to_f32(p.bias[min(nb + 4 * j + c, N - 1)]);
+        o[4 * j + c] = f32_to_bf16(v);
+      }
+    bf16_t* cp = p.c + (int64_t)m * p.ldc + nb;
+    if (vec_ok && WF % 2 == 0 && nb + 4 * WF - 1 < N) {
+#pragma unroll
+      for (int h = 0; h < WF / 2; h++) {
+        uint4 pk;
+        pk.x = (uint32_t)o[8 * h + 0] | ((uint32_t)o[8 * h + 1] << 16);
+        pk.y = (uint32_t)o[8 * h + 2] | ((uint32_t)o[8 * h + 3] << 16);
+        pk.z = (uint32_t)o[8 * h + 4] | ((uint32_t)o[8 * h + 5] << 16);
+        pk.w = (uint32_t)o[8 * h + 6] | ((uint32_t)o[8 * h + 7] << 16);
+        *(uint4*)(cp + 8 * h) = pk;
+      }
+    } else if (WF == 1 && (p.ldc & 3) == 0 && ((uintptr_t)p.c & 7) == 0 && nb + 3 < N) {
+      uint2 pk;
+      pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+      pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+      *(uint2*)cp = pk;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4 * WF; e++)
+        if (nb + e < N) cp[e] = o[e];
+    }
+  }
+}
+
+template <int XF, int WF, int S, int KSUB>
+static inline bool gemm_ring_launch_t(const GemmParams& p, hipStream_t stream) {
+  constexpr int BM = 32 * XF, BN = 32 * WF, LDS = S * KSUB * (BM + BN) * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)gemm_ring_kernel<XF, WF, S, KSUB>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    attr_set = true;
+  }
+  const int64_t gy = ((int64_t)p.M + BM - 1) / BM, gx = ((int64_t)p.N + BN - 1) / BN;
+  if (gy > 65535 || gx > 0x7fffffffLL || p.K % (64 * KSUB) != 0) return false;
+  gemm_ring_kernel<XF, WF, S, KSUB><<<dim3((unsigned)gx, (unsigned)gy), 256, LDS, stream>>>(p);
+  return true;
+}
+// Ring configurations (rows x weight rows per workgroup, stages, 64-wide k sub-tiles per stage):
+//   0: 64x64 S3 K1   1: 64x64 S2 K2   2: 64x64 S3 K2   3: 32x64 S3 K2   4: 32x32 S3 K4
+//   5: 32x64 S4 K1   6: 32x32 S4 K1
+static inline bool gemm_ring_launch(const GemmParams& p, int shape, hipStream_t stream) {
+  if (p.K % 64 != 0 || p.M <= 0 || p.N <= 0) return false;
+  const int64_t lim = (int64_t)1 << 32;
+  if (((int64_t)p.M * p.ldx + p.K) * 2 >= lim || ((int64_t)p.N * p.ldw + p.K) * 2 >= lim) return false;
+  switch (shape) {
+    case 0: return gemm_ring_launch_t<2, 2, 3, 1>(p, stream);
+    case 1: return gemm_ring_launch_t<2, 2, 2, 2>(p, stream);
+    case 2: return gemm_ring_launch_t<2, 2, 3, 2>(p, stream);
+    case 3: return gemm_ring_launch_t<1, 2, 3, 2>(p, stream);
+    case 4: return gemm_ring_launch_t<1, 1, 3, 4>(p, stream);
+    case 5: return gemm_ring_launch_t<1, 2, 4, 1>(p, stream);
+    case 6: return gemm_ring_launch_t<1, 1, 4, 1>(p, stream);
+    default: return false;
+  }
+}
+
+// Picks the ring configuration for a decode-sized batch (measured on M = 128 .. 512 against the
+// qkv / o / router projections of the 30B-A3B shape): enough workgroups to occupy every CU first,
+// then the largest tile (least L2 -> LDS traffic), then fewer, longer steps when K allows.
+static inline bool gemm_ring_auto(const GemmParams& p, hipStream_t stream) {
+  const int64_t m64 = (p.M + 63) / 64, m32 = (p.M + 31) / 32;
+  const int64_t n64 = (p.N + 63) / 64, n32 = (p.N + 31) / 32;
+  const bool k2 = p.K % 128 == 0, k4 = p.K % 256 == 0;
+  int shape;
+  if (m64 * n64 >= 512) shape = 0;
+  else if (m64 * n64 >= 300) shape = k2 ? 1 : 0;
+  else if (m64 * n64 >= 200) shape = k2 ? 2 : 0;
+  else if (m32 * n64 >= 200) shape = k2 ? 3 : 5;
+  else shape = k4 ? 4 : 6;
+  (void)n32;
+  return gemm_ring_launch(p, shape, stream);
+}
+
 }  // namespace vx
