@@ -105,7 +105,10 @@ int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_
 /* Causal GQA attention, bf16, head dims (Dk, Dv) in {(32,32),(64,64),(128,128),(192,128),(256,256)}.
  *   mode 0: paged decode - every sequence has at most one query token; KV is split into fixed
  *           256-key chunks (absolute positions) and folded in ascending order; needs
- *           vx_paged_attn_decode_workspace_bytes(num_seqs, Hq, Dv, max_pages * page_size) bytes
+ *           vx_paged_attn_decode_workspace_bytes(num_seqs, Hq, Hkv, Dv, max_pages * page_size) bytes
+ *           (modes 3 and 4 are mode 0 with the kernel forced: 3 = one wavefront per chunk plus a
+ *           combine launch, 4 = chunks folded inside one workgroup per (sequence, kv head); mode 0
+ *           takes 4 when num_seqs * Hkv fills the machine. The results are bit-identical.)
  *   mode 1: paged general (chunked prefill, mixed batches) - same arithmetic per row as mode 0
  *   mode 2: packed K/V [Tk, Hkv, D] with cu_seqlens_k (skp = row stride, no block table)
  * q [total_q, Hq, Dk], k/v cache [blocks, page, Hkv, D], out [total_q, Hq, Dv];
@@ -113,7 +116,7 @@ int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_
  * Replaces _paged_attn_fwd_block_kernel / _PagedFlashAttentionVarlen.forward and the forward of
  * _varlen_attn_fwd_block_kernel, vexact/batch_invariant_ops/triton_invariant_attention.py:433-692, 47-190. */
 int vx_attn_chunk_size(void);
-int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Dv,
+int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Hkv, int64_t Dv,
                                              int64_t max_kv_len);
 int vx_attention(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens_q,
                  const int* seqused_k, const int* cu_seqlens_k, const int* block_table,

@@ -19,7 +19,7 @@ def test_library_is_built_and_loads():
     if not os.path.exists(_build.LIB_PATH):
         _build.build()
     lib = _lib.load()
-    assert lib.vx_abi_version() == 1
+    assert lib.vx_abi_version() == 2
     assert lib.vx_status_string(0) == b"ok"
     assert b"workspace" in lib.vx_status_string(-3)
 
@@ -37,8 +37,10 @@ def test_host_only_helpers():
     lib = _lib.load()
     assert lib.vx_attn_chunk_size() == 256
     # partial states: (Dv + 2) floats per (sequence, head, 256-key chunk)
-    assert lib.vx_paged_attn_decode_workspace_bytes(64, 16, 128, 4096) == 64 * 16 * 16 * 130 * 4
-    assert lib.vx_paged_attn_decode_workspace_bytes(1, 1, 128, 1) == 130 * 4
+    # one 9-slot (8 accumulator + 1 max/sum) x 64-lane x 16-byte image per (sequence, kv head, chunk)
+    assert lib.vx_paged_attn_decode_workspace_bytes(64, 16, 4, 128, 4096) == 64 * 4 * 16 * 9 * 1024
+    assert lib.vx_paged_attn_decode_workspace_bytes(1, 1, 1, 128, 1) == 9 * 1024
+    assert lib.vx_paged_attn_decode_workspace_bytes(2, 64, 2, 256, 257) == 2 * 2 * 2 * (2 * 2 * 8 + 2) * 1024
     # 16 bytes per (row, 4096-column chunk)
     assert lib.vx_log_softmax_workspace_bytes(7, 151936) == 7 * 38 * 16
     assert lib.vx_moe_max_tiles(2048, 128, 32) == 128 + 64

@@ -245,3 +245,35 @@ def test_packed_non_causal_matches_eager():
                                     max_seqlen_q=9, max_seqlen_k=12, causal=False)
     ref = torch.cat([OA.eager_attention(a, b, c, 64**-0.5, causal=False) for a, b, c in zip(q, k, v)])
     torch.testing.assert_close(out.cpu(), ref, atol=3e-3, rtol=3e-3)
+
+
+@pytest.mark.parametrize(
+    ("qh", "kh", "dk", "dv", "page", "head_major"),
+    [(32, 4, 128, 128, 16, True), (8, 8, 64, 64, 16, False), (48, 2, 128, 128, 32, False), (16, 1, 192, 128, 16, False),
+     (4, 2, 32, 32, 24, False)],
+)
+def test_decode_forms_agree_bitwise(qh, kh, dk, dv, page, head_major):
+    """One wavefront per chunk + combine launch vs chunks folded inside the workgroup: same bits, for
+    lengths around the 256-key chunk edges, 1..9 chunks, GQA groups of 1 / 8 / 16 / 24 heads, a page
+    size that is not a power of two, and the head-major physical cache layout."""
+    from vexact_amd import ops
+
+    kv_lens = [1, 63, 64, 255, 256, 257, 511, 513, 1024, 1025, 1300, 2047, 2048, 2049, 700, 40]
+    g = torch.Generator().manual_seed(11)
+    k = [(torch.randn(n, kh, dk, generator=g) * 0.3).to(torch.bfloat16) for n in kv_lens]
+    v = [(torch.randn(n, kh, dv, generator=g) * 0.3).to(torch.bfloat16) for n in kv_lens]
+    q = (torch.randn(len(kv_lens), qh, dk, generator=g) * 0.3).to(torch.bfloat16).cuda()
+    perm = torch.randperm(sum((n + page - 1) // page for n in kv_lens), generator=g)
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, page, perm=perm)
+    kc, vc = k_cache.cuda(), v_cache.cuda()
+    if head_major:
+        kc = kc.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        vc = vc.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    cu = torch.arange(len(kv_lens) + 1, dtype=torch.int32).cuda()
+    used = torch.tensor(kv_lens, dtype=torch.int32).cuda()
+    outs = {kind: ops.paged_attention(q, kc, vc, cu, used, table.cuda(), dk**-0.5, 1, decode_kernel=kind)
+            for kind in ("split", "fused", "auto")}
+    assert_bitwise(outs["fused"], outs["split"], "fused vs split decode")
+    assert_bitwise(outs["auto"], outs["split"], "auto vs split decode")
+    ref = torch.stack([OA.eager_attention(q[i : i + 1].cpu(), k[i], v[i], dk**-0.5)[0] for i in range(len(kv_lens))])
+    torch.testing.assert_close(outs["fused"].cpu(), ref, atol=3e-3, rtol=3e-3)

@@ -184,6 +184,6 @@ const char* vx_status_string(int code) {
   }
 }
 
-int vx_abi_version() { return 1; }
+int vx_abi_version() { return 2; }
 
 }  // extern "C"

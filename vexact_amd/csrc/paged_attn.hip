@@ -49,9 +49,9 @@ struct AttnParams {
   int Hq, Hkv, num_seqs;
   float qk_scale;  // scale * log2(e)
   int causal;
-  // decode split workspace
-  float* part_acc;  // [B, Hq, max_chunks, DV]
-  float* part_ml;   // [B, Hq, max_chunks, 2]
+  // decode split workspace: one register image per (sequence, kv head, chunk), see part_image_floats
+  float* part;
+  int64_t img_floats;
   int max_chunks;
 };
 
@@ -335,31 +335,27 @@ __device__ __forceinline__ void attn_decode_split_body(const AttnParams& p) {
   const KVSource<KIND> src = make_source<KIND>(p, seq, kvh, 0, kv_len);
   w.run_chunk(src, kstart, min(kstart + ATT_CHUNK, kv_len), kv_len, p.qk_scale);
 
-  // write the chunk state: lane holds dims 128 ds + 32 g + 8 r + td for head column r16
+  // Write the chunk state as the wavefront holds it: float4 slot i of lane l lands at
+  // image[(i * 64 + l) * 4], so every store instruction writes whole 128-byte lines (a layout by
+  // head and dim would scatter 16-byte pieces). Slot ((t NDV + ds) 4 + r) 2 + h holds dims
+  // 128 ds + 32 g + 8 r + 4 h .. +4 of head 16 t + r16; slot NI + t holds (m, l) of that head.
+  constexpr int NDV = (DV + 127) / 128, NI = QT * NDV * 8;
+  float4* ip = (float4*)(p.part + ((int64_t)(seq * p.Hkv + kvh) * p.max_chunks + chunk) * p.img_floats) + lane;
 #pragma unroll
   for (int t = 0; t < QT; t++) {
-    const int hl = 16 * t + r16;
-    if (hl >= G) continue;
-    const int64_t slot = ((int64_t)seq * p.Hq + kvh * G + hl) * p.max_chunks + chunk;
-    if (g == 0) {
-      p.part_ml[slot * 2] = w.m[t];
-      p.part_ml[slot * 2 + 1] = w.l[t];
-    }
-    float* pa = p.part_acc + slot * DV;
+    if (16 * t + r16 >= G) continue;
 #pragma unroll
-    for (int ds = 0; ds < (DV + 127) / 128; ds++)
+    for (int ds = 0; ds < NDV; ds++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const int d0 = 128 * ds + 32 * g + 8 * r;
-        if (d0 < DV) {
-          float4 a = make_float4(w.acc[t][ds * 8 + 0][r], w.acc[t][ds * 8 + 1][r],
-                                 w.acc[t][ds * 8 + 2][r], w.acc[t][ds * 8 + 3][r]);
-          float4 b = make_float4(w.acc[t][ds * 8 + 4][r], w.acc[t][ds * 8 + 5][r],
-                                 w.acc[t][ds * 8 + 6][r], w.acc[t][ds * 8 + 7][r]);
-          *(float4*)(pa + d0) = a;
-          *(float4*)(pa + d0 + 4) = b;
-        }
+        if (128 * ds + 32 * g + 8 * r >= DV) continue;
+        const int sl = ((t * NDV + ds) * 4 + r) * 2;
+        ip[sl * 64] = make_float4(w.acc[t][ds * 8 + 0][r], w.acc[t][ds * 8 + 1][r], w.acc[t][ds * 8 + 2][r],
+                                  w.acc[t][ds * 8 + 3][r]);
+        ip[(sl + 1) * 64] = make_float4(w.acc[t][ds * 8 + 4][r], w.acc[t][ds * 8 + 5][r],
+                                        w.acc[t][ds * 8 + 6][r], w.acc[t][ds * 8 + 7][r]);
       }
+    ip[(NI + t) * 64] = make_float4(w.m[t], w.l[t], 0.f, 0.f);
   }
 }
 
@@ -375,38 +371,186 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) void at
   attn_decode_split_body<DK, DV, QT, KIND>(p);
 }
 
-// grid = (Hq, B); 64 threads, lane handles dims lane, lane + 64, ...
-template <int DV>
+// ---------------------------------------------------------------------------------------
+// Decode, chunks folded inside the workgroup: grid = (Hkv, B), NW wavefronts per block. Wavefront v
+// takes chunks v, v + NW, ... of its (sequence, kv head); after each round the NW chunk states go to
+// LDS (same register image as the split kernel writes to HBM) and are folded, in ascending chunk
+// order, into a running state that lives in LDS, one owner thread per (head, 4 dims). Same fold
+// arithmetic as attn_decode_combine_kernel, so both decode paths give the same bits; this one has
+// no HBM round trip for the chunk states and no second launch, but needs B * Hkv * NW wavefronts to
+// fill the machine.
+// ---------------------------------------------------------------------------------------
+template <int DK, int DV, int QT, int KIND, int NW>
+__device__ __forceinline__ void attn_decode_fused_body(const AttnParams& p) {
+  constexpr int NDV = (DV + 127) / 128, NI = QT * NDV * 8;
+  constexpr int IMG4 = (NI + QT) * 64;   // float4 per chunk image
+  constexpr int MAXE = 16 * QT * (DV / 4);  // owner elements: (head, 4 dims)
+  extern __shared__ __attribute__((aligned(16))) uint8_t fz_lds[];
+  float4* img = (float4*)fz_lds;                    // [NW][IMG4]
+  float4* racc = img + NW * IMG4;                   // [MAXE] running accumulators
+  float2* rml = (float2*)(racc + MAXE);             // [MAXE] running (M, L), one private copy per element
+
+  const int kvh = blockIdx.x, seq = blockIdx.y;
+  const int q0 = p.cu_q[seq];
+  const int qlen = p.cu_q[seq + 1] - q0;
+  const int kv_len = p.seqused_k[seq];
+  if (qlen <= 0 || kv_len <= 0) return;  // uniform over the block
+  const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+  const int wave = tid >> 6;
+  const int G = p.Hq / p.Hkv;
+  const int64_t tok = q0 + qlen - 1;
+  const int pos = kv_len - 1;
+  const int nch = (kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
+  const int nelem = G * (DV / 4);
+
+  for (int e = tid; e < nelem; e += 64 * NW) {
+    racc[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    rml[e] = make_float2(-INFINITY, 0.f);
+  }
+
+  AttnWave<DK, DV, QT> w;
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int hl = 16 * t + r16;
+    const bool ok = hl < G;
+    w.qpos[t] = ok ? pos : -1;
+    const bf16_t* qp = p.q + tok * p.sqt + (int64_t)(kvh * G + (ok ? hl : 0)) * p.sqh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DK / 32; s++) w.qf[t][s] = ldg16(qp + 32 * s, ok);
+  }
+  const KVSource<KIND> src = make_source<KIND>(p, seq, kvh, 0, kv_len);
+
+  for (int c0 = 0; c0 < nch; c0 += NW) {
+    const int c = c0 + wave;
+    if (c < nch) w.run_chunk(src, c * ATT_CHUNK, min(c * ATT_CHUNK + ATT_CHUNK, kv_len), kv_len, p.qk_scale);
+    __syncthreads();  // the previous round's fold has finished reading the images
+    if (c < nch) {
+      float4* ip = img + wave * IMG4 + lane;
+#pragma unroll
+      for (int t = 0; t < QT; t++) {
+        if (16 * t + r16 >= G) continue;
+#pragma unroll
+        for (int ds = 0; ds < NDV; ds++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            if (128 * ds + 32 * g + 8 * r >= DV) continue;
+            const int sl = ((t * NDV + ds) * 4 + r) * 2;
+            ip[sl * 64] = make_float4(w.acc[t][ds * 8 + 0][r], w.acc[t][ds * 8 + 1][r],
+                                      w.acc[t][ds * 8 + 2][r], w.acc[t][ds * 8 + 3][r]);
+            ip[(sl + 1) * 64] = make_float4(w.acc[t][ds * 8 + 4][r], w.acc[t][ds * 8 + 5][r],
+                                            w.acc[t][ds * 8 + 6][r], w.acc[t][ds * 8 + 7][r]);
+          }
+        ip[(NI + t) * 64] = make_float4(w.m[t], w.l[t], 0.f, 0.f);
+      }
+    }
+    __syncthreads();
+    const int nr = min(NW, nch - c0);  // chunk states of this round
+    for (int e = tid; e < nelem; e += 64 * NW) {
+      const int hl = e / (DV / 4), d = 4 * (e % (DV / 4));
+      const int t = hl >> 4, hr = hl & 15;
+      const int sl = ((t * NDV + d / 128) * 4 + (d % 32) / 8) * 2 + (d % 8) / 4;
+      const int ln = 16 * ((d % 128) / 32) + hr;
+      float4 A4 = racc[e];
+      float M = rml[e].x, L = rml[e].y;
+      for (int j = 0; j < nr; j++) {
+        const float4 ml = img[j * IMG4 + (NI + t) * 64 + hr];
+        const float4 a = img[j * IMG4 + sl * 64 + ln];
+        float Mn, A, B;
+        fold_scales(M, ml.x, Mn, A, B);
+        L = L * A + ml.y * B;
+        A4.x = A4.x * A + a.x * B;
+        A4.y = A4.y * A + a.y * B;
+        A4.z = A4.z * A + a.z * B;
+        A4.w = A4.w * A + a.w * B;
+        M = Mn;
+      }
+      racc[e] = A4;
+      rml[e] = make_float2(M, L);
+    }
+  }
+  // every thread reads back only what it wrote itself
+  for (int e = tid; e < nelem; e += 64 * NW) {
+    const int hl = e / (DV / 4), d = 4 * (e % (DV / 4));
+    const float4 a = racc[e];
+    const float L = rml[e].y;
+    uint2 pk;
+    pk.x = pack_bf16x2(a.x / L, a.y / L);
+    pk.y = pack_bf16x2(a.z / L, a.w / L);
+    *(uint2*)(p.o + tok * p.sot + (int64_t)(kvh * G + hl) * p.soh + d) = pk;
+  }
+}
+
+template <int DK, int DV, int QT, int KIND, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_decode_fused_kernel(AttnParams p) {
+  attn_decode_fused_body<DK, DV, QT, KIND, NW>(p);
+}
+template <int DK, int DV, int QT, int KIND, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) void attn_decode_fused_kernel_occ2(AttnParams p) {
+  attn_decode_fused_body<DK, DV, QT, KIND, NW>(p);
+}
+
+template <int DV, int QT, int NW>
+constexpr int fused_lds_bytes() {
+  return (NW * (QT * ((DV + 127) / 128) * 8 + QT) * 64 + 16 * QT * (DV / 4)) * 16 + 16 * QT * (DV / 4) * 8;
+}
+
+// Folds the chunk images of one (sequence, kv head) in ascending chunk order. grid = (Hkv, B),
+// one wavefront with the lane layout of the split kernel: lane (r16, g) owns head 16 t + r16, dims
+// 128 ds + 32 g + 8 r + (0..7), reads its own slots of every image and writes 16 bytes per (ds, r).
+template <int DV, int QT>
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
-  const int head = blockIdx.x, seq = blockIdx.y;
+  const int kvh = blockIdx.x, seq = blockIdx.y;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
   if (qlen <= 0 || kv_len <= 0) return;
   const int nch = (kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
-  const int64_t slot0 = ((int64_t)seq * p.Hq + head) * p.max_chunks;
-  constexpr int PER = (DV + 63) / 64;
-  float M = -INFINITY, L = 0.f, ACC[PER];
-#pragma unroll
-  for (int i = 0; i < PER; i++) ACC[i] = 0.f;
-  for (int c = 0; c < nch; c++) {
-    const float mc = p.part_ml[(slot0 + c) * 2], lc = p.part_ml[(slot0 + c) * 2 + 1];
-    float Mn, A, B;
-    fold_scales(M, mc, Mn, A, B);
-    L = L * A + lc * B;
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-      const int d = threadIdx.x + 64 * i;
-      const float a = (d < DV) ? p.part_acc[(slot0 + c) * DV + d] : 0.f;
-      ACC[i] = ACC[i] * A + a * B;
-    }
-    M = Mn;
-  }
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int G = p.Hq / p.Hkv;
+  constexpr int NDV = (DV + 127) / 128, NI = QT * NDV * 8;
+  const float4* ip0 = (const float4*)(p.part + (int64_t)(seq * p.Hkv + kvh) * p.max_chunks * p.img_floats) + lane;
   const int64_t tok = q0 + qlen - 1;
 #pragma unroll
-  for (int i = 0; i < PER; i++) {
-    const int d = threadIdx.x + 64 * i;
-    if (d < DV) p.o[tok * p.sot + (int64_t)head * p.soh + d] = f32_to_bf16(ACC[i] / L);
+  for (int t = 0; t < QT; t++) {
+    const int hl = 16 * t + r16;
+    if (hl >= G) continue;
+    float M = -INFINITY, L = 0.f;
+    float4 ACC[NDV * 8];
+#pragma unroll
+    for (int i = 0; i < NDV * 8; i++) ACC[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int c = 0; c < nch; c++) {
+      const float4* ip = ip0 + (int64_t)c * (p.img_floats / 4);
+      const float4 ml = ip[(NI + t) * 64];
+      float Mn, A, B;
+      fold_scales(M, ml.x, Mn, A, B);
+      L = L * A + ml.y * B;
+#pragma unroll
+      for (int i = 0; i < NDV * 8; i++) {
+        const int ds = i >> 3, r = (i >> 1) & 3;
+        if (128 * ds + 32 * g + 8 * r >= DV) continue;
+        const float4 a = ip[(t * NDV * 8 + i) * 64];
+        ACC[i].x = ACC[i].x * A + a.x * B;
+        ACC[i].y = ACC[i].y * A + a.y * B;
+        ACC[i].z = ACC[i].z * A + a.z * B;
+        ACC[i].w = ACC[i].w * A + a.w * B;
+      }
+      M = Mn;
+    }
+    bf16_t* op = p.o + tok * p.sot + (int64_t)(kvh * G + hl) * p.soh;
+#pragma unroll
+    for (int ds = 0; ds < NDV; ds++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int d0 = 128 * ds + 32 * g + 8 * r;
+        if (d0 >= DV) continue;
+        const float4 lo = ACC[(ds * 4 + r) * 2], hi = ACC[(ds * 4 + r) * 2 + 1];
+        uint4 pk;
+        pk.x = pack_bf16x2(lo.x / L, lo.y / L);
+        pk.y = pack_bf16x2(lo.z / L, lo.w / L);
+        pk.z = pack_bf16x2(hi.x / L, hi.y / L);
+        pk.w = pack_bf16x2(hi.z / L, hi.w / L);
+        *(uint4*)(op + d0) = pk;
+      }
   }
 }
 
@@ -520,8 +664,46 @@ __global__ __launch_bounds__(256) void store_kv_kernel(const uint8_t* __restrict
 template <int DK, int DV>
 static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hipStream_t stream) {
   const bool fast = p.page_shift >= 4;  // page size a power of two >= 16
-  if (mode == 0) {  // decode split + combine
+  if (mode == 0 || mode == 3 || mode == 4) {
+    // decode: chunks folded inside one workgroup per (sequence, kv head) when that fills the machine
+    // (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3). Same bits.
     const int G = p.Hq / p.Hkv;
+    constexpr int NW = 4;
+    if (G > 32) return VX_ERR_UNSUPPORTED;
+    const bool fits = (G <= 16 ? fused_lds_bytes<DV, 1, NW>() : fused_lds_bytes<DV, 2, NW>()) <= 160 * 1024;
+    if (mode == 4 && !fits) return VX_ERR_UNSUPPORTED;
+    const bool fused = mode == 4 || (mode == 0 && fits && (int64_t)p.num_seqs * p.Hkv * NW >= 2048);
+    if (fused) {
+      const dim3 grid(p.Hkv, p.num_seqs);
+#define VX_FUSED(KERNEL, QTV, KINDV)                                                               \
+  do {                                                                                             \
+    constexpr int LDSB = fused_lds_bytes<DV, QTV, NW>();                                           \
+    static bool attr_set = false;                                                                  \
+    if (!attr_set) {                                                                               \
+      if (hipFuncSetAttribute((const void*)KERNEL<DK, DV, QTV, KINDV, NW>,                         \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, LDSB) != hipSuccess) {   \
+        (void)hipGetLastError();                                                                   \
+        return VX_ERR_LAUNCH;                                                                      \
+      }                                                                                            \
+      attr_set = true;                                                                             \
+    }                                                                                              \
+    KERNEL<DK, DV, QTV, KINDV, NW><<<grid, 64 * NW, LDSB, stream>>>(p);                            \
+  } while (0)
+      if (G <= 16) {
+        if constexpr (DK <= 128 && DV <= 128) {
+          if (fast) VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_FAST);
+          else VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_GENERIC);
+        } else {
+          if (fast) VX_FUSED(attn_decode_fused_kernel, 1, SRC_FAST);
+          else VX_FUSED(attn_decode_fused_kernel, 1, SRC_GENERIC);
+        }
+      } else {
+        if (fast) VX_FUSED(attn_decode_fused_kernel, 2, SRC_FAST);
+        else VX_FUSED(attn_decode_fused_kernel, 2, SRC_GENERIC);
+      }
+#undef VX_FUSED
+      return launch_status();
+    }
     dim3 grid(p.Hkv, p.num_seqs, p.max_chunks);
     if (G <= 16) {
       if constexpr (DK <= 128 && DV <= 128) {
@@ -531,13 +713,12 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
         if (fast) attn_decode_split_kernel<DK, DV, 1, SRC_FAST><<<grid, 64, 0, stream>>>(p);
         else attn_decode_split_kernel<DK, DV, 1, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
       }
-    } else if (G <= 32) {
+    } else {
       if (fast) attn_decode_split_kernel<DK, DV, 2, SRC_FAST><<<grid, 64, 0, stream>>>(p);
       else attn_decode_split_kernel<DK, DV, 2, SRC_GENERIC><<<grid, 64, 0, stream>>>(p);
-    } else {
-      return VX_ERR_UNSUPPORTED;
     }
-    attn_decode_combine_kernel<DV><<<dim3(p.Hq, p.num_seqs), 64, 0, stream>>>(p);
+    if (G <= 16) attn_decode_combine_kernel<DV, 1><<<dim3(p.Hkv, p.num_seqs), 64, 0, stream>>>(p);
+    else attn_decode_combine_kernel<DV, 2><<<dim3(p.Hkv, p.num_seqs), 64, 0, stream>>>(p);
   } else {
     constexpr int QT = (DK > 128) ? 1 : 2;
     const int rows = max_q > 0 ? max_q : total_q;
@@ -557,14 +738,23 @@ extern "C" {
 
 int vx_attn_chunk_size() { return ATT_CHUNK; }
 
-// bytes of workspace the decode path needs
-int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Dv,
-                                             int64_t max_kv_len) {
-  const int64_t nch = (max_kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
-  return num_seqs * Hq * nch * (Dv + 2) * 4;
+// floats of one chunk image: per q-tile (16 heads) and 128-dim set, 8 float4 slots per lane, plus one
+// slot per q-tile for (m, l); 64 lanes x 4 floats per slot
+static inline int64_t part_image_floats(int64_t Hq, int64_t Hkv, int64_t Dv) {
+  const int64_t qt = (Hq / Hkv + 15) / 16, ndv = (Dv + 127) / 128;
+  return (qt * ndv * 8 + qt) * 256;
 }
 
-// mode: 0 = paged decode (every sequence has <= 1 query token; needs workspace),
+// bytes of workspace the decode path needs
+int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Hkv, int64_t Dv,
+                                             int64_t max_kv_len) {
+  if (num_seqs <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Dv <= 0 || max_kv_len <= 0) return 0;
+  const int64_t nch = (max_kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
+  return num_seqs * Hkv * nch * part_image_floats(Hq, Hkv, Dv) * 4;
+}
+
+// mode: 0 = paged decode (every sequence has <= 1 query token; needs workspace); 3 / 4 = the same,
+//       forcing the split + combine kernels / the fused kernel (0 chooses; results are identical),
 //       1 = paged general (prefill / mixed), 2 = packed K/V (cu_seqlens_k, no page table).
 int vx_attention(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens_q,
                  const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
@@ -575,10 +765,11 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
                  int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (!q || !k || !v || !out || !cu_seqlens_q) return VX_ERR_ARG;
   if (total_q < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return VX_ERR_ARG;
-  if (mode < 0 || mode > 2) return VX_ERR_ARG;
+  if (mode < 0 || mode > 4) return VX_ERR_ARG;
   if (mode != 2 && (!seqused_k || !block_table || page_size <= 0 || max_pages <= 0)) return VX_ERR_ARG;
   if (mode == 2 && !cu_seqlens_k) return VX_ERR_ARG;
-  if (mode == 0 && !causal) return VX_ERR_UNSUPPORTED;
+  const bool decode = mode == 0 || mode == 3 || mode == 4;
+  if (decode && !causal) return VX_ERR_UNSUPPORTED;
   if (total_q == 0 || num_seqs == 0) return VX_OK;
   if (num_seqs > 65535 || Hq > 65535) return VX_ERR_UNSUPPORTED;
   // 16-byte row accesses
@@ -601,15 +792,15 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
   p.Hq = Hq; p.Hkv = Hkv; p.num_seqs = (int)num_seqs;
   p.qk_scale = softmax_scale * 1.44269504f;
   p.causal = causal;
-  if (mode == 0) {
+  if (decode) {
     const int64_t max_kv = max_pages * (int64_t)page_size;
     const int64_t nch = (max_kv + ATT_CHUNK - 1) / ATT_CHUNK;
     if (nch > 0x7fffffff) return VX_ERR_ARG;
-    const int64_t need = num_seqs * Hq * nch * (Dv + 2) * 4;
-    if (!workspace || workspace_bytes < need) return VX_ERR_WORKSPACE;
+    p.img_floats = part_image_floats(Hq, Hkv, Dv);
+    const int64_t need = num_seqs * Hkv * nch * p.img_floats * 4;
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return VX_ERR_WORKSPACE;
     p.max_chunks = (int)nch;
-    p.part_acc = (float*)workspace;
-    p.part_ml = (float*)workspace + num_seqs * Hq * nch * Dv;
+    p.part = (float*)workspace;
   }
   const int tq = (int)total_q;
   if (Dk == 128 && Dv == 128) return launch_attn<128, 128>(p, mode, max_seqlen_q, tq, stream);

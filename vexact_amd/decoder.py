@@ -199,7 +199,8 @@ class StepBuffers:
         self.max_tiles = lib.vx_moe_max_tiles(T * k, cfg.num_experts, self.bm)
         self.route_ints = z(2 * cfg.num_experts + 1 + 3 * T * k + 3 * self.max_tiles, dtype=i32)
         self.attn_ws = torch.empty(
-            max(16, lib.vx_paged_attn_decode_workspace_bytes(B, cfg.num_heads, cfg.head_dim, self.max_blocks * cfg.page_size)),
+            max(16, lib.vx_paged_attn_decode_workspace_bytes(B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
+                                                            self.max_blocks * cfg.page_size)),
             dtype=torch.uint8, device=device)
         # sampling: one row per sequence
         self.last_h = z(B, H, dtype=bf)

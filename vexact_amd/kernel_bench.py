@@ -122,7 +122,7 @@ def main() -> None:
         used = torch.tensor(L, dtype=torch.int32, device=dev)
         btd = torch.tensor(bt, device=dev)
         out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
-        ws = torch.empty(_lib.load().vx_paged_attn_decode_workspace_bytes(B, Hq, D, 4096), dtype=torch.uint8, device=dev)
+        ws = torch.empty(_lib.load().vx_paged_attn_decode_workspace_bytes(B, Hq, Hkv, D, 4096), dtype=torch.uint8, device=dev)
         report(f"paged decode attention (sum L={int(L.sum())})",
                timeit(lambda li: ops.paged_attention(q, kc[li], vc[li], cu, used, btd, D**-0.5, 1, out=out, workspace=ws)),
                int(L.sum()) * 2 * Hkv * D * 2 + 2 * B * Hq * D * 2 + sum(pages) * 4)

@@ -349,9 +349,12 @@ def paged_attention(
     max_seqlen_q: int = 0,
     out: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
+    decode_kernel: str = "auto",
 ) -> torch.Tensor:
     """Causal paged attention. ``max_seqlen_q == 1`` selects the split-KV decode kernels; any other
-    value the general kernel (identical bits per row)."""
+    value the general kernel (identical bits per row). ``decode_kernel`` forces one of the two decode
+    forms ("split": one wavefront per 256-key chunk plus a combine launch, "fused": chunks folded
+    inside one workgroup per (sequence, kv head)); "auto" picks by batch size. Same bits either way."""
     T, Hq, Dk = q.shape
     Hkv, Dv = k_cache.shape[2], v_cache.shape[-1]
     o = out if out is not None else torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
@@ -365,10 +368,10 @@ def paged_attention(
     B = seqused_k.numel()
     page = k_cache.shape[1]
     max_pages = page_table.shape[1]
-    mode = 0 if max_seqlen_q == 1 else 1
+    mode = {"auto": 0, "split": 3, "fused": 4}[decode_kernel] if max_seqlen_q == 1 else 1
     ws = None
-    if mode == 0:
-        need = lib.vx_paged_attn_decode_workspace_bytes(B, Hq, Dv, max_pages * page)
+    if mode != 1:
+        need = lib.vx_paged_attn_decode_workspace_bytes(B, Hq, Hkv, Dv, max_pages * page)
         ws = workspace if workspace is not None and workspace.numel() * workspace.element_size() >= need else _workspace(need, q.device)
     _lib.check(
         lib.vx_attention(
