@@ -668,14 +668,14 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
     // decode: chunks folded inside one workgroup per (sequence, kv head) when that fills the machine
     // (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3). Same bits.
     const int G = p.Hq / p.Hkv;
-    constexpr int NW = 4;
+    constexpr int NW1 = 8, NW2 = 4;  // wavefronts per block for one / two q-tiles (LDS: 84 / 96 KB at Dv = 128)
     if (G > 32) return VX_ERR_UNSUPPORTED;
-    const bool fits = (G <= 16 ? fused_lds_bytes<DV, 1, NW>() : fused_lds_bytes<DV, 2, NW>()) <= 160 * 1024;
+    const bool fits = (G <= 16 ? fused_lds_bytes<DV, 1, NW1>() : fused_lds_bytes<DV, 2, NW2>()) <= 160 * 1024;
     if (mode == 4 && !fits) return VX_ERR_UNSUPPORTED;
-    const bool fused = mode == 4 || (mode == 0 && fits && (int64_t)p.num_seqs * p.Hkv * NW >= 2048);
+    const bool fused = mode == 4 || (mode == 0 && fits && (int64_t)p.num_seqs * p.Hkv >= 512);
     if (fused) {
       const dim3 grid(p.Hkv, p.num_seqs);
-#define VX_FUSED(KERNEL, QTV, KINDV)                                                               \
+#define VX_FUSED(KERNEL, QTV, KINDV, NW)                                                             \
   do {                                                                                             \
     constexpr int LDSB = fused_lds_bytes<DV, QTV, NW>();                                           \
     static bool attr_set = false;                                                                  \
@@ -691,15 +691,15 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
   } while (0)
       if (G <= 16) {
         if constexpr (DK <= 128 && DV <= 128) {
-          if (fast) VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_FAST);
-          else VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_GENERIC);
+          if (fast) VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_FAST, NW1);
+          else VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_GENERIC, NW1);
         } else {
-          if (fast) VX_FUSED(attn_decode_fused_kernel, 1, SRC_FAST);
-          else VX_FUSED(attn_decode_fused_kernel, 1, SRC_GENERIC);
+          if (fast) VX_FUSED(attn_decode_fused_kernel, 1, SRC_FAST, NW1);
+          else VX_FUSED(attn_decode_fused_kernel, 1, SRC_GENERIC, NW1);
         }
       } else {
-        if (fast) VX_FUSED(attn_decode_fused_kernel, 2, SRC_FAST);
-        else VX_FUSED(attn_decode_fused_kernel, 2, SRC_GENERIC);
+        if (fast) VX_FUSED(attn_decode_fused_kernel, 2, SRC_FAST, NW2);
+        else VX_FUSED(attn_decode_fused_kernel, 2, SRC_GENERIC, NW2);
       }
 #undef VX_FUSED
       return launch_status();
