@@ -148,11 +148,13 @@ int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, i
  *   epi 0: plain store (replaces group_gemm_same_nk, group_gemm/kernel/group_gemm.py:65-237)
  *   epi 1: w = gate rows, w2 = up rows, C = round(round(round(silu(round(g))) * round(u)) * s) with
  *          s = row_scale[row_scale_idx[row]] (adds the glue of fused_moe.py:75-88)
- * bm (rows per tile) must match the tile table: 16 / 32 / 64 stream weights, 128 is LDS-tiled. */
+ * bm (rows per tile) must match the tile table: 16 / 32 / 64 stream weights, 128 is LDS-tiled,
+ * 256 uses 256x256 tiles with direct-to-LDS loads (prefill sizes; needs K % 64 == 0 and x_rows = the
+ * number of rows addressable in x, which bounds its 32-bit load offsets; other bm ignore x_rows). */
 int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64_t ldw,
                 int64_t w_gstride, void* c, int64_t ldc, int64_t N, int64_t K, const int* tile_group,
                 const int* tile_row0, const int* tile_rows, int64_t max_tiles, int bm,
-                const int* row_src, const void* row_scale, const int* row_scale_idx, int epi,
+                const int* row_src, const void* row_scale, const int* row_scale_idx, int epi, int64_t x_rows,
                 hipStream_t stream);
 
 /* Replace expert_histogram / moe_scatter / moe_gather, group_gemm/kernel/moe.py:52-81, 304-335, 131-161.

@@ -69,7 +69,7 @@ def test_router_tie_rule():
 
 
 @pytest.mark.parametrize("T,E,k,bm", [(1, 128, 8, 32), (256, 128, 8, 32), (4096, 128, 8, 128), (700, 6, 2, 64), (33, 4, 1, 16),
-                                      (1500, 128, 8, 64)])
+                                      (1500, 128, 8, 64), (9000, 64, 4, 256)])
 def test_routing_integers_exact(T, E, k, bm):
     g = torch.Generator().manual_seed(T)
     sel = torch.randint(0, E, (T, k), generator=g)
@@ -160,6 +160,27 @@ def test_fused_moe_rows_do_not_depend_on_token_count():
     assert_bitwise(one, full[3000:3001], "token 3000 alone")
     ref = OM.fused_moe_ref(x[:128], w[:128], sel[:128], gate, up, down)
     assert_bf16_close(full[:128], ref, max_ulp=2, atol_frac=2e-3, what="T=4096 rows vs oracle")
+
+
+def test_wide_expert_tiles_agree_bitwise():
+    # prefill-sized batch: 256-row expert tiles (direct-to-LDS kernel, gate/up rows interleaved per
+    # wavefront) against 128-row tiles, against a short slice of the same tokens, and the oracle
+    T, H, I, E, k = 8300, 512, 192, 24, 4
+    x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=21)
+    xg, wg, sg, gg, ug, dg = (t.cuda() for t in (x, w, sel, gate, up, down))
+    assert ops.moe_tile_rows(T) == 256
+    full = fused_moe_forward(E, wg, sg, xg, gg, ug, dg)
+    outs = {}
+    for bm in (128, 256):
+        r = ops.moe_route(sg, E, bm=bm)
+        hw = ops.moe_gemm(xg, gg, r, w2=ug, row_src=r.sorted_token, row_scale=wg, row_scale_idx=r.sorted_flat)
+        outs[bm] = (hw, ops.moe_gemm(hw, dg, r))
+    assert_bitwise(outs[256][0], outs[128][0], "gate/up + SwiGLU, 256- vs 128-row tiles")
+    assert_bitwise(outs[256][1], outs[128][1], "down, 256- vs 128-row tiles")
+    part = fused_moe_forward(E, wg[:300], sg[:300], xg[:300], gg, ug, dg)
+    assert_bitwise(part, full[:300], "first 300 tokens alone vs inside 8300")
+    ref = OM.fused_moe_ref(x[:96], w[:96], sel[:96], gate, up, down)
+    assert_bf16_close(full[:96], ref, max_ulp=2, atol_frac=2e-3, what="T=8300 rows vs oracle")
 
 
 def test_gather_with_fused_norm_equals_separate_kernels():

@@ -38,7 +38,7 @@ PROTOTYPES = {
     "vx_moe_route": (_I, [_P, _I, _L, _I, _I, _I] + [_P] * 8 + [_L, _P]),
     "vx_moe_gemm": (
         _I,
-        [_P, _L, _P, _P, _L, _L, _P, _L, _L, _L, _P, _P, _P, _L, _I, _P, _P, _P, _I, _P],
+        [_P, _L, _P, _P, _L, _L, _P, _L, _L, _L, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _P],
     ),
     "vx_expert_histogram": (_I, [_P, _I, _L, _I, _P, _P]),
     "vx_moe_scatter": (_I, [_P, _P, _P, _L, _I, _L, _L, _L, _P]),

@@ -8,6 +8,7 @@
 //   group_gemm_same_nk                                group_gemm/kernel/group_gemm.py:65-237
 //   silu * up * routing-weight glue                   fused_moe.py:75-88
 #include "gemm_core.h"
+#include "gemm_wide.h"
 
 namespace vx {
 
@@ -372,12 +373,13 @@ int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, i
 
 // Grouped GEMM over a tile table: C[rows of tile] = X[row_src[rows]] * W[group]^T.
 // epi 0: plain bf16 store. epi 1: SwiGLU with w = gate rows, w2 = up rows, scaled per row by
-// row_scale[row_scale_idx[row]].  bm in {16, 32, 64} selects the streaming kernel, 128 the tiled one.
+// row_scale[row_scale_idx[row]].  bm in {16, 32, 64} selects the streaming kernel, 128 the tiled one,
+// 256 the wide one (x_rows = rows addressable in x; only that kernel needs it).
 int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64_t ldw,
                 int64_t w_gstride, void* c, int64_t ldc, int64_t N, int64_t K, const int* tile_group,
                 const int* tile_row0, const int* tile_rows, int64_t max_tiles, int bm,
                 const int* row_src, const void* row_scale, const int* row_scale_idx, int epi,
-                hipStream_t stream) {
+                int64_t x_rows, hipStream_t stream) {
   if (!x || !w || !c || !tile_group || !tile_row0 || !tile_rows) return VX_ERR_ARG;
   if (N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff || max_tiles < 0) return VX_ERR_ARG;
   if (epi != EPI_PLAIN && epi != EPI_SWIGLU) return VX_ERR_ARG;
@@ -414,6 +416,9 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
         gemm_tiled_kernel<EPI_PLAIN, true><<<dim3((unsigned)((N + 127) / 128), my), 256, 0, stream>>>(p);
       break;
     }
+    case 256:  // prefill sizes: 256x256 tiles, direct-to-LDS loads (needs K % 64 == 0 and x_rows)
+      if (x_rows <= 0 || !gemm_wide_grouped_launch(p, epi, max_tiles, x_rows, stream)) return VX_ERR_UNSUPPORTED;
+      break;
     default: return VX_ERR_ARG;
   }
 #undef VX_GG

@@ -446,13 +446,16 @@ def router_topk(
     return w, idx
 
 
-def moe_tile_rows(num_tokens: int) -> int:
-    """Rows per expert tile, chosen from the token count only (any choice gives the same bits)."""
+def moe_tile_rows(num_tokens: int, wide_ok: bool = True) -> int:
+    """Rows per expert tile, chosen from the token count only (any choice gives the same bits).
+    ``wide_ok``: both GEMM depths are multiples of 64, which the 256-row kernel needs."""
     if num_tokens <= 256:
         return 32
     if num_tokens <= 1024:
         return 64
-    return 128
+    if num_tokens < 8192 or not wide_ok:
+        return 128
+    return 256
 
 
 class MoeRouting:
@@ -517,7 +520,7 @@ def moe_gemm(
             x.data_ptr(), x.stride(0), w.data_ptr(), _ptr(w2), w.stride(1), w.stride(0), c.data_ptr(), c.stride(0),
             N, K, routing.tile_group.data_ptr(), routing.tile_row0.data_ptr(), routing.tile_rows.data_ptr(),
             routing.max_tiles, routing.bm, _ptr(row_src), _ptr(row_scale), _ptr(row_scale_idx),
-            1 if w2 is not None else 0, _stream(),
+            1 if w2 is not None else 0, x.shape[0], _stream(),
         ),
         "vx_moe_gemm",
     )
@@ -601,7 +604,9 @@ def fused_moe(
     k = selected_experts.shape[1]
     x = hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous()
     rw = routing_weights.contiguous()
-    r = moe_route(selected_experts, num_experts)
+    H_, I_ = gate_w.shape[-1], down_w.shape[-1]
+    r = moe_route(selected_experts, num_experts,
+                  bm=moe_tile_rows(selected_experts.shape[0], wide_ok=(H_ % 64 == 0 and I_ % 64 == 0)))
     hw = moe_gemm(x, gate_w, r, w2=up_w, row_src=r.sorted_token, row_scale=rw, row_scale_idx=r.sorted_flat)
     o = moe_gemm(hw, down_w, r)
     return moe_gather(o, r.scatter_index, residual=residual, out=out)
