@@ -144,6 +144,37 @@ def main() -> None:
             report(f"prefill gemm {name} M={M} N={N} K={K}", timeit(lambda li: ops.gemm_nt(xx, w_, out=c), n_layers=2),
                    flops=2 * M * N * K)
             del w_, xx, c
+    if "prefill" in what:
+        # MoE expert GEMMs over a prefill chunk (256-row expert tiles)
+        for T in (8192, 32768):
+            x = rnd(T, H, std=1.0)
+            logits = torch.randn(T, E, generator=g, device=dev)
+            w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
+            r = ops.moe_route(idx, E, bm=ops.moe_tile_rows(T))
+            gu = rnd(E, 2 * I, H)
+            dn = rnd(E, H, I)
+            hw = torch.empty(T * k, I, dtype=torch.bfloat16, device=dev)
+            eo = torch.empty(T * k, H, dtype=torch.bfloat16, device=dev)
+            report(f"prefill moe gate/up T={T}",
+                   timeit(lambda li: ops.moe_gemm(x, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=w,
+                                                  row_scale_idx=r.sorted_flat, out=hw), n_layers=2),
+                   flops=2 * T * k * 2 * I * H)
+            report(f"prefill moe down T={T}", timeit(lambda li: ops.moe_gemm(hw, dn, r, out=eo), n_layers=2),
+                   flops=2 * T * k * H * I)
+            del x, logits, gu, dn, hw, eo
+        # causal attention over whole prompts: 8 sequences of 1024 tokens, paged cache
+        Hq, Hkv, D, page, S, Lp = 32, 4, 128, 16, 8, 1024
+        npg = S * Lp // page
+        kc = rnd(npg, Hkv, page, D, std=1.0).permute(0, 2, 1, 3)
+        vc = rnd(npg, Hkv, page, D, std=1.0).permute(0, 2, 1, 3)
+        q = rnd(S * Lp, Hq, D, std=1.0)
+        cu = torch.arange(0, S * Lp + 1, Lp, dtype=torch.int32, device=dev)
+        used = torch.full((S,), Lp, dtype=torch.int32, device=dev)
+        bt = torch.arange(npg, dtype=torch.int32, device=dev).view(S, Lp // page)
+        out = torch.empty(S * Lp, Hq, D, dtype=torch.bfloat16, device=dev)
+        report(f"prefill attention {S} x {Lp} tokens",
+               timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, bt, D**-0.5, Lp, out=out), n_layers=2),
+               flops=4 * S * Hq * D * Lp * (Lp + 1) // 2)
     if "small" in what:
         one = torch.zeros(64, dtype=torch.int32, device=dev)
         lib = _lib.load()
