@@ -60,6 +60,24 @@ def test_router_topk_indices_exact(T, E, k, logit_dtype):
     torch.testing.assert_close(w32.cpu(), w_ref32, atol=1e-6, rtol=1e-5)
 
 
+@pytest.mark.parametrize("T,E,k", [(300, 128, 8), (64, 200, 6), (40, 512, 8), (7, 60, 60)])
+def test_router_bf16_kernel_equals_generic_kernel(T, E, k):
+    """bf16 logits take a packed-key kernel; the same values as fp32 take the generic one. Heavy ties
+    (values on a coarse grid, +-0) must select the same experts with the same weights."""
+    g = torch.Generator().manual_seed(E + k)
+    logits = (torch.randint(-6, 7, (T, E), generator=g).float() * 0.25).to(torch.bfloat16)
+    logits[0, :] = 0.0
+    logits[1, ::2] = -0.0
+    for renorm in (True, False):
+        wb, ib = ops.router_topk(logits.cuda(), k, renorm=renorm)
+        wf, i_f = ops.router_topk(logits.float().cuda(), k, renorm=renorm)
+        assert torch.equal(ib.cpu(), i_f.cpu())
+        assert_bitwise(wb, wf, "router weights, bf16-logit kernel vs generic kernel")
+    w_ref, i_ref = OM.router_ref(logits.float(), k)
+    wb, ib = ops.router_topk(logits.cuda(), k)
+    assert torch.equal(ib.cpu().long(), i_ref.long())
+
+
 def test_router_tie_rule():
     logits = torch.zeros(3, 16)
     logits[1, [5, 9, 2]] = 1.0

@@ -85,6 +85,79 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict
   }
 }
 
+// bf16 logits: value and expert index fit one 32-bit key (order-preserving 16 bits of the value above
+// 0xffff - e), so a round of the selection is one integer max over the wavefront, done with DPP row
+// operations and four lane reads instead of 18 cross-lane permutes. Same selections, same tie rule
+// (equal values: lower index; -0 and +0 are equal), and the selected probability is recomputed from
+// the winner's value with the expression its owner used, so the outputs are bit-identical to the
+// kernel above.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false));   // lanes i ^ 1
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false));   // lanes i ^ 2
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false));  // half-row mirror
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false));  // row mirror
+  const uint32_t a = __builtin_amdgcn_readlane((int)v, 0), b = __builtin_amdgcn_readlane((int)v, 16);
+  const uint32_t c = __builtin_amdgcn_readlane((int)v, 32), d = __builtin_amdgcn_readlane((int)v, 48);
+  return max(max(a, b), max(c, d));
+}
+
+template <int PER, bool OUT_BF16, bool IDX64>
+__global__ __launch_bounds__(256) void router_topk_bf16_kernel(const bf16_t* __restrict__ logits,
+                                                               void* __restrict__ weights_out,
+                                                               void* __restrict__ idx_out, int64_t T,
+                                                               int E, int k, int64_t ld, int renorm) {
+  const int64_t tok = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tok >= T) return;
+  const int lane = threadIdx.x & 63;
+  float x[PER];
+  uint32_t key[PER];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    const int e = lane + 64 * i;
+    key[i] = 0;  // below every real key
+    x[i] = -INFINITY;
+    if (e < E) {
+      uint32_t b = logits[tok * ld + e];
+      x[i] = bf16_to_f32((bf16_t)b);
+      if (b == 0x8000u) b = 0;  // -0 ties with +0
+      const uint32_t ord = (b & 0x8000u) ? (~b & 0xffffu) : (b | 0x8000u);
+      key[i] = (ord << 16) | (0xffffu - (uint32_t)e);
+    }
+    mx = fmaxf(mx, x[i]);
+  }
+  mx = wave_max(mx);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; i++) s += (lane + 64 * i < E) ? expf(x[i] - mx) : 0.f;
+  s = wave_sum(s);
+  float wsel = 0.f;
+  int isel = 0;
+  float tot = 0.f;
+  for (int j = 0; j < k; j++) {
+    uint32_t best = key[0];
+#pragma unroll
+    for (int i = 1; i < PER; i++) best = max(best, key[i]);
+    best = wave_max_u32(best);
+    const int bi = (int)(0xffffu - (best & 0xffffu));
+    const uint32_t ord = best >> 16;
+    const uint32_t bits = (ord & 0x8000u) ? (ord & 0x7fffu) : (~ord & 0xffffu);
+    const float p = expf(bf16_to_f32((bf16_t)bits) - mx) / s;
+#pragma unroll
+    for (int i = 0; i < PER; i++)
+      if (key[i] == best) key[i] = 0;
+    tot += p;
+    if (lane == j) { wsel = p; isel = bi; }
+  }
+  if (lane < k) {
+    const float w = renorm ? wsel / tot : wsel;
+    if constexpr (OUT_BF16) ((bf16_t*)weights_out)[tok * k + lane] = f32_to_bf16(w);
+    else ((float*)weights_out)[tok * k + lane] = w;
+    if constexpr (IDX64) ((int64_t*)idx_out)[tok * k + lane] = isel;
+    else ((int*)idx_out)[tok * k + lane] = isel;
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // Routing integers, one 1024-thread block. For n = T*k flat entries (token-major, slot-minor):
 //   splits[e]         = number of entries routed to expert e
@@ -324,6 +397,20 @@ int vx_router_topk(const void* logits, void* weights_out, void* idx_out, int64_t
 #define VX_RT(LB, OB, I64)                                                                   \
   router_topk_kernel<LB, OB, I64><<<(unsigned)blocks, 256, 0, stream>>>(logits, weights_out, \
                                                                         idx_out, T, E, k, ld, renorm)
+  if (logits_bf16) {
+#define VX_RTB(PERV)                                                                                  \
+  do {                                                                                                \
+    if (out_bf16 && idx_i64) router_topk_bf16_kernel<PERV, true, true><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)logits, weights_out, idx_out, T, E, k, ld, renorm); \
+    else if (out_bf16) router_topk_bf16_kernel<PERV, true, false><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)logits, weights_out, idx_out, T, E, k, ld, renorm); \
+    else if (idx_i64) router_topk_bf16_kernel<PERV, false, true><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)logits, weights_out, idx_out, T, E, k, ld, renorm); \
+    else router_topk_bf16_kernel<PERV, false, false><<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)logits, weights_out, idx_out, T, E, k, ld, renorm); \
+  } while (0)
+    if (E <= 128) VX_RTB(2);
+    else if (E <= 256) VX_RTB(4);
+    else VX_RTB(8);
+#undef VX_RTB
+    return launch_status();
+  }
   const int sel = (logits_bf16 ? 4 : 0) | (out_bf16 ? 2 : 0) | (idx_i64 ? 1 : 0);
   switch (sel) {
     case 0: VX_RT(false, false, false); break;

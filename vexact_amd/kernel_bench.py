@@ -97,7 +97,8 @@ def main() -> None:
         report("moe route", timeit(lambda li: ops.moe_route(idx, E, bm=32)), B * k * 16)
         report("moe gather + residual", timeit(lambda li: ops.moe_gather(eo, r.scatter_index, residual=x, out=y)),
                B * k * H * 2 + 2 * B * H * 2)
-        report("router top-k", timeit(lambda li: ops.router_topk(logits, k, index_dtype=torch.int32)), B * E * 4)
+        lb = logits.to(torch.bfloat16)
+        report("router top-k (bf16 logits)", timeit(lambda li: ops.router_topk(lb, k, index_dtype=torch.int32)), B * E * 2)
     if "attn" in what:
         Hq, Hkv, D, page = 32, 4, 128, a.page
         rng = np.random.default_rng(5)
