@@ -339,9 +339,19 @@ __global__ __launch_bounds__(256) void moe_gather_vec_kernel(const bf16_t* __res
     const int c = 4 * (tid + 256 * j);
     if (c < H) {
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-      for (int i = 0; i < k; i++) {
-        const uint2 raw = *(const uint2*)(x + (int64_t)index[t * k + i] * ldx + c);
-        a0 += bf16lo(raw.x); a1 += bf16hi(raw.x); a2 += bf16lo(raw.y); a3 += bf16hi(raw.y);
+      // slots are summed in ascending order, eight rows requested at a time so that their loads
+      // overlap (a slot past k re-reads the last row and is not added)
+      for (int i0 = 0; i0 < k; i0 += 8) {
+        uint2 raw[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+          raw[u] = *(const uint2*)(x + (int64_t)index[t * k + min(i0 + u, k - 1)] * ldx + c);
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          if (i0 + u < k) {
+            a0 += bf16lo(raw[u].x); a1 += bf16hi(raw[u].x); a2 += bf16lo(raw[u].y); a3 += bf16hi(raw[u].y);
+          }
+        }
       }
       uint2 pk;
       pk.x = pack_bf16x2(a0, a1);
