@@ -39,6 +39,17 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
       *(uint2*)(v_cache + crow + (int64_t)(h - Hq - Hkv) * csh + 4 * lane) = raw;
     return;
   }
+  // position, norm weight and rotary rows are requested before the reduction so that their
+  // latency overlaps it
+  const bf16_t* w = (h < Hq) ? qw : kw;
+  int64_t pos = (int64_t)positions[t];
+  pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+  uint2 wr = make_uint2(0, 0), cr = make_uint2(0, 0), sr = make_uint2(0, 0);
+  if (own) {
+    wr = *(const uint2*)(w + 4 * lane);
+    cr = *(const uint2*)(cos_t + pos * D + 4 * lane);
+    sr = *(const uint2*)(sin_t + pos * D + 4 * lane);
+  }
   float x[4] = {bf16lo(raw.x), bf16hi(raw.x), bf16lo(raw.y), bf16hi(raw.y)};
   float acc = 0.f;
   if (own) {
@@ -47,15 +58,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   }
   const float tot = wave_sum(acc);
   const float inv = 1.0f / sqrtf(tot / (float)D + eps);
-  const bf16_t* w = (h < Hq) ? qw : kw;
-  int64_t pos = (int64_t)positions[t];
-  pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
   float y[4], cs[4], sn[4];
   if (own) {
-    const uint2 wr = *(const uint2*)(w + 4 * lane);
     const float wf[4] = {bf16lo(wr.x), bf16hi(wr.x), bf16lo(wr.y), bf16hi(wr.y)};
-    const uint2 cr = *(const uint2*)(cos_t + pos * D + 4 * lane);
-    const uint2 sr = *(const uint2*)(sin_t + pos * D + 4 * lane);
     cs[0] = bf16lo(cr.x); cs[1] = bf16hi(cr.x); cs[2] = bf16lo(cr.y); cs[3] = bf16hi(cr.y);
     sn[0] = bf16lo(sr.x); sn[1] = bf16hi(sr.x); sn[2] = bf16lo(sr.y); sn[3] = bf16hi(sr.y);
 #pragma unroll

@@ -84,7 +84,7 @@ def main() -> None:
         w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
         r = ops.moe_route(idx, E, bm=ops.moe_tile_rows(B))
         U = int((r.splits > 0).sum())
-        gu = [rnd(E, 2 * I, H) for _ in range(NL)]
+        gu = [rnd(E, 2 * I, H + 64)[..., :H] for _ in range(NL)]  # 128 bytes of row padding, as the decoder allocates them
         dn = [rnd(E, H, I) for _ in range(NL)]
         hw = torch.empty(B * k, I, dtype=torch.bfloat16, device=dev)
         eo = torch.empty(B * k, H, dtype=torch.bfloat16, device=dev)
