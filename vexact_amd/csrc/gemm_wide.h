@@ -46,53 +46,95 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 __device__ __forceinline__ int wd_swz_x(int R) { return (R >> 1) & 7; }
 __device__ __forceinline__ int wd_swz_w(int R) { return (((R >> 4) & 3) << 1) | ((R >> 1) & 1); }
 
-static __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t wd_lds[];
+// One tile of the walk: rows [row0, row0 + rows) of C, output columns from n0, weights at wbase.
+struct WideTile {
+  int row0, rows, n0;
+  int64_t wbase;
+  bool ok;
+};
 
-  const int M = p.M, N = p.N, K = p.K;
+// GROUPED (MoE expert GEMMs at prefill sizes): row tiles come from the tile table of the routing
+// kernel (group, first row, row count; built for 256-row tiles, compact, -1 after the last used
+// entry), activation rows may be gathered through row_src, and tiles are numbered row-tile major, so
+// the workgroups of an XCD share one expert's weights and a few activation panels. tiles_m is then
+// the length of the table.
+// EPI_SWIGLU: the 256 weight rows of a tile are 128 gate rows and the 128 up rows of the same
+// output columns, interleaved so that wavefront wn holds gate columns [32 wn, +32) in its weight
+// fragments 0, 1 and the matching up columns in fragments 2, 3: LDS row 64 wn + 16 a + 4 j + b is
+// column 32 wn + 8 a + 4 (j & 1) + b of gate (j < 2) or up (j >= 2). A tile then yields 128 output
+// columns and a lane 8 consecutive ones per activation row.
+template <int EPI, bool GROUPED>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t wd_lds[];
+  constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;  // output columns per tile
+
+  const int N = p.N, K = p.K;
   const int tiles = tiles_m * tiles_n;
   const int G = gridDim.x;  // multiple of 8
   const int first = (blockIdx.x & 7) * (G >> 3) + (blockIdx.x >> 3);
-  if (first >= tiles) return;
+
+  auto tile_at = [&](int lin) {
+    WideTile t;
+    if constexpr (GROUPED) {
+      const int mt = lin / tiles_n;
+      const int grp = p.tile_group[mt];
+      t.ok = grp >= 0;
+      t.row0 = p.tile_row0[mt];
+      t.rows = p.tile_rows[mt];
+      t.n0 = (lin - mt * tiles_n) * NOUT;
+      t.wbase = (int64_t)(t.ok ? grp : 0) * p.w_gstride;
+    } else {
+      const int span = WD_GROUP_M * tiles_n;
+      const int grp = lin / span;
+      const int gm0 = grp * WD_GROUP_M;
+      const int gsz = min(WD_GROUP_M, tiles_m - gm0);
+      const int rem = lin - grp * span;
+      t.row0 = (gm0 + rem % gsz) * WD_BM;
+      t.rows = min(WD_BM, p.M - t.row0);
+      t.n0 = (rem / gsz) * NOUT;
+      t.wbase = 0;
+      t.ok = true;
+    }
+    return t;
+  };
+  if (first >= tiles || !tile_at(first).ok) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, g = lane >> 4;
   const int wm = wave >> 2, wn = wave & 3;
 
-  auto tile_origin = [&](int lin, int& row0, int& n0) {
-    const int span = WD_GROUP_M * tiles_n;
-    const int grp = lin / span;
-    const int gm0 = grp * WD_GROUP_M;
-    const int gsz = min(WD_GROUP_M, tiles_m - gm0);
-    const int rem = lin - grp * span;
-    row0 = (gm0 + rem % gsz) * WD_BM;
-    n0 = (rem / gsz) * WD_BN;
-  };
-
   // ---- load stream: instruction q of a step fills tile rows [8 (wave + 8 (q & 3)), +8) of X (q < 4)
   // or W (q >= 4). Byte offsets from the operand base fit 32 bits (host check).
   const int lrow = lane >> 3, lslot = lane & 7;
   uint32_t ld_off[8];
-  auto set_load_tile = [&](int lin) {
-    int row0, n0;
-    tile_origin(lin, row0, n0);
+  int64_t ld_wbase = 0;
+  auto set_load_tile = [&](const WideTile& t) {
+    ld_wbase = t.wbase;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int R = 8 * (wave + 8 * j) + lrow;
-      ld_off[j] = (uint32_t)(((int64_t)min(row0 + R, M - 1) * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
-      ld_off[4 + j] = (uint32_t)(((int64_t)min(n0 + R, N - 1) * p.ldw + (lslot ^ wd_swz_w(R)) * 8) * 2);
+      const int rr = t.row0 + min(R, t.rows - 1);  // rows past the tile re-read its last row (not stored)
+      const int64_t sr = (GROUPED && p.row_src) ? (int64_t)p.row_src[rr] : (int64_t)rr;
+      ld_off[j] = (uint32_t)((sr * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
+      int col;
+      if constexpr (EPI == EPI_SWIGLU) col = t.n0 + 32 * (R >> 6) + 8 * ((R >> 4) & 3) + 4 * ((R >> 2) & 1) + (R & 3);
+      else col = t.n0 + R;
+      ld_off[4 + j] = (uint32_t)(((int64_t)min(col, N - 1) * p.ldw + (lslot ^ wd_swz_w(R)) * 8) * 2);
     }
   };
   int ld_lin = first, ld_k = 0;
-  set_load_tile(ld_lin);
+  set_load_tile(tile_at(first));
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)wd_lds + wave * 1024;
+  // EPI_SWIGLU: weight rows 8 q .. 8 q + 7 of load instruction q = wave + 8 j have bit 3 of the row
+  // index equal to the parity of the wavefront, which says gate or up
+  const bf16_t* wsrc = (EPI == EPI_SWIGLU && (wave & 1)) ? p.w2 : p.w;
   // The loads are written as asm so that the compiler does not track them: told that they write LDS,
   // it would wait for them (vmcnt(0)) before the first fragment read after they are issued. The
   // wait that matters is the explicit one before the barrier that precedes their first use.
   auto issue_one = [&](int q, int stage) {
     const uint32_t dst = lds0 + stage * WD_STAGE + (q >> 2) * WD_XBYTES + (q & 3) * 8192;
-    const bf16_t* base = (q < 4 ? p.x : p.w) + ld_k;
+    const bf16_t* base = (q < 4 ? p.x : wsrc + ld_wbase) + ld_k;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
   };
@@ -100,9 +142,13 @@ static __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int
     ld_k += WD_BK;
     if (ld_k >= K) {
       ld_k = 0;
-      if (ld_lin + G < tiles) {
-        ld_lin += G;
-        set_load_tile(ld_lin);
+      const int nl = ld_lin + G;
+      if (nl < tiles) {
+        const WideTile t = tile_at(nl);
+        if (t.ok) {
+          ld_lin = nl;
+          set_load_tile(t);
+        }
       }
     }
   };
@@ -165,8 +211,8 @@ static __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int
   int st = 0;  // stage of the current step
   const bool vec_ok = (p.ldc & 7) == 0 && ((uintptr_t)p.c & 15) == 0;
   for (int lin = first; lin < tiles; lin += G) {
-    int row0, n0;
-    tile_origin(lin, row0, n0);
+    const WideTile t = tile_at(lin);
+    if (!t.ok) break;
     for (int kt = 0; kt < nk; kt++) {
       const uint8_t* cur_sb = wd_lds + st * WD_STAGE;
       const uint8_t* oth_sb = wd_lds + (st ^ 1) * WD_STAGE;
@@ -179,197 +225,15 @@ static __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int
       st ^= 1;
     }
 
-    // ---- epilogue: lane holds C[row0 + 128 wm + 16 i + r16][n0 + 64 wn + 16 g + 4 j + c]
-    const int nb = n0 + 64 * wn + 16 * g;
-    float bv[16];
-    if (p.bias) {
-#pragma unroll
-      for (int e = 0; e < 16; e++) bv[e] = bf16_to_f32(p.bias[min(nb + e, N - 1)]);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int m = row0 + 128 * wm + 16 * i + r16;
-      bf16_t o[16];
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          float v = acc[i][j][c];
-          if (p.bias) v += bv[4 * j + c];
-          o[4 * j + c] = f32_to_bf16(v);
-          acc[i][j][c] = 0.f;
-        }
-      if (m >= M) continue;
-      bf16_t* cp = p.c + (int64_t)m * p.ldc + nb;
-      if (vec_ok && nb + 15 < N) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          uint4 pk;
-          pk.x = (uint32_t)o[8 * h + 0] | ((uint32_t)o[8 * h + 1] << 16);
-          pk.y = (uint32_t)o[8 * h + 2] | ((uint32_t)o[8 * h + 3] << 16);
-          pk.z = (uint32_t)o[8 * h + 4] | ((uint32_t)o[8 * h + 5] << 16);
-          pk.w = (uint32_t)o[8 * h + 6] | ((uint32_t)o[8 * h + 7] << 16);
-          *(uint4*)(cp + 8 * h) = pk;
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 16; e++)
-          if (nb + e < N) cp[e] = o[e];
-      }
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // loads past the last step still target our LDS
-}
-
-// ---------------------------------------------------------------------------------------
-// Grouped form of the wide kernel (MoE expert GEMMs at prefill sizes). Row tiles come from the tile
-// table of the routing kernel (group, first row, row count; built for 256-row tiles, compact, -1
-// after the last used entry); activation rows may be gathered through row_src. Tiles are numbered
-// row-tile major (all column tiles of a row tile are consecutive), so the workgroups of an XCD share
-// one expert's weights and a few activation panels.
-// EPI_SWIGLU: the 256 weight rows of a tile are 128 gate rows and the 128 up rows of the same
-// output columns, interleaved so that wavefront wn holds gate columns [32 wn, +32) in its weight
-// fragments 0, 1 and the matching up columns in fragments 2, 3: LDS row 64 wn + 16 a + 4 j + b is
-// column 32 wn + 8 a + 4 (j & 1) + b of gate (j < 2) or up (j >= 2). A tile then yields 128 output
-// columns and a lane 8 consecutive ones per activation row.
-// ---------------------------------------------------------------------------------------
-template <int EPI>
-__global__ __launch_bounds__(512) void gemm_wide_grouped_kernel(GemmParams p, int max_m_tiles, int tiles_n) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t wd_lds[];
-  constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;  // output columns per tile
-
-  const int N = p.N, K = p.K;
-  const int tiles = max_m_tiles * tiles_n;
-  const int G = gridDim.x;  // multiple of 8
-  const int first = (blockIdx.x & 7) * (G >> 3) + (blockIdx.x >> 3);
-  if (first >= tiles || p.tile_group[first / tiles_n] < 0) return;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r16 = lane & 15, g = lane >> 4;
-  const int wm = wave >> 2, wn = wave & 3;
-
-  // ---- load stream
-  const int lrow = lane >> 3, lslot = lane & 7;
-  uint32_t ld_off[8];
-  int64_t ld_wbase = 0;
-  auto set_load_tile = [&](int lin) {  // the tile must be a used one
-    const int mt = lin / tiles_n, n0 = (lin - mt * tiles_n) * NOUT;
-    const int row0 = p.tile_row0[mt], rows = p.tile_rows[mt];
-    ld_wbase = (int64_t)p.tile_group[mt] * p.w_gstride;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int R = 8 * (wave + 8 * j) + lrow;
-      const int rr = row0 + min(R, rows - 1);
-      const int64_t sr = p.row_src ? (int64_t)p.row_src[rr] : (int64_t)rr;
-      ld_off[j] = (uint32_t)((sr * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
-      int col;
-      if constexpr (EPI == EPI_SWIGLU) col = n0 + 32 * (R >> 6) + 8 * ((R >> 4) & 3) + 4 * ((R >> 2) & 1) + (R & 3);
-      else col = n0 + R;
-      ld_off[4 + j] = (uint32_t)(((int64_t)min(col, N - 1) * p.ldw + (lslot ^ wd_swz_w(R)) * 8) * 2);
-    }
-  };
-  int ld_lin = first, ld_k = 0;
-  set_load_tile(ld_lin);
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)wd_lds + wave * 1024;
-  // weight rows 8 q .. 8 q + 7 of load instruction q = wave + 8 j: bit 3 of the row index, i.e. the
-  // parity of the wavefront, says gate or up
-  const bf16_t* wsrc = (EPI == EPI_SWIGLU && (wave & 1)) ? p.w2 : p.w;
-  auto issue_one = [&](int q, int stage) {
-    const uint32_t dst = lds0 + stage * WD_STAGE + (q >> 2) * WD_XBYTES + (q & 3) * 8192;
-    const bf16_t* base = (q < 4 ? p.x : wsrc + ld_wbase) + ld_k;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
-  };
-  auto advance_loads = [&]() {
-    ld_k += WD_BK;
-    if (ld_k >= K) {
-      ld_k = 0;
-      const int nl = ld_lin + G;
-      if (nl < tiles && p.tile_group[nl / tiles_n] >= 0) {
-        ld_lin = nl;
-        set_load_tile(ld_lin);
-      }
-    }
-  };
-
-  f32x4 acc[8][4];
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  const int xoff = (128 * wm + r16) * 128 + ((g ^ (r16 >> 1)) * 16);
-  const int woff = WD_XBYTES + (64 * wn + 16 * (r16 >> 2) + (r16 & 3)) * 128 +
-                   ((g ^ (((r16 >> 2) << 1) | ((r16 >> 1) & 1))) * 16);
-  struct Frag { uint4 w[4], x[8]; };
-  auto read_one = [&](Frag& f, int r, const uint8_t* sb, int ks) {
-    if (r < 4) f.w[r] = *(const uint4*)(sb + (woff ^ (64 * ks)) + r * 512);
-    else f.x[r - 4] = *(const uint4*)(sb + (xoff ^ (64 * ks)) + (r - 4) * 2048);
-  };
-  auto half_step = [&](const Frag& cur, Frag& nxt, const uint8_t* nxt_sb, int nxt_ks, auto LOADS,
-                       int ld_stage) {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) acc[i][j] = mfma16(cur.w[j], cur.x[i], acc[i][j]);
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (decltype(LOADS)::value) {
-        if (i < 4) {
-          issue_one(2 * i, ld_stage);
-          issue_one(2 * i + 1, ld_stage);
-        }
-      }
-      if (i < 4) {
-        read_one(nxt, 2 * i, nxt_sb, nxt_ks);
-        read_one(nxt, 2 * i + 1, nxt_sb, nxt_ks);
-      } else {
-        read_one(nxt, 4 + i, nxt_sb, nxt_ks);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  const int nk = K / WD_BK;
-  Frag f0, f1;
-#pragma unroll
-  for (int q = 0; q < 8; q++) issue_one(q, 0);
-  advance_loads();
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-#pragma unroll
-  for (int q = 0; q < 8; q++) issue_one(q, 1);
-  advance_loads();
-#pragma unroll
-  for (int r = 0; r < 12; r++) read_one(f0, r, wd_lds, 0);
-
-  int st = 0;
-  const bool vec_ok = (p.ldc & 7) == 0 && ((uintptr_t)p.c & 15) == 0;
-  for (int lin = first; lin < tiles; lin += G) {
-    const int mt = lin / tiles_n, n0 = (lin - mt * tiles_n) * NOUT;
-    if (p.tile_group[mt] < 0) break;
-    const int row0 = p.tile_row0[mt], rows = p.tile_rows[mt];
-    for (int kt = 0; kt < nk; kt++) {
-      const uint8_t* cur_sb = wd_lds + st * WD_STAGE;
-      const uint8_t* oth_sb = wd_lds + (st ^ 1) * WD_STAGE;
-      half_step(f0, f1, cur_sb, 1, std::false_type{}, 0);
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-      __syncthreads();
-      __builtin_amdgcn_sched_barrier(0);
-      half_step(f1, f0, oth_sb, 0, std::true_type{}, st);
-      advance_loads();
-      st ^= 1;
-    }
-
     if constexpr (EPI == EPI_SWIGLU) {
       // lane holds gate (fragments 0, 1) and up (2, 3) of columns n0 + 32 wn + 8 g + 4 j + c
-      const int nb = n0 + 32 * wn + 8 * g;
+      const int nb = t.n0 + 32 * wn + 8 * g;
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         const int m = 128 * wm + 16 * i + r16;
         float wr = 0.f;
-        if (m < rows) {
-          const int64_t orow = row0 + m;
+        if (m < t.rows) {
+          const int64_t orow = t.row0 + m;
           wr = bf16_to_f32(p.row_scale[p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow]);
         }
         bf16_t o[8];
@@ -381,8 +245,8 @@ __global__ __launch_bounds__(512) void gemm_wide_grouped_kernel(GemmParams p, in
             acc[i][j][c] = 0.f;
             acc[i][j + 2][c] = 0.f;
           }
-        if (m >= rows) continue;
-        bf16_t* cp = p.c + (int64_t)(row0 + m) * p.ldc + nb;
+        if (m >= t.rows) continue;
+        bf16_t* cp = p.c + (int64_t)(t.row0 + m) * p.ldc + nb;
         if (vec_ok && nb + 7 < N) {
           uint4 pk;
           pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
@@ -397,7 +261,13 @@ __global__ __launch_bounds__(512) void gemm_wide_grouped_kernel(GemmParams p, in
         }
       }
     } else {
-      const int nb = n0 + 64 * wn + 16 * g;
+      // lane holds C[row0 + 128 wm + 16 i + r16][n0 + 64 wn + 16 g + 4 j + c]
+      const int nb = t.n0 + 64 * wn + 16 * g;
+      float bv[16];
+      if (p.bias) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) bv[e] = bf16_to_f32(p.bias[min(nb + e, N - 1)]);
+      }
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         const int m = 128 * wm + 16 * i + r16;
@@ -406,11 +276,13 @@ __global__ __launch_bounds__(512) void gemm_wide_grouped_kernel(GemmParams p, in
         for (int j = 0; j < 4; j++)
 #pragma unroll
           for (int c = 0; c < 4; c++) {
-            o[4 * j + c] = f32_to_bf16(acc[i][j][c]);
+            float v = acc[i][j][c];
+            if (p.bias) v += bv[4 * j + c];
+            o[4 * j + c] = f32_to_bf16(v);
             acc[i][j][c] = 0.f;
           }
-        if (m >= rows) continue;
-        bf16_t* cp = p.c + (int64_t)(row0 + m) * p.ldc + nb;
+        if (m >= t.rows) continue;
+        bf16_t* cp = p.c + (int64_t)(t.row0 + m) * p.ldc + nb;
         if (vec_ok && nb + 15 < N) {
 #pragma unroll
           for (int h = 0; h < 2; h++) {
@@ -429,58 +301,46 @@ __global__ __launch_bounds__(512) void gemm_wide_grouped_kernel(GemmParams p, in
       }
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // loads past the last step still target our LDS
 }
 
-// Launches the grouped wide kernel for a 256-row tile table. x_rows = rows addressable in x
-// (bounds the 32-bit load offsets).
-static inline bool gemm_wide_grouped_launch(const GemmParams& p, int epi, int64_t max_m_tiles, int64_t x_rows,
-                                            hipStream_t stream) {
-  if (p.K % WD_BK != 0 || p.N <= 0 || max_m_tiles <= 0) return false;
+// Launch helper shared by the dense and the grouped entry points. x_rows = rows addressable in x
+// (bounds the 32-bit load offsets). Returns false (nothing launched) when the shape does not qualify.
+template <int EPI, bool GROUPED>
+static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int64_t x_rows, hipStream_t stream) {
+  constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;
+  if (p.K % WD_BK != 0 || p.N <= 0 || tiles_m <= 0 || x_rows <= 0) return false;
   const int64_t lim = (int64_t)1 << 32;
   if ((x_rows * p.ldx + p.K) * 2 >= lim || ((int64_t)p.N * p.ldw + p.K) * 2 >= lim) return false;
-  const int nout = epi == EPI_SWIGLU ? 128 : 256;
-  const int64_t tn = ((int64_t)p.N + nout - 1) / nout;
-  const int64_t tiles = max_m_tiles * tn;
+  const int64_t tn = ((int64_t)p.N + NOUT - 1) / NOUT;
+  const int64_t tiles = tiles_m * tn;
   if (tiles > (1 << 30)) return false;
-  static bool attr_set[2] = {false, false};
-  const void* fn = epi == EPI_SWIGLU ? (const void*)gemm_wide_grouped_kernel<EPI_SWIGLU>
-                                     : (const void*)gemm_wide_grouped_kernel<EPI_PLAIN>;
-  if (!attr_set[epi]) {
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, WD_LDS) != hipSuccess) {
-      (void)hipGetLastError();
-      return false;
-    }
-    attr_set[epi] = true;
-  }
-  const unsigned grid = (unsigned)(tiles >= 256 ? 256 : (tiles + 7) / 8 * 8);
-  if (epi == EPI_SWIGLU) gemm_wide_grouped_kernel<EPI_SWIGLU><<<grid, 512, WD_LDS, stream>>>(p, (int)max_m_tiles, (int)tn);
-  else gemm_wide_grouped_kernel<EPI_PLAIN><<<grid, 512, WD_LDS, stream>>>(p, (int)max_m_tiles, (int)tn);
-  return true;
-}
-
-// Launches the wide kernel. Returns false (nothing launched) when the shape does not qualify.
-static inline bool gemm_wide_launch(const GemmParams& p, hipStream_t stream) {
-  if (p.K % WD_BK != 0 || p.M <= 0 || p.N <= 0) return false;
-  const int64_t lim = (int64_t)1 << 32;
-  if (((int64_t)p.M * p.ldx + p.K) * 2 >= lim || ((int64_t)p.N * p.ldw + p.K) * 2 >= lim) return false;
-  static bool attr_set = false;  // per process; the attribute is a property of the loaded function
+  static bool attr_set = false;  // per process and instantiation; a property of the loaded function
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)gemm_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            WD_LDS) != hipSuccess) {
+    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, GROUPED>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, WD_LDS) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
     attr_set = true;
   }
-  const int64_t tm = ((int64_t)p.M + WD_BM - 1) / WD_BM, tn = ((int64_t)p.N + WD_BN - 1) / WD_BN;
-  const int64_t tiles = tm * tn;
-  if (tiles > (1 << 30)) return false;
   const unsigned grid = (unsigned)(tiles >= 256 ? 256 : (tiles + 7) / 8 * 8);
-  gemm_wide_kernel<<<grid, 512, WD_LDS, stream>>>(p, (int)tm, (int)tn);
+  gemm_wide_kernel<EPI, GROUPED><<<grid, 512, WD_LDS, stream>>>(p, (int)tiles_m, (int)tn);
   return true;
 }
 
+// dense: C[M, N] = X W^T (+ bias)
+static inline bool gemm_wide_launch(const GemmParams& p, hipStream_t stream) {
+  if (p.M <= 0) return false;
+  return gemm_wide_launch_t<EPI_PLAIN, false>(p, ((int64_t)p.M + WD_BM - 1) / WD_BM, p.M, stream);
+}
+
+// grouped, over a 256-row tile table of max_m_tiles entries
+static inline bool gemm_wide_grouped_launch(const GemmParams& p, int epi, int64_t max_m_tiles, int64_t x_rows,
+                                            hipStream_t stream) {
+  if (epi == EPI_SWIGLU) return gemm_wide_launch_t<EPI_SWIGLU, true>(p, max_m_tiles, x_rows, stream);
+  return gemm_wide_launch_t<EPI_PLAIN, true>(p, max_m_tiles, x_rows, stream);
+}
 
 // ---------------------------------------------------------------------------------------
 // Ring kernel for a few hundred rows (decode-sized batches against dense weights), where one
