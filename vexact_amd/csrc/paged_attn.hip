@@ -107,6 +107,68 @@ struct KVSource {
   }
 };
 
+// Online-softmax update of one 16-query tile from the raw score tiles st (S^T: lane holds keys
+// kb + 16 tt + 4 g + r of query column r16) of the 64-key block at kb: masks keys past qpos, updates
+// the running max m and sum l, rescales the NACC accumulators and packs P (rounded to bf16; the sum
+// uses the rounded values) as the two B operands of the P V MFMAs. Shared by every attention kernel.
+template <int NACC>
+__device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float c, int qpos, float& m, float& l,
+                                                  f32x4 (&acc)[NACC], uint4 (&pf)[2], bool all_visible = false) {
+  const int lane = threadIdx.x & 63, g = lane >> 4;
+  float bm = -INFINITY;
+  if (all_visible) {  // wave-uniform: every key of the block is visible to every row of the tile
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        st[tt][r] = st[tt][r] * c;
+        bm = fmaxf(bm, st[tt][r]);
+      }
+  } else {
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int key = kb + 16 * tt + 4 * g + r;
+        float tv = st[tt][r] * c;
+        tv = (key <= qpos) ? tv : -INFINITY;
+        st[tt][r] = tv;
+        bm = fmaxf(bm, tv);
+      }
+  }
+  bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+  bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+  const float mn = fmaxf(m, bm);
+  const float ms = (mn == -INFINITY) ? 0.f : mn;  // fully masked so far: everything stays 0
+  const float alpha = fast_exp2(m - ms);
+  float rs = 0.f;
+  uint32_t pw[4][2];
+#pragma unroll
+  for (int tt = 0; tt < 4; tt++) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      // two probabilities rounded to bf16 at once; the row sum adds the rounded values
+      const uint32_t pk = pack_bf16x2(fast_exp2(st[tt][2 * h] - ms), fast_exp2(st[tt][2 * h + 1] - ms));
+      rs += bf16lo(pk);
+      rs += bf16hi(pk);
+      pw[tt][h] = pk;
+    }
+  }
+  rs += __shfl_xor(rs, 16, 64);
+  rs += __shfl_xor(rs, 32, 64);
+  l = l * alpha + rs;
+  m = mn;
+  // multiplying by exactly 1 changes nothing: skip the rescale when no lane's maximum moved
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+    for (int i = 0; i < NACC; i++) {
+      acc[i][0] *= alpha; acc[i][1] *= alpha; acc[i][2] *= alpha; acc[i][3] *= alpha;
+    }
+  }
+  pf[0] = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
+  pf[1] = make_uint4(pw[2][0], pw[2][1], pw[3][0], pw[3][1]);
+}
+
 template <int DK, int DV, int QT>
 struct AttnWave {
   static constexpr int KS = DK / 32;           // MFMA k-steps for S
@@ -167,7 +229,6 @@ struct AttnWave {
 
   // scores of the 64-key block at kb from kf, online-softmax update, P packed for the PV MFMAs
   __device__ __forceinline__ void scores(int kb, float c, uint4 (&pf)[QT][2]) {
-    const int lane = threadIdx.x & 63, g = lane >> 4;
 #pragma unroll
     for (int t = 0; t < QT; t++) {
       // S^T tiles: lane holds keys kb + 16 tt + 4 g + r for query column r16
@@ -178,47 +239,13 @@ struct AttnWave {
 #pragma unroll
         for (int s = 0; s < KS; s++) st[tt] = mfma16(kf[tt][s], qf[t][s], st[tt]);
       }
-      float bm = -INFINITY;
-#pragma unroll
-      for (int tt = 0; tt < 4; tt++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const int key = kb + 16 * tt + 4 * g + r;
-          float tv = st[tt][r] * c;
-          tv = (key <= qpos[t]) ? tv : -INFINITY;
-          st[tt][r] = tv;
-          bm = fmaxf(bm, tv);
-        }
-      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
-      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-      const float mn = fmaxf(m[t], bm);
-      const float ms = (mn == -INFINITY) ? 0.f : mn;  // fully masked so far: everything stays 0
-      const float alpha = fast_exp2(m[t] - ms);
-      float rs = 0.f;
-      uint32_t pw[4][2];
-#pragma unroll
-      for (int tt = 0; tt < 4; tt++) {
-        float pv[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const bf16_t pb = f32_to_bf16(fast_exp2(st[tt][r] - ms));
-          pv[r] = bf16_to_f32(pb);
-          rs += pv[r];
-        }
-        pw[tt][0] = pack_bf16x2(pv[0], pv[1]);
-        pw[tt][1] = pack_bf16x2(pv[2], pv[3]);
-      }
-      rs += __shfl_xor(rs, 16, 64);
-      rs += __shfl_xor(rs, 32, 64);
-      l[t] = l[t] * alpha + rs;
-      m[t] = mn;
-#pragma unroll
-      for (int i = 0; i < NACC; i++) {
-        acc[t][i][0] *= alpha; acc[t][i][1] *= alpha; acc[t][i][2] *= alpha; acc[t][i][3] *= alpha;
-      }
-      pf[t][0] = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
-      pf[t][1] = make_uint4(pw[2][0], pw[2][1], pw[3][0], pw[3][1]);
+      softmax_tile(t, st, kb, c, pf);
     }
+  }
+
+  // online-softmax update of q-tile t from the raw score tiles st of the 64-key block at kb
+  __device__ __forceinline__ void softmax_tile(int t, f32x4 (&st)[4], int kb, float c, uint4 (&pf)[QT][2]) {
+    attn_softmax_tile(st, kb, c, qpos[t], m[t], l[t], acc[t], pf[t]);
   }
 
   // acc += P V with the block's values in vr. Values of keys past the end are zeroed first (their
@@ -559,28 +586,41 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
 // wavefront v owns query rows [64 QT bx + 16 QT v, +16 QT) of the sequence (local indices).
 // ---------------------------------------------------------------------------------------
 template <int DK, int DV, int QT, int KIND>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
-  const int head = blockIdx.y, seq = blockIdx.z;
+__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw) {
+  // The 4 * QT query tiles (16 rows each) of a block are spread over hpw query heads of one kv head
+  // and 4 * QT / hpw row tiles: tile slot s = wave * QT + t -> head s % hpw, row tile s / hpw. With
+  // hpw > 1 the wavefronts of a block walk the same keys at the same time, so K and V mostly come
+  // from the CU's L1 after the first wavefront has fetched them.
+  const int seq = blockIdx.z;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   int kv_len, k0 = 0;
   if constexpr (KIND != SRC_PACKED) kv_len = p.seqused_k[seq];
   else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-  const int i0 = (blockIdx.x * 4 + wave) * 16 * QT;
-  if (qlen <= 0 || kv_len <= 0 || i0 >= qlen) return;
-  const int kvh = head / (p.Hq / p.Hkv);
+  const int rows_per_block = 16 * (4 * QT / hpw);
+  int head_of[QT], i0_of[QT];
+  bool any = false;
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int s = wave * QT + t;
+    head_of[t] = blockIdx.y * hpw + s % hpw;
+    i0_of[t] = blockIdx.x * rows_per_block + 16 * (s / hpw);
+    any = any || i0_of[t] < qlen;
+  }
+  if (qlen <= 0 || kv_len <= 0 || !any) return;
+  const int kvh = head_of[0] / (p.Hq / p.Hkv);  // all heads of a block share the kv head
   const int shift = kv_len - qlen;  // absolute position of local row 0
 
   AttnWave<DK, DV, QT> w;
   int maxpos = -1;
 #pragma unroll
   for (int t = 0; t < QT; t++) {
-    const int i = i0 + 16 * t + r16;
+    const int i = i0_of[t] + r16;
     const bool ok = i < qlen;
     const int pos = p.causal ? shift + i : kv_len - 1;
     w.qpos[t] = (ok && pos >= 0) ? pos : -1;
-    const bf16_t* qp = p.q + (int64_t)(q0 + (ok ? i : 0)) * p.sqt + (int64_t)head * p.sqh + 8 * g;
+    const bf16_t* qp = p.q + (int64_t)(q0 + (ok ? i : 0)) * p.sqt + (int64_t)head_of[t] * p.sqh + 8 * g;
 #pragma unroll
     for (int s = 0; s < DK / 32; s++) w.qf[t][s] = ldg16(qp + 32 * s, ok);
     maxpos = max(maxpos, w.qpos[t]);
@@ -616,9 +656,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
 
 #pragma unroll
   for (int t = 0; t < QT; t++) {
-    const int i = i0 + 16 * t + r16;
+    const int i = i0_of[t] + r16;
     if (i >= qlen) continue;
-    bf16_t* op = p.o + (int64_t)(q0 + i) * p.sot + (int64_t)head * p.soh;
+    bf16_t* op = p.o + (int64_t)(q0 + i) * p.sot + (int64_t)head_of[t] * p.soh;
     const bool dead = w.qpos[t] < 0;  // no visible key: define the output as 0
 #pragma unroll
     for (int ds = 0; ds < (DV + 127) / 128; ds++)
@@ -636,6 +676,233 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
           *(uint4*)(op + d0) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
         }
       }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// General kernel for head size 128, K and V through LDS. Same tile slots as attn_prefill_kernel
+// (4 wavefronts x 2 query tiles spread over hpw heads of one kv head), but every 64-key block is
+// brought in once per workgroup by direct-to-LDS loads (no staging registers) into one of two
+// 32 KB stages, and all wavefronts take their operands from there:
+//   * rows are 256 bytes; 16-byte piece c of key row r is stored at piece c ^ (r & 15), which makes
+//     both kinds of read below conflict free;
+//   * S: the A operand (16 keys x 32 dims) is a 16-byte read per lane, as from global memory before;
+//   * P V: the A operand (16 dims x 32 keys) comes from two transposing reads (ds_read_b64_tr_b16):
+//     the 16 lanes of a group address 4 keys x 16 dims in 8-byte pieces and each lane receives one
+//     dim of those 4 keys. Lane (r16, g) of fragment f ends up with dim 16 f + r16 for the keys
+//     16 (idx / 4) + 4 g + idx % 4 of k-slot idx = the slot order of P in AttnWave::scores, so no
+//     register transposes are needed. The accumulator of fragment f holds dims 16 f + 4 g + r.
+// Scores, softmax, chunk folding are the code of AttnWave; each output element sees the same operand
+// values in the same MFMA k-slots as in the other attention kernels, so the bits are the same.
+// ---------------------------------------------------------------------------------------
+typedef short v4s_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+constexpr int PFL_WAVES = 8, PFL_QT = 2, PFL_SLOTS = PFL_WAVES * PFL_QT;  // 16 query tiles per block
+constexpr int PFL_STAGE = 2 * ATT_BLOCK * 256;                             // K block, then V block
+constexpr int PFL_NS = 3;                                                   // K/V stages in flight
+constexpr int PFL_LDS = PFL_NS * PFL_STAGE + PFL_SLOTS * 16 * 256;         // stages + the query tiles = 160 KB
+
+template <int KIND>
+__global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnParams p, int hpw) {
+  constexpr int D = 128, QT = PFL_QT, KS = D / 32;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t pf_lds[];
+
+  const int seq = blockIdx.z;
+  const int q0 = p.cu_q[seq];
+  const int qlen = p.cu_q[seq + 1] - q0;
+  int kv_len, k0 = 0;
+  if constexpr (KIND != SRC_PACKED) kv_len = p.seqused_k[seq];
+  else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int rows_per_block = 16 * (PFL_SLOTS / hpw);
+  const int i_base = blockIdx.x * rows_per_block;
+  if (qlen <= 0 || kv_len <= 0 || i_base >= qlen) return;  // uniform over the block
+  const int shift = kv_len - qlen;  // absolute position of local row 0
+  // last key any row of the block may see (uniform): every wavefront walks the blocks up to it
+  const int blk_maxpos = p.causal ? shift + min(i_base + rows_per_block, qlen) - 1 : kv_len - 1;
+  if (blk_maxpos < 0) {  // no visible key for any row: outputs are defined as 0
+    for (int e = threadIdx.x; e < rows_per_block * hpw * (D / 8); e += 64 * PFL_WAVES) {
+      const int row = i_base + e / (hpw * (D / 8)), rem = e % (hpw * (D / 8));
+      if (row < qlen)
+        *(uint4*)(p.o + (int64_t)(q0 + row) * p.sot + (int64_t)(blockIdx.y * hpw + rem / (D / 8)) * p.soh +
+                  8 * (rem % (D / 8))) = make_uint4(0, 0, 0, 0);
+    }
+    return;
+  }
+
+  int head_of[QT], i0_of[QT];
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int s = wave * QT + t;
+    head_of[t] = blockIdx.y * hpw + s % hpw;
+    i0_of[t] = i_base + 16 * (s / hpw);
+  }
+  const int kvh = (blockIdx.y * hpw) / (p.Hq / p.Hkv);
+
+  // ---- this wavefront's query tiles go to its own LDS region (read back every block, which frees
+  // 32 registers); piece c of row r at piece c ^ r, like the key rows
+  uint8_t* qs = pf_lds + PFL_NS * PFL_STAGE + wave * (QT * 16 * 256);
+  int qpos[QT];
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int i = i0_of[t] + r16;
+    const bool ok = i < qlen;
+    const int pos = p.causal ? shift + i : kv_len - 1;
+    qpos[t] = (ok && pos >= 0) ? pos : -1;
+    const bf16_t* qp = p.q + (int64_t)(q0 + (ok ? i : 0)) * p.sqt + (int64_t)head_of[t] * p.sqh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < KS; s++)
+      *(uint4*)(qs + (16 * t + r16) * 256 + (((4 * s + g) ^ r16) * 16)) = ldg16(qp + 32 * s, ok);
+  }
+  // smallest last-visible key over the rows of each tile (wave-uniform; -1 if a row is not valid):
+  // blocks that end at or before it need no masking
+  int qpos_min[QT];
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    int v = qpos[t];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+    qpos_min[t] = v;
+  }
+
+  float m[QT], l[QT], M[QT], L[QT];
+  f32x4 acc[QT][8], ACC[QT][8];
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    M[t] = -INFINITY; L[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) ACC[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const KVSource<KIND> src = make_source<KIND>(p, seq, kvh, k0, kv_len);
+  // ---- loads: wavefront v brings in keys [8 v, 8 v + 8) of a block, K and V, 4 keys (1 KB) per
+  // instruction; lane l writes slot l % 16 of its key row and therefore fetches logical piece
+  // (l % 16) ^ (row & 15)
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)pf_lds;
+  auto issue_block = [&](int kb, int stage) {
+    const typename KVSource<KIND>::Tiles tl = src.tiles(kb);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int row = 8 * wave + 4 * j + (lane >> 4);  // key row inside the block
+      const int tt = row >> 4, within = row & 15;
+      const bool ok = kb + row < kv_len;
+      const int piece = (lane & 15) ^ (row & 15);
+      const bf16_t* kp = src.krow(tl, kb, tt, ok ? within : 0) + 8 * piece;
+      const bf16_t* vp = src.vrow(tl, kb, tt, ok ? within : 0) + 8 * piece;
+      const uint32_t dst = lds0 + stage * PFL_STAGE + (8 * wave + 4 * j) * 256;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :: "s"(dst), "v"(kp) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :: "s"(dst + ATT_BLOCK * 256), "v"(vp) : "memory", "m0");
+    }
+  };
+
+  auto block_compute = [&](int kb, int stage) {
+    const uint8_t* ks = pf_lds + stage * PFL_STAGE;
+    const uint8_t* vs = ks + ATT_BLOCK * 256;
+    // ---- S^T = K Q^T: the key fragments are shared by both query tiles; per accumulator the k-steps
+    // run in ascending order as everywhere else
+    f32x4 st[QT][4];
+#pragma unroll
+    for (int t = 0; t < QT; t++)
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) st[t][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      uint4 qfr[QT];
+#pragma unroll
+      for (int t = 0; t < QT; t++) qfr[t] = *(const uint4*)(qs + (16 * t + r16) * 256 + (((4 * s + g) ^ r16) * 16));
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) {
+        const int row = 16 * tt + r16;
+        const uint4 kfr = *(const uint4*)(ks + row * 256 + (((4 * s + g) ^ (row & 15)) * 16));
+#pragma unroll
+        for (int t = 0; t < QT; t++) st[t][tt] = mfma16(kfr, qfr[t], st[t][tt]);
+      }
+    }
+    uint4 pf[QT][2];
+#pragma unroll
+    for (int t = 0; t < QT; t++)
+      attn_softmax_tile(st[t], kb, p.qk_scale, qpos[t], m[t], l[t], acc[t], pf[t], kb + ATT_BLOCK - 1 <= qpos_min[t]);
+    // ---- P V. For k-slots idx = 0..3 (first read) and 4..7 (second) of 32-key chunk ch, addressing
+    // lane i = r16 of group g points at key 32 ch + 16 (idx / 4) + 4 g + i / 4, dims 16 f + 4 (i % 4) .. +3
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++) {
+#pragma unroll
+      for (int f = 0; f < 8; f++) {
+        const int byte = 32 * f + 8 * (r16 & 3);
+        const int row_lo = 32 * ch + 4 * g + (r16 >> 2), row_hi = row_lo + 16;
+        const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) v4s_t*)(vs + row_lo * 256 + (((byte >> 4) ^ (row_lo & 15)) * 16) + (byte & 15)));
+        const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) v4s_t*)(vs + row_hi * 256 + (((byte >> 4) ^ (row_hi & 15)) * 16) + (byte & 15)));
+        uint4 vf;
+        vf.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+        vf.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+        vf.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+        vf.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+#pragma unroll
+        for (int t = 0; t < QT; t++) acc[t][f] = mfma16(vf, pf[t][ch], acc[t][f]);
+      }
+    }
+  };
+
+  const int nblk = blk_maxpos / ATT_BLOCK + 1;
+#pragma unroll
+  for (int i = 0; i < PFL_NS; i++)
+    if (i < nblk) issue_block(i * ATT_BLOCK, i);
+  int stage = 0;
+  for (int b = 0; b < nblk; b++) {
+    const int kb = b * ATT_BLOCK;
+    if ((kb & (ATT_CHUNK - 1)) == 0) {
+#pragma unroll
+      for (int t = 0; t < QT; t++) {
+        m[t] = -INFINITY; l[t] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    // block b has landed; the 4 loads each of up to PFL_NS - 1 later blocks may still be in flight
+    const int ahead = min(PFL_NS - 1, nblk - 1 - b);
+    if (ahead >= 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (ahead == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    block_compute(kb, stage);
+    __syncthreads();  // everyone is done with this stage
+    if (b + PFL_NS < nblk) issue_block(kb + PFL_NS * ATT_BLOCK, stage);
+    stage = stage + 1 == PFL_NS ? 0 : stage + 1;
+    if (((kb + ATT_BLOCK) & (ATT_CHUNK - 1)) == 0 || b + 1 == nblk) {
+#pragma unroll
+      for (int t = 0; t < QT; t++) {
+        float Mn, A, B;
+        fold_scales(M[t], m[t], Mn, A, B);
+        L[t] = L[t] * A + l[t] * B;
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) ACC[t][i][r] = ACC[t][i][r] * A + acc[t][i][r] * B;
+        M[t] = Mn;
+      }
+    }
+  }
+
+  // lane (r16 = query row, g) holds dims 16 f + 4 g + r of fragment f
+#pragma unroll
+  for (int t = 0; t < QT; t++) {
+    const int i = i0_of[t] + r16;
+    if (i >= qlen) continue;
+    bf16_t* op = p.o + (int64_t)(q0 + i) * p.sot + (int64_t)head_of[t] * p.soh;
+    const bool dead = qpos[t] < 0;
+#pragma unroll
+    for (int f = 0; f < 8; f++) {
+      uint2 pk;
+      pk.x = pack_bf16x2(dead ? 0.f : ACC[t][f][0] / L[t], dead ? 0.f : ACC[t][f][1] / L[t]);
+      pk.y = pack_bf16x2(dead ? 0.f : ACC[t][f][2] / L[t], dead ? 0.f : ACC[t][f][3] / L[t]);
+      *(uint2*)(op + 16 * f + 4 * g) = pk;
+    }
   }
 }
 
@@ -722,10 +989,37 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
   } else {
     constexpr int QT = (DK > 128) ? 1 : 2;
     const int rows = max_q > 0 ? max_q : total_q;
-    dim3 grid((rows + 64 * QT - 1) / (64 * QT), p.Hq, p.num_seqs);
-    if (mode == 2) attn_prefill_kernel<DK, DV, QT, SRC_PACKED><<<grid, 256, 0, stream>>>(p);
-    else if (fast) attn_prefill_kernel<DK, DV, QT, SRC_FAST><<<grid, 256, 0, stream>>>(p);
-    else attn_prefill_kernel<DK, DV, QT, SRC_GENERIC><<<grid, 256, 0, stream>>>(p);
+    // query heads of one kv head that share a block (a divisor of the group size and of the 4 * QT
+    // tile slots)
+    const int G = p.Hq / p.Hkv;
+    int hpw = 1;
+    while (hpw * 2 <= 4 * QT && G % (hpw * 2) == 0) hpw *= 2;
+    const int rpb = 16 * (4 * QT / hpw);
+    dim3 grid((rows + rpb - 1) / rpb, p.Hq / hpw, p.num_seqs);
+    if constexpr (DK == 128 && DV == 128) {
+      // K and V through LDS, shared by the 16 query tiles of a block
+      int hp = 1;
+      while (hp * 2 <= 8 && G % (hp * 2) == 0) hp *= 2;
+      const int rb = 16 * (PFL_SLOTS / hp);
+      const dim3 lgrid((rows + rb - 1) / rb, p.Hq / hp, p.num_seqs);
+      static bool attr_set = false;
+      if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<SRC_PACKED>, hipFuncAttributeMaxDynamicSharedMemorySize, PFL_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<SRC_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, PFL_LDS) != hipSuccess ||
+            hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<SRC_GENERIC>, hipFuncAttributeMaxDynamicSharedMemorySize, PFL_LDS) != hipSuccess) {
+          (void)hipGetLastError();
+          return VX_ERR_LAUNCH;
+        }
+        attr_set = true;
+      }
+      if (mode == 2) attn_prefill_lds_kernel<SRC_PACKED><<<lgrid, 64 * PFL_WAVES, PFL_LDS, stream>>>(p, hp);
+      else if (fast) attn_prefill_lds_kernel<SRC_FAST><<<lgrid, 64 * PFL_WAVES, PFL_LDS, stream>>>(p, hp);
+      else attn_prefill_lds_kernel<SRC_GENERIC><<<lgrid, 64 * PFL_WAVES, PFL_LDS, stream>>>(p, hp);
+      return launch_status();
+    }
+    if (mode == 2) attn_prefill_kernel<DK, DV, QT, SRC_PACKED><<<grid, 256, 0, stream>>>(p, hpw);
+    else if (fast) attn_prefill_kernel<DK, DV, QT, SRC_FAST><<<grid, 256, 0, stream>>>(p, hpw);
+    else attn_prefill_kernel<DK, DV, QT, SRC_GENERIC><<<grid, 256, 0, stream>>>(p, hpw);
   }
   return launch_status();
 }

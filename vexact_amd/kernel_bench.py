@@ -176,6 +176,30 @@ def main() -> None:
         report(f"prefill attention {S} x {Lp} tokens",
                timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, bt, D**-0.5, Lp, out=out), n_layers=2),
                flops=4 * S * Hq * D * Lp * (Lp + 1) // 2)
+    if "prefill" in what:
+        # chunked prefill: 16 sequences, a 512-token chunk on a cached prefix of 0..8192 tokens, Hq=32, Hkv=8
+        Hq, Hkv, D, page, S, C = 32, 8, 128, 16, 16, 512
+        rng = np.random.default_rng(3)
+        prefix = rng.integers(0, 8193, size=S)
+        Ls = prefix + C
+        pages = [(int(n) + page - 1) // page for n in Ls]
+        pool = sum(pages)
+        perm = rng.permutation(pool)
+        bt = np.full((S, max(pages)), -1, np.int32)
+        o = 0
+        for i, pg in enumerate(pages):
+            bt[i, :pg] = perm[o : o + pg]
+            o += pg
+        kc = rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3)
+        vc = rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3)
+        q = rnd(S * C, Hq, D, std=1.0)
+        cu = torch.arange(0, S * C + 1, C, dtype=torch.int32, device=dev)
+        used = torch.tensor(Ls, dtype=torch.int32, device=dev)
+        btd = torch.tensor(bt, device=dev)
+        out = torch.empty(S * C, Hq, D, dtype=torch.bfloat16, device=dev)
+        fl = 4 * Hq * D * int(sum(C * int(pf) + C * (C + 1) // 2 for pf in prefix))
+        report(f"chunked prefill attention 16 x 512 on prefixes (sum L={int(Ls.sum())})",
+               timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, btd, D**-0.5, C, out=out), n_layers=2), flops=fl)
     if "small" in what:
         one = torch.zeros(64, dtype=torch.int32, device=dev)
         lib = _lib.load()
