@@ -838,11 +838,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
             (__attribute__((address_space(3))) v4s_t*)(vs + row_lo * 256 + (((byte >> 4) ^ (row_lo & 15)) * 16) + (byte & 15)));
         const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) v4s_t*)(vs + row_hi * 256 + (((byte >> 4) ^ (row_hi & 15)) * 16) + (byte & 15)));
-        uint4 vf;
-        vf.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-        vf.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-        vf.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-        vf.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+        const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+        const uint4 vf = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
 #pragma unroll
         for (int t = 0; t < QT; t++) acc[t][f] = mfma16(vf, pf[t][ch], acc[t][f]);
       }
