@@ -166,7 +166,7 @@ def test_fused_moe_batch_invariance_reference_shapes(batch_size, seq_len, H, I, 
 
 
 def test_fused_moe_rows_do_not_depend_on_token_count():
-    # same rows at T = 1, 64, 256 (streaming tiles) and 1100, 4096 (64- and 128-row tiles)
+    # same rows at T = 1, 64, 256 (streaming tiles), 1100 (128-row tiles) and 4096 (256-row tiles)
     T, H, I, E, k = 4096, 512, 256, 32, 4
     x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=13)
     xg, wg, sg, gg, ug, dg = (t.cuda() for t in (x, w, sel, gate, up, down))

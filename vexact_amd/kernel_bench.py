@@ -226,6 +226,58 @@ def main() -> None:
                2 * B * 5120 * 2)
         logits = rnd(B, 151936, std=1.0)
         report("greedy token + logprob", timeit(lambda li: ops.logprobs(logits, None, return_tokens=True)), B * 151936 * 2)
+    if "configs" in what:
+        # ---- the reference's other benchmark configurations, at their own shapes
+        # C1: RMSNorm -> lm_head GEMM -> fp32 log_softmax on M rows (Qwen3-1.7B op chain)
+        V = 151936
+        wl = rnd(V, H)
+        wn = rnd(H, std=1.0)
+        for M in (1, 7, 64):
+            x = rnd(M, H, std=1.0)
+            hn = torch.empty_like(x)
+            lg = torch.empty(M, V, dtype=torch.bfloat16, device=dev)
+            report(f"C1 lm_head gemm M={M}", timeit(lambda li: ops.gemm_nt(x, wl, out=lg), n_layers=2), 2 * (V * H + M * H + M * V))
+            lf = lg.float()
+            report(f"C1 log_softmax fp32 M={M}", timeit(lambda li: ops.log_softmax(lf), n_layers=2), 2 * M * V * 4)
+            report(f"C1 rms_norm M={M}", timeit(lambda li: ops.rms_norm(x, wn, 1e-6, hf_two_rounding=True, out=hn), n_layers=2),
+                   2 * M * H * 2 + 2 * H)
+        del wl
+        # C2: decode attention, 64 sequences, context 128..4096, Hq=16, Hkv=8, D=128, page 16
+        Hq, Hkv, D, page, S = 16, 8, 128, 16, 64
+        rng = np.random.default_rng(2)
+        L = rng.integers(128, 4097, size=S)
+        pages = [(int(n) + page - 1) // page for n in L]
+        pool = 32768
+        perm = rng.permutation(pool)
+        bt = np.full((S, 256), -1, np.int32)
+        o = 0
+        for i, pg in enumerate(pages):
+            bt[i, :pg] = perm[o : o + pg]
+            o += pg
+        kc = rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3)
+        vc = rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3)
+        q = rnd(S, Hq, D, std=1.0)
+        cu = torch.arange(S + 1, dtype=torch.int32, device=dev)
+        used = torch.tensor(L, dtype=torch.int32, device=dev)
+        btd = torch.tensor(bt, device=dev)
+        out = torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev)
+        report(f"C2 decode attention B=64 (sum L={int(L.sum())})",
+               timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, btd, D**-0.5, 1, out=out), n_layers=2),
+               int(L.sum()) * 2 * Hkv * D * 2 + 2 * S * Hq * D * 2 + sum(pages) * 4)
+        del kc, vc
+        # C4: fused MoE block at T tokens
+        gu = rnd(E, 2 * I, H + 64)[..., :H]
+        dn = rnd(E, H, I)
+        for T in (1, 64, 256, 4096):
+            x = rnd(T, H, std=1.0)
+            logits = torch.randn(T, E, generator=g, device=dev)
+            w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
+            U = int(torch.unique(idx).numel())
+            y = torch.empty_like(x)
+            t = timeit(lambda li: ops.fused_moe(x, w, idx, gu[:, :I, :], gu[:, I:, :], dn, E, out=y), n_layers=2)
+            report(f"C4 fused MoE T={T} ({U} experts)", t, U * 3 * H * I * 2 + 2 * T * H * 2 + T * k * 6)
+            if T == 4096 and t is not None:
+                print(f"{'':34s} = {T * k * 6 * H * I / t / 1e12:.1f} TFLOP/s", flush=True)
     if "copy" in what:
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()

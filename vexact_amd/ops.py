@@ -453,7 +453,7 @@ def moe_tile_rows(num_tokens: int, wide_ok: bool = True) -> int:
         return 32
     if num_tokens <= 1024:
         return 64
-    if num_tokens < 8192 or not wide_ok:
+    if num_tokens < 2048 or not wide_ok:
         return 128
     return 256
 
