@@ -102,9 +102,8 @@ def main():
             tot += len(prompts[s])
             s += 1
         reqs = [dict(num_computed_tokens=len(prompts[i]), tokens_this_step=len(prompts[i]), block_ids=blocks[i]) for i in grp]
-        meta = build_step_metadata(reqs, cfg.page_size, max_blocks)
-        pb.load(meta, np.concatenate([prompts[i] for i in grp]))
-        dec.step(pb, meta["max_seqlen_q"])
+        _, _, max_q = pb.load_requests(reqs, np.concatenate([prompts[i] for i in grp]), cfg.page_size)
+        dec.step(pb, max_q)
         first_tokens[grp] = pb.tokens[: len(grp)].cpu().numpy()
     torch.cuda.synchronize()
     print(f"[bench] prefill of {int(prompt_lens.sum())} tokens: {time.time() - t0:.1f}s", file=sys.stderr, flush=True)

@@ -190,6 +190,36 @@ int vx_embedding(const void* table, const void* ids, int ids_i64, void* out, int
                  int64_t vocab, hipStream_t stream);
 int vx_fill_i32(int* p, int value, int64_t n, hipStream_t stream);
 
+/* ---- host-side step metadata and block allocator (CPU code, no device work, no stream) -------- */
+
+/* Integer metadata of one step, written into host buffers sized for a graph bucket (cap_tokens
+ * tokens, cap_seqs sequences): positions [cap_tokens] (int64), slot_mapping [cap_tokens],
+ * query_start_loc [cap_seqs + 1], context_lens [cap_seqs], block_tables [cap_seqs, max_blocks].
+ * Request s has context length num_computed[s] AFTER this step, tokens_this_step[s] query tokens
+ * and the block ids block_ids[block_offsets[s] .. block_offsets[s + 1]). Padding: tokens past the
+ * step get slot -1 / position 0; sequences past it get query_start_loc = total tokens, context
+ * length 0 and an all-zero block-table row; unused entries of real rows are -1.
+ * Replaces _prepare_gen_ctx (vexact/inferencer/inferencer.py:193-291) and the static-buffer padding
+ * of prepare_cudagraph_gen_ctx (inferencer.py:306-324) in one pass. VX_ERR_ARG if the step does not
+ * fit the bucket or a request's blocks do not cover its context. */
+int vx_host_step_metadata(int64_t num_reqs, const int64_t* num_computed, const int64_t* tokens_this_step,
+                          const int32_t* block_ids, const int64_t* block_offsets, int32_t page_size,
+                          int64_t max_blocks, int64_t cap_tokens, int64_t cap_seqs, int64_t* positions,
+                          int32_t* slot_mapping, int32_t* query_start_loc, int32_t* context_lens,
+                          int32_t* block_tables, int64_t* total_tokens, int32_t* max_seqlen_q);
+
+/* Block allocator that always hands out the lowest free ids (KVCacheManager,
+ * vexact/batch_invariant_ops/kv_cache_context.py:141-217). allocate: the blocks a request holding
+ * num_current_blocks needs to cover total_tokens, ascending, into out; returns their number, 0 if
+ * none are needed, -1 (nothing allocated) if too few are free or out_capacity is too small.
+ * free: ids out of range or already free are ignored; returns the number freed. Not thread-safe. */
+void* vx_kv_allocator_create(int64_t num_blocks);
+void vx_kv_allocator_destroy(void* allocator);
+int64_t vx_kv_allocator_num_free(const void* allocator);
+int64_t vx_kv_allocator_allocate(void* allocator, int64_t total_tokens, int64_t num_current_blocks,
+                                 int32_t page_size, int32_t* out, int64_t out_capacity);
+int64_t vx_kv_allocator_free(void* allocator, const int32_t* ids, int64_t n);
+
 #ifdef __cplusplus
 }
 #endif

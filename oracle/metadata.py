@@ -61,3 +61,33 @@ def pad_for_graph_ref(ctx, capture_tokens: int, graph_num_seqs: int):
     qsl[B + 1 :] = T
     return {"slot_mapping": slot, "positions": pos, "context_lens": lens, "block_tables": bt,
             "query_start_loc": qsl, "max_seqlen_q": ctx["max_seqlen_q"]}
+
+
+class BlockAllocatorRef:
+    """Scan-based restatement of the block allocator (vexact/batch_invariant_ops/kv_cache_context.py:
+    141-217): a set of free ids, ``min`` of it per allocated block, frees only ids it handed out."""
+
+    def __init__(self, num_blocks: int, page_size: int):
+        self.page_size = page_size
+        self.allocated = set()
+        self.free = set(range(num_blocks))
+
+    def allocate(self, total_tokens: int, num_current_blocks: int = 0):
+        delta = (total_tokens + self.page_size - 1) // self.page_size - num_current_blocks
+        if delta <= 0:
+            return []
+        if len(self.free) < delta:
+            return None
+        out = []
+        for _ in range(delta):
+            b = min(self.free)
+            self.free.remove(b)
+            self.allocated.add(b)
+            out.append(b)
+        return out
+
+    def release(self, block_ids):
+        for b in block_ids:
+            if b in self.allocated:
+                self.allocated.remove(b)
+                self.free.add(b)

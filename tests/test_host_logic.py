@@ -73,6 +73,65 @@ def test_bucket_padding_rules():
         StepBuffers(cfg, 8, 2, "cpu").load(meta, np.array([1, 2, 3]))
 
 
+def test_native_builder_pads_like_the_two_step_restatement():
+    # one native pass (metadata + padding) == prepare_gen_ctx_ref followed by pad_for_graph_ref
+    cfg = tiny_config()
+    maxb = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
+    rng = np.random.default_rng(5)
+    for n, cap_t, cap_s in ((0, 4, 2), (1, 16, 1), (3, 64, 4), (7, 128, 8)):
+        reqs = []
+        for s in range(n):
+            done = int(rng.integers(1, cfg.max_model_len))
+            this = 1 if rng.random() < 0.5 else int(rng.integers(1, min(done, 16) + 1))
+            nb = (done + cfg.page_size - 1) // cfg.page_size + int(rng.integers(0, 2))
+            reqs.append(dict(num_computed_tokens=done, tokens_this_step=this,
+                             block_ids=rng.permutation(1000)[:min(nb, maxb)].tolist()))
+        T = sum(r["tokens_this_step"] for r in reqs)
+        ids = rng.integers(0, cfg.vocab_size, T)
+        b = StepBuffers(cfg, cap_t, cap_s, "cpu")
+        b.meta_host.fill_(0x5A)                           # stale contents must all be overwritten
+        assert b.load_requests(reqs, ids, cfg.page_size) == (T, n, max([r["tokens_this_step"] for r in reqs], default=0))
+        ref = OMeta.pad_for_graph_ref(OMeta.prepare_gen_ctx_ref(reqs, cfg.page_size, maxb), cap_t, cap_s)
+        for k in ("slot_mapping", "positions", "context_lens", "block_tables", "query_start_loc"):
+            assert np.array_equal(getattr(b, k).numpy(), ref[k]), (n, k)
+        assert b.input_ids.tolist() == ids.tolist() + [0] * (cap_t - T)
+
+
+def test_native_builder_rejects_inconsistent_steps():
+    good = dict(num_computed_tokens=9, tokens_this_step=2, block_ids=[4, 1, 7])
+    # positions 7, 8 -> block 1 row 3, block 7 row 0
+    assert build_step_metadata([good], 4, 3)["slot_mapping"].tolist() == [1 * 4 + 3, 7 * 4 + 0]
+    for bad in (dict(good, block_ids=[4, 1]),                    # 9 tokens need 3 blocks
+                dict(good, tokens_this_step=10),                 # more new tokens than context
+                dict(good, tokens_this_step=-1),
+                dict(good, block_ids=[4, 1, 7, 2])):             # more blocks than a table row holds
+        with pytest.raises(ValueError, match="inconsistent step"):
+            build_step_metadata([bad], 4, 3)
+
+
+def test_block_allocator_matches_the_scan_restatement():
+    rng = np.random.default_rng(11)
+    for num_blocks, page in ((1, 1), (37, 16), (500, 256)):
+        cfg = types.SimpleNamespace(max_cache_blocks=num_blocks, page_size=page)
+        m, ref = KC.KVCacheManager(cfg), OMeta.BlockAllocatorRef(num_blocks, page)
+        held = []
+        for _ in range(400):
+            if held and rng.random() < 0.45:
+                ids = held.pop(int(rng.integers(len(held))))
+                if rng.random() < 0.3:                           # double frees and foreign ids are ignored
+                    ids = ids + ids[:1] + [num_blocks + 3, -1]
+                m.free_blocks(ids)
+                ref.release(ids)
+            else:
+                tokens = int(rng.integers(0, page * max(2, num_blocks // 3)))
+                cur = int(rng.integers(0, 3))
+                got, want = m.allocate_blocks(tokens, cur), ref.allocate(tokens, cur)
+                assert got == want, (num_blocks, tokens, cur)
+                if got:
+                    held.append(got)
+            assert m.num_free_blocks() == len(ref.free) and m.num_allocated_blocks() == len(ref.allocated)
+
+
 def test_capture_sizes_and_byte_model():
     assert capture_sizes(1) == [1]
     assert capture_sizes(5) == [1, 2, 4, 8]

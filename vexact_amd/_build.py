@@ -14,8 +14,8 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvexact_hip.so")
-SOURCES = ["row_ops.hip", "gemm.hip", "paged_attn.hip", "moe.hip", "glue.hip"]
-HEADERS = ["common.h", "gemm_core.h"]
+SOURCES = ["row_ops.hip", "gemm.hip", "paged_attn.hip", "moe.hip", "glue.hip", "host_meta.cpp"]
+HEADERS = ["common.h", "gemm_core.h", "gemm_wide.h"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -ffp-contract=off: kernels that must agree bit for bit share source-level expressions, so the
@@ -33,8 +33,11 @@ FLAGS = [
 
 
 def _compile_one(src: str, obj_dir: str) -> str:
-    obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+    if src.endswith(".cpp"):  # host-only code: plain C++, no device pass
+        cmd = [HIPCC, "-x", "c++", "-O3", "-std=c++17", "-fPIC", "-c", os.path.join(CSRC, src), "-o", obj]
+    else:
+        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stderr[-4000:]}")

@@ -50,6 +50,12 @@ PROTOTYPES = {
     ),
     "vx_embedding": (_I, [_P, _P, _I, _P, _L, _L, _L, _P]),
     "vx_fill_i32": (_I, [_P, _I, _L, _P]),
+    "vx_host_step_metadata": (_I, [_L, _P, _P, _P, _P, _I, _L, _L, _L] + [_P] * 7),
+    "vx_kv_allocator_create": (_P, [_L]),
+    "vx_kv_allocator_destroy": (None, [_P]),
+    "vx_kv_allocator_num_free": (_L, [_P]),
+    "vx_kv_allocator_allocate": (_L, [_P, _L, _L, _I, _P, _L]),
+    "vx_kv_allocator_free": (_L, [_P, _P, _L]),
 }
 
 _lib = None

@@ -7,14 +7,14 @@ Mirrors ``vexact/batch_invariant_ops/kv_cache_context.py`` of the reference: ``K
 
 from __future__ import annotations
 
-import heapq
+import ctypes
 import threading
 from dataclasses import dataclass
 from typing import Iterable, Optional
 
 import torch
 
-from .. import ops
+from .. import _lib, ops
 
 _context_storage = threading.local()
 
@@ -97,15 +97,24 @@ def clear_kv_cache_context() -> None:
 class KVCacheManager:
     """Block allocator: always hands out the lowest free block id, ``None`` when out of blocks.
 
-    Same observable behaviour as the reference allocator; the free list is a heap so an
-    allocation costs O(log n) instead of a scan of the free set.
+    Same observable behaviour as the reference allocator (kv_cache_context.py:141-217); the free
+    list is a native min-heap (``vx_kv_allocator_*``), so an allocation costs O(log n) per block
+    instead of a scan of the free set. Not thread-safe, like the reference's.
     """
 
     def __init__(self, cache_config):
         self.cache_config = cache_config
-        self.allocated_blocks: set[int] = set()
-        self._free_heap = list(range(cache_config.max_cache_blocks))  # already a valid heap
-        self.free_blocks_set = set(self._free_heap)
+        self._lib = _lib.load()
+        self._num_blocks = int(cache_config.max_cache_blocks)
+        self._h = self._lib.vx_kv_allocator_create(self._num_blocks)
+        if not self._h:
+            raise ValueError(f"cannot create a block allocator for {cache_config.max_cache_blocks} blocks")
+        self._out = (ctypes.c_int32 * max(1, self._num_blocks))()
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.vx_kv_allocator_destroy(h)
 
     def _num_blocks_needed(self, num_tokens: int) -> int:
         return (num_tokens + self.cache_config.page_size - 1) // self.cache_config.page_size
@@ -114,30 +123,21 @@ class KVCacheManager:
         delta = self._num_blocks_needed(total_tokens) - num_current_blocks
         if delta <= 0:
             return []
-        if len(self.free_blocks_set) < delta:
+        if delta > self._num_blocks:
             return None
-        allocated = []
-        while len(allocated) < delta:
-            block_id = heapq.heappop(self._free_heap)
-            if block_id not in self.free_blocks_set:  # stale heap entry
-                continue
-            self.free_blocks_set.remove(block_id)
-            self.allocated_blocks.add(block_id)
-            allocated.append(block_id)
-        return allocated
+        n = self._lib.vx_kv_allocator_allocate(self._h, int(delta), 0, 1, self._out, self._num_blocks)
+        return None if n < 0 else self._out[:n]
 
     def num_free_blocks(self) -> int:
-        return len(self.free_blocks_set)
+        return int(self._lib.vx_kv_allocator_num_free(self._h))
 
     def num_allocated_blocks(self) -> int:
-        return len(self.allocated_blocks)
+        return self._num_blocks - self.num_free_blocks()
 
     def free_blocks(self, block_ids):
-        for block_id in block_ids:
-            if block_id in self.allocated_blocks:
-                self.allocated_blocks.remove(block_id)
-                self.free_blocks_set.add(block_id)
-                heapq.heappush(self._free_heap, block_id)
+        ids = [int(b) for b in block_ids if -(2 ** 31) <= int(b) < 2 ** 31]
+        if ids:
+            self._lib.vx_kv_allocator_free(self._h, (ctypes.c_int32 * len(ids))(*ids), len(ids))
 
 
 class KVCacheStore:

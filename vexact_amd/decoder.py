@@ -13,6 +13,8 @@ residual -> RMSNorm -> router -> fused experts -> residual), all pipeline stages
 
 from __future__ import annotations
 
+import ctypes
+import itertools
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
@@ -127,28 +129,58 @@ def rope_tables(cfg: DecoderConfig, device) -> tuple[torch.Tensor, torch.Tensor]
     return emb.cos().to(torch.bfloat16).to(device), emb.sin().to(torch.bfloat16).to(device)
 
 
-def build_step_metadata(requests: Sequence[dict], page_size: int, max_blocks_per_req: int) -> dict:
-    """Integer metadata of one step, vectorised numpy (exact). ``requests`` hold
-    ``num_computed_tokens`` (after this step), ``tokens_this_step`` and ``block_ids``."""
-    n_tok = np.array([r["tokens_this_step"] for r in requests], dtype=np.int64)
-    done = np.array([r["num_computed_tokens"] for r in requests], dtype=np.int64)
+def _flatten_requests(requests: Sequence[dict]):
+    """``requests`` hold ``num_computed_tokens`` (after this step), ``tokens_this_step`` and
+    ``block_ids``; returns the flat int arrays the native builder reads."""
     B = len(requests)
-    qsl = np.zeros(B + 1, dtype=np.int32)
-    np.cumsum(n_tok, out=qsl[1:])
-    total = int(qsl[-1])
-    seq_of_tok = np.repeat(np.arange(B), n_tok)
-    positions = np.arange(total, dtype=np.int64) - np.repeat(qsl[:-1].astype(np.int64), n_tok) + np.repeat(done - n_tok, n_tok)
-    block_tables = np.full((B, max_blocks_per_req), -1, dtype=np.int32)
-    for s, r in enumerate(requests):
-        ids = r["block_ids"]
-        block_tables[s, : len(ids)] = ids
-    slot = block_tables[seq_of_tok, positions // page_size].astype(np.int64) * page_size + positions % page_size
+    done = np.fromiter((r["num_computed_tokens"] for r in requests), np.int64, B)
+    n_tok = np.fromiter((r["tokens_this_step"] for r in requests), np.int64, B)
+    offs = np.zeros(B + 1, np.int64)
+    np.cumsum(np.fromiter((len(r["block_ids"]) for r in requests), np.int64, B), out=offs[1:])
+    if B and all(isinstance(r["block_ids"], np.ndarray) for r in requests):  # the fast form: no per-id Python work
+        ids = np.concatenate([r["block_ids"] for r in requests]).astype(np.int32, copy=False)
+    else:
+        ids = np.fromiter(itertools.chain.from_iterable(r["block_ids"] for r in requests), np.int32, int(offs[-1]))
+    return done, n_tok, ids, offs
+
+
+def _native_step_metadata(requests, page_size, max_blocks, cap_tokens, cap_seqs, positions, slot, qsl, lens, bt):
+    """One call of ``vx_host_step_metadata`` writing into the given host addresses (ints)."""
+    from . import _lib
+
+    done, n_tok, ids, offs = _flatten_requests(requests)
+    total, maxq = ctypes.c_int64(0), ctypes.c_int32(0)
+    rc = _lib.load().vx_host_step_metadata(
+        len(requests), done.ctypes.data, n_tok.ctypes.data, ids.ctypes.data, offs.ctypes.data, page_size, max_blocks,
+        cap_tokens, cap_seqs, positions, slot, qsl, lens, bt, ctypes.byref(total), ctypes.byref(maxq))
+    if rc != 0:
+        # say which of the reference's conditions failed (inferencer.py:306-311), else the generic message
+        if len(requests) > cap_seqs:
+            raise ValueError(f"graph_num_seqs cannot be smaller than num_seqs: {cap_seqs} < {len(requests)}")
+        if int(n_tok.sum()) > cap_tokens:
+            raise ValueError(f"total_tokens exceeds capture_tokens: {int(n_tok.sum())} > {cap_tokens}")
+        raise ValueError("inconsistent step: a request's token counts or block ids do not cover its context, "
+                         f"or it holds more than {max_blocks} blocks")
+    return total.value, maxq.value
+
+
+def build_step_metadata(requests: Sequence[dict], page_size: int, max_blocks_per_req: int) -> dict:
+    """Integer metadata of one step at its exact size (no bucket padding), built by the native
+    host routine. ``requests`` hold ``num_computed_tokens`` (after this step), ``tokens_this_step``
+    and ``block_ids``."""
+    B = len(requests)
+    T = int(sum(max(0, r["tokens_this_step"]) for r in requests))
+    positions, slot = np.empty(T, np.int64), np.empty(T, np.int32)
+    qsl, lens = np.empty(B + 1, np.int32), np.empty(B, np.int32)
+    bt = np.empty((B, max_blocks_per_req), np.int32)
+    _, maxq = _native_step_metadata(requests, page_size, max_blocks_per_req, T, B, positions.ctypes.data, slot.ctypes.data,
+                                    qsl.ctypes.data, lens.ctypes.data, bt.ctypes.data)
     return {
-        "slot_mapping": slot.astype(np.int32),
-        "context_lens": done.astype(np.int32),
-        "block_tables": block_tables,
+        "slot_mapping": slot,
+        "context_lens": lens,
+        "block_tables": bt,
         "query_start_loc": qsl,
-        "max_seqlen_q": int(n_tok.max()) if B else 0,
+        "max_seqlen_q": maxq,
         "positions": positions,
     }
 
@@ -174,12 +206,27 @@ class StepBuffers:
         self.max_blocks = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
         i32, i64, bf = torch.int32, torch.int64, torch.bfloat16
         z = lambda *s, dtype: torch.zeros(s, dtype=dtype, device=device)  # noqa: E731
-        self.input_ids = z(T, dtype=i64)
-        self.positions = z(T, dtype=i64)
-        self.slot_mapping = torch.full((T,), -1, dtype=i32, device=device)
-        self.block_tables = torch.full((B, self.max_blocks), -1, dtype=i32, device=device)
-        self.context_lens = z(B, dtype=i32)
-        self.query_start_loc = z(B + 1, dtype=i32)
+        # All integer metadata lives in ONE device allocation mirrored by one (pinned) host staging
+        # buffer with the same layout, so that a step costs one host-to-device copy.
+        mb = self.max_blocks
+        segs = (("positions", i64, (T,)), ("input_ids", i64, (T,)), ("slot_mapping", i32, (T,)),
+                ("query_start_loc", i32, (B + 1,)), ("context_lens", i32, (B,)), ("block_tables", i32, (B, mb)))
+        offs, end = {}, 0
+        for name, dt, shape in segs:
+            offs[name] = end
+            end += -(-int(np.prod(shape)) * (8 if dt == i64 else 4) // 64) * 64
+        on_gpu = torch.device(device).type == "cuda"
+        self.meta_dev = torch.zeros(end, dtype=torch.uint8, device=device)
+        self.meta_host = torch.zeros(end, dtype=torch.uint8, pin_memory=on_gpu)
+        self._host = {}
+        for name, dt, shape in segs:
+            n = int(np.prod(shape)) * (8 if dt == i64 else 4)
+            setattr(self, name, self.meta_dev[offs[name]: offs[name] + n].view(dt).view(shape))
+            self._host[name] = self.meta_host[offs[name]: offs[name] + n].view(dt).view(shape).numpy()
+        self._host_ptr = {k: v.ctypes.data for k, v in self._host.items()}
+        self._host["slot_mapping"].fill(-1)
+        self._host["block_tables"].fill(-1)
+        self.meta_dev.copy_(self.meta_host)
         H, k = cfg.hidden_size, cfg.top_k
         self.x = z(T, H, dtype=bf)
         self.h = z(T, H, dtype=bf)
@@ -217,18 +264,33 @@ class StepBuffers:
             raise ValueError(f"total_tokens exceeds capture_tokens: {T} > {self.num_tokens}")
         if B > self.num_seqs:
             raise ValueError(f"graph_num_seqs cannot be smaller than num_seqs: {self.num_seqs} < {B}")
-        ids = np.zeros(self.num_tokens, np.int64); ids[:T] = input_ids
-        pos = np.zeros(self.num_tokens, np.int64); pos[:T] = meta["positions"]
-        slot = np.full(self.num_tokens, -1, np.int32); slot[:T] = meta["slot_mapping"]
-        bt = np.zeros((self.num_seqs, self.max_blocks), np.int32)
-        bt[:B] = -1
-        w = meta["block_tables"].shape[1]
-        bt[:B, :w] = meta["block_tables"][:, : self.max_blocks]
-        lens = np.zeros(self.num_seqs, np.int32); lens[:B] = meta["context_lens"]
-        qsl = np.full(self.num_seqs + 1, T, np.int32); qsl[: B + 1] = meta["query_start_loc"]
-        for dst, src in ((self.input_ids, ids), (self.positions, pos), (self.slot_mapping, slot), (self.block_tables, bt),
-                         (self.context_lens, lens), (self.query_start_loc, qsl)):
-            dst.copy_(torch.from_numpy(src), non_blocking=False)
+        h = self._host
+        h["positions"][:T] = meta["positions"]; h["positions"][T:] = 0
+        h["slot_mapping"][:T] = meta["slot_mapping"]; h["slot_mapping"][T:] = -1
+        w = min(meta["block_tables"].shape[1], self.max_blocks)
+        h["block_tables"][:B] = -1; h["block_tables"][B:] = 0
+        h["block_tables"][:B, :w] = meta["block_tables"][:, :w]
+        h["context_lens"][:B] = meta["context_lens"]; h["context_lens"][B:] = 0
+        h["query_start_loc"][: B + 1] = meta["query_start_loc"]; h["query_start_loc"][B + 1:] = T
+        return self._commit(T, B, input_ids)
+
+    def load_requests(self, requests: Sequence[dict], input_ids: np.ndarray, page_size: int) -> tuple[int, int, int]:
+        """Build the step's metadata with the bucket padding straight into the staging buffer
+        (native, one pass) and copy it to the device. Returns (tokens, sequences, max_seqlen_q)."""
+        p = self._host_ptr
+        T, maxq = _native_step_metadata(requests, page_size, self.max_blocks, self.num_tokens, self.num_seqs,
+                                        p["positions"], p["slot_mapping"], p["query_start_loc"], p["context_lens"],
+                                        p["block_tables"])
+        if len(input_ids) != T:
+            raise ValueError(f"{len(input_ids)} input ids for a step of {T} tokens")
+        self._commit(T, len(requests), input_ids)
+        return T, len(requests), maxq
+
+    def _commit(self, T: int, B: int, input_ids) -> tuple[int, int]:
+        ids = self._host["input_ids"]
+        ids[:T] = input_ids
+        ids[T:] = 0
+        self.meta_dev.copy_(self.meta_host, non_blocking=False)
         return T, B
 
 
