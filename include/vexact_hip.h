@@ -190,6 +190,22 @@ int vx_embedding(const void* table, const void* ids, int ids_i64, void* out, int
                  int64_t vocab, hipStream_t stream);
 int vx_fill_i32(int* p, int value, int64_t n, hipStream_t stream);
 
+/* ---- token sampler ------------------------------------------------------------------------- */
+
+/* One token per row of logits [rows, V] (dtype 0 bf16, 1 fp32; ld = row pitch in elements):
+ * x = f32(logit) * (1 / temperature); top_k (<= 0 or >= V: off) masks keys below the k-th largest;
+ * top_p (>= 1: off) masks the keys whose inclusive ascending probability mass is <= 1 - p (integer
+ * masses floor(exp(x - max) * 2^32), equal logits treated alike); the token is the winner of an
+ * exponential race argmin E_i / exp(x_i - max) whose noise is Philox4x32-10 keyed by seeds[row] with
+ * counter (token / 4, positions[row]), so it depends on (logits row, seed, position) only: not on
+ * the batch or the row's place in it. Needs temperature > 0 and top_p > 0 (greedy decoding is
+ * vx_logprobs with labels == NULL). No workspace, no host synchronisation.
+ * Replaces Sampler.batch_sample_token / apply_top_k_top_p / _random_sample / _seeded_sample,
+ * vexact/inferencer/sampler.py:29-189 (the seeded path there calls vLLM's Gumbel kernel). */
+int vx_sample_tokens(const void* logits, int dtype, int64_t ld, int64_t rows, int64_t V, float temperature,
+                     int top_k, float top_p, const int64_t* seeds, const int64_t* positions,
+                     int64_t* tokens_out, hipStream_t stream);
+
 /* ---- host-side step metadata and block allocator (CPU code, no device work, no stream) -------- */
 
 /* Integer metadata of one step, written into host buffers sized for a graph bucket (cap_tokens

@@ -167,3 +167,50 @@ def test_graph_replay_with_padding_equals_eager():
     g.replay()
     torch.cuda.synchronize()
     assert_bitwise(bg.logprobs.cpu()[:2], lp_eager[sub], "graph replay with another batch composition")
+
+
+def test_sampled_decode_is_batch_invariant_and_graph_safe():
+    cfg, w, dec, prompts, blocks = _setup(num_seqs=5, seed=7)
+    allseq = list(range(5))
+    tok, _, _, _ = _prefill(dec, cfg, prompts, blocks, allseq)
+    first = tok.numpy()
+    sampling = (0.8, 20, 0.9)
+    seeds = torch.tensor([11, 22, 33, 44, 55], dtype=torch.int64)
+    dmeta = _decode_meta(cfg, prompts, blocks, allseq)
+    be = dec.bucket(5, 5)
+    be.load(dmeta, first)
+    be.seeds.copy_(seeds)
+    dec.step(be, 1, sampling=sampling)
+    torch.cuda.synchronize()
+    tok_e, lp_e = be.tokens.cpu().clone(), be.logprobs.cpu().clone()
+    # the token is one of the 20 most likely and the logprob is that token's
+    logits = be.logits.float().cpu()
+    assert bool((logits.topk(20, dim=-1).indices == tok_e[:, None]).any(dim=1).all())
+    want_lp = torch.log_softmax(logits, -1).gather(1, tok_e[:, None])[:, 0]
+    assert float((lp_e - want_lp).abs().max()) < 1e-4
+    # each request alone draws the same token with the same logprob bits
+    b1 = dec.bucket(1, 1)
+    for s in allseq:
+        b1.load(_decode_meta(cfg, prompts, blocks, [s]), first[s : s + 1])
+        b1.seeds.copy_(seeds[s : s + 1])
+        dec.step(b1, 1, sampling=sampling)
+        torch.cuda.synchronize()
+        assert int(b1.tokens[0]) == int(tok_e[s])
+        assert_bitwise(b1.logprobs.cpu(), lp_e[s : s + 1], f"sampled logprob of request {s} alone")
+    # padded graph replay, twice, and with the requests in another order
+    bg = dec.bucket(8, 8)
+    bg.load(dmeta, first)
+    bg.seeds[:5].copy_(seeds)
+    g = dec.capture(bg, 1, sampling=sampling)
+    for rep in range(2):
+        bg.load(dmeta, first)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(bg.tokens.cpu()[:5], tok_e)
+        assert_bitwise(bg.logprobs.cpu()[:5], lp_e, f"sampled graph replay {rep}")
+    order = [3, 0, 4, 2, 1]
+    bg.load(_decode_meta(cfg, prompts, blocks, order), first[order])
+    bg.seeds[:5].copy_(seeds[order])
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(bg.tokens.cpu()[:5], tok_e[order])

@@ -50,6 +50,7 @@ PROTOTYPES = {
     ),
     "vx_embedding": (_I, [_P, _P, _I, _P, _L, _L, _L, _P]),
     "vx_fill_i32": (_I, [_P, _I, _L, _P]),
+    "vx_sample_tokens": (_I, [_P, _I, _L, _L, _L, _F, _I, _F, _P, _P, _P, _P]),
     "vx_host_step_metadata": (_I, [_L, _P, _P, _P, _P, _I, _L, _L, _L] + [_P] * 7),
     "vx_kv_allocator_create": (_P, [_L]),
     "vx_kv_allocator_destroy": (None, [_P]),

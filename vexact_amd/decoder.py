@@ -254,6 +254,8 @@ class StepBuffers:
         self.logits = z(B, cfg.vocab_size, dtype=bf)
         self.logprobs = z(B, dtype=torch.float32)
         self.tokens = z(B, dtype=i64)
+        self.seeds = z(B, dtype=i64)       # per-sequence sampling seeds (set by the caller)
+        self.sample_pos = z(B, dtype=i64)  # position of the token being sampled = context length
 
     def load(self, meta: dict, input_ids: np.ndarray) -> tuple[int, int]:
         """Copy one step's metadata in, applying the bucket padding rules (inferencer.py:306-324):
@@ -308,7 +310,7 @@ class Qwen3MoeDecoder:
         self.value_cache = [torch.zeros(shape, dtype=torch.bfloat16, device=device).permute(0, 2, 1, 3)
                             for _ in range(cfg.num_layers)]
         self.buffers: dict[tuple[int, int], StepBuffers] = {}
-        self.graphs: dict[tuple[int, int, int], torch.cuda.CUDAGraph] = {}
+        self.graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
 
     def bucket(self, num_tokens: int, num_seqs: int) -> StepBuffers:
         key = (num_tokens, num_seqs)
@@ -360,8 +362,10 @@ class Qwen3MoeDecoder:
             "vx_router_topk",
         )
 
-    def sample(self, b: StepBuffers, decode: bool) -> None:
-        """Last token of each sequence -> lm_head -> greedy token and its fp32 logprob."""
+    def sample(self, b: StepBuffers, decode: bool, sampling: Optional[tuple] = None) -> None:
+        """Last token of each sequence -> lm_head -> token and its fp32 logprob. ``sampling`` is
+        ``None`` for greedy decoding or ``(temperature, top_k, top_p)``: then row s draws its token
+        with the noise stream of (``b.seeds[s]``, its context length), whatever batch it is in."""
         if decode and b.num_tokens == b.num_seqs:
             last = b.h  # every token is a last token
         else:
@@ -369,27 +373,34 @@ class Qwen3MoeDecoder:
             torch.index_select(b.h, 0, idx, out=b.last_h)
             last = b.last_h
         ops.gemm_nt(last, self.w.lm_head, out=b.logits)
-        lp, tok = ops.logprobs(b.logits, None, return_tokens=True)
+        if sampling is None:
+            lp, tok = ops.logprobs(b.logits, None, return_tokens=True)
+            b.tokens.copy_(tok)
+        else:
+            temperature, top_k, top_p = sampling
+            b.sample_pos.copy_(b.context_lens)
+            ops.sample_tokens(b.logits, temperature, top_k, top_p, b.seeds, b.sample_pos, out=b.tokens)
+            lp = ops.logprobs(b.logits, b.tokens)
         b.logprobs.copy_(lp)
-        b.tokens.copy_(tok)
 
-    def step(self, b: StepBuffers, max_seqlen_q: int, routing_log: Optional[list] = None) -> None:
+    def step(self, b: StepBuffers, max_seqlen_q: int, routing_log: Optional[list] = None,
+             sampling: Optional[tuple] = None) -> None:
         self.forward(b, max_seqlen_q, routing_log)
-        self.sample(b, decode=(max_seqlen_q == 1))
+        self.sample(b, decode=(max_seqlen_q == 1), sampling=sampling)
 
-    def capture(self, b: StepBuffers, max_seqlen_q: int = 1) -> torch.cuda.CUDAGraph:
-        key = (b.num_tokens, b.num_seqs, max_seqlen_q)
+    def capture(self, b: StepBuffers, max_seqlen_q: int = 1, sampling: Optional[tuple] = None) -> torch.cuda.CUDAGraph:
+        key = (b.num_tokens, b.num_seqs, max_seqlen_q, sampling)
         if key in self.graphs:
             return self.graphs[key]
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
-            self.step(b, max_seqlen_q)  # warm-up on a side stream
+            self.step(b, max_seqlen_q, sampling=sampling)  # warm-up on a side stream
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            self.step(b, max_seqlen_q)
+            self.step(b, max_seqlen_q, sampling=sampling)
         self.graphs[key] = g
         return g
 

@@ -78,6 +78,16 @@ def main() -> None:
             print(f"{name:34s} {t * 1e6:9.1f} us  {nbytes / t / 1e9:8.1f} GB/s  ({nbytes / t / HBM_PEAK * 100:5.1f}% of 8 TB/s)  {nbytes / 1e6:.1f} MB", flush=True)
 
     what = a.what.split(",")
+    if "sampler" in what:
+        V = 151936
+        lg = (torch.randn(B, V, generator=g, device=dev) * 2.5).to(torch.bfloat16)
+        seeds = torch.arange(B, dtype=torch.int64, device=dev) + 1234
+        pos = torch.arange(B, dtype=torch.int64, device=dev) + 1000
+        out = torch.empty(B, dtype=torch.int64, device=dev)
+        for name, k, p in (("plain", None, 1.0), ("top-p 0.9", None, 0.9), ("top-k 50", 50, 1.0), ("top-k 50 + top-p 0.9", 50, 0.9)):
+            report(f"sampler {name} (B={B}, V={V})",
+                   timeit(lambda li: ops.sample_tokens(lg, 0.8, k, p, seeds, pos, out=out), n_layers=4), B * V * 2)
+        report("greedy argmax + logprob", timeit(lambda li: ops.logprobs(lg, None, return_tokens=True), n_layers=4), B * V * 2)
     if "moe" in what:
         x = rnd(B, H, std=1.0)
         logits = torch.randn(B, E, generator=g, device=dev)

@@ -184,6 +184,37 @@ def logprobs(
     return (out, toks) if return_tokens else out
 
 
+def sample_tokens(
+    logits: torch.Tensor, temperature: float, top_k: Optional[int], top_p: float, seeds: torch.Tensor,
+    positions: torch.Tensor, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """One sampled token per row of ``logits`` [B, V] (bf16 or fp32): temperature, top-k, top-p and a
+    Philox-seeded exponential race in one kernel. ``seeds`` / ``positions`` are int64 [B] on the device;
+    a row's token depends only on (its logits, its seed, its position)."""
+    _need_gpu("logits", logits)
+    if logits.dim() != 2 or logits.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"sample_tokens: need [B, V] bf16 or fp32 logits, got {tuple(logits.shape)} {logits.dtype}")
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    B, V = logits.shape
+    if not (temperature > 0 and top_p > 0):
+        raise ValueError("sample_tokens: temperature and top_p must be positive (greedy decoding is logprobs(labels=None))")
+    for name, t in (("seeds", seeds), ("positions", positions)):
+        if t.dtype != torch.int64 or t.numel() != B or not t.is_contiguous() or t.device != logits.device:
+            raise ValueError(f"sample_tokens: {name} must be a contiguous int64 [B] tensor on the logits' device")
+    if out is None:
+        out = torch.empty(B, dtype=torch.int64, device=logits.device)
+    _lib.check(
+        _lib.load().vx_sample_tokens(
+            logits.data_ptr(), 0 if logits.dtype == torch.bfloat16 else 1, logits.stride(0), B, V, float(temperature),
+            int(top_k) if top_k is not None else 0, float(top_p), seeds.data_ptr(), positions.data_ptr(), out.data_ptr(),
+            _stream(),
+        ),
+        "vx_sample_tokens",
+    )
+    return out
+
+
 # ----------------------------------------------------------------------------- GEMM
 
 
