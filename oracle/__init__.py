@@ -27,10 +27,16 @@ routing_integers_ref   brute-force counting; numpy stable argsort twice (fused_m
 fused_moe_ref          k=1,w=1 => plain SwiGLU MLP; all tokens on one expert => dense formula;
                        fp64 brute force on tiny shapes; HF-eager form within bf16 tolerance
 prepare_gen_ctx_ref    hand-worked example; vectorised numpy twin
+BlockAllocatorRef      scan restatement of the reference allocator; hand-worked sequence
+sampler.philox4x32     Random123 known-answer vectors
+sampler.exp32 / log    numpy exp / log within 4e-7 / 2e-6
+sampler.kept_mask_spec the reference's sort + cumsum rule (apply_top_k_top_p_ref) on tie-free rows
+sample_tokens_ref      argmax(probs / q) with the same variates; softmax frequencies (chi-square
+                       style bound); (seed, position) keyed: order invariance
 =====================  ===========================================================================
 
 Parity unpinned (arithmetic lives in third-party wheels that are not in the reference tree, and
 only invariance tests cover them there): the exact bit patterns of flash-attn 3/4 attention,
-flash-attn 2.8.4 cross-entropy, quack 0.3.4 grouped GEMM and veomni 0.1.9a5 fused MoE. Parity
+flash-attn 2.8.4 cross-entropy, quack 0.3.4 grouped GEMM and veomni 0.1.9a5 fused MoE, and the noise stream of vLLM's seeded Gumbel sampling kernel. Parity
 against those is by the closed forms above within the stated tolerances.
 """

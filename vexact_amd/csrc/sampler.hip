@@ -22,6 +22,8 @@
 //          on ties, E_i = -log32(u_i), u_i = (2 n_i + 1) / 2^33, n_i = Philox output for token i
 // exp32 / log32 are fixed polynomial evaluations in fp32 made of IEEE add / mul / div only (this file
 // is compiled without contraction), integer sums are order-free, so any tiling gives the same bits.
+#include <type_traits>
+
 #include "common.h"
 
 namespace vx {
@@ -29,6 +31,10 @@ namespace vx {
 constexpr int SM_THREADS = 1024;
 constexpr int SM_WAVES = SM_THREADS / 64;
 constexpr float SM_CUTOFF = -32.0f;
+// Radix digits of the 32-bit keys, most significant first: 12 + 10 + 10 bits. The wide first digit
+// (sign, exponent, three mantissa bits) spreads a row of logits over a few hundred bins, which keeps
+// the LDS atomics of the first pass from piling onto a handful of addresses.
+constexpr int SM_BINS0 = 4096;
 
 __device__ __forceinline__ uint32_t float_key(float x) {
   const uint32_t b = __builtin_bit_cast(uint32_t, x);
@@ -173,29 +179,30 @@ __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
 
 // hist[bin] += w for the lanes with valid set. When every valid lane of the wavefront hits one bin
 // (the common case for the leading digits of float keys) the wavefront adds once.
+template <bool COUNT>  // COUNT: every w is 1
 __device__ __forceinline__ void hist_add(unsigned long long* hist, bool valid, uint32_t bin, uint64_t w) {
   const uint64_t mask = __ballot(valid);
   if (mask == 0) return;
   const int leader = __ffsll((long long)mask) - 1;
   const uint32_t b0 = __shfl(bin, leader, 64);
   if (__ballot(valid && bin != b0) == 0) {
-    const uint64_t s = wave_sum_u64(valid ? w : 0ull);
+    const uint64_t s = COUNT ? (uint64_t)__popcll(mask) : wave_sum_u64(valid ? w : 0ull);
     if ((int)(threadIdx.x & 63) == leader) atomicAdd(&hist[b0], (unsigned long long)s);
   } else if (valid) {
     atomicAdd(&hist[bin], (unsigned long long)w);
   }
 }
 
-// Wavefront 0: first bin b (0..255) whose inclusive prefix sum reaches target; writes b and the
+// Wavefront 0: first bin b (0..nbins-1) whose inclusive prefix sum reaches target; writes b and the
 // exclusive prefix at b to res[0], res[1]. If the total is below target, the last non-empty bin.
-__device__ __forceinline__ void pick_bin(const unsigned long long* hist, uint64_t target, unsigned long long* res) {
+// Lane l owns the nbins / 64 consecutive bins starting at l * nbins / 64.
+__device__ __forceinline__ void pick_bin(const unsigned long long* hist, int nbins, uint64_t target,
+                                         unsigned long long* res) {
   const int lane = threadIdx.x & 63;
-  uint64_t h[4], local = 0;
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    h[j] = hist[4 * lane + j];
-    local += h[j];
-  }
+  const int per = nbins >> 6;
+  const unsigned long long* mine = hist + lane * per;
+  uint64_t local = 0;
+  for (int j = 0; j < per; j++) local += mine[j];
   uint64_t incl = local;  // inclusive scan over lanes
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
@@ -204,37 +211,25 @@ __device__ __forceinline__ void pick_bin(const unsigned long long* hist, uint64_
   }
   const uint64_t hit = __ballot(incl >= target);
   const uint64_t nonempty = __ballot(local != 0);
-  int pick_lane;
-  bool fallback = false;
-  if (hit) {
-    pick_lane = __ffsll((long long)hit) - 1;
-  } else {
-    fallback = true;
-    pick_lane = nonempty ? 63 - __builtin_clzll(nonempty) : 0;
-  }
+  const bool fallback = hit == 0;
+  const int pick_lane = !fallback ? __ffsll((long long)hit) - 1 : (nonempty ? 63 - __builtin_clzll(nonempty) : 0);
   if (lane == pick_lane) {
     uint64_t ex = incl - local;
-    int b = 4 * lane;
+    int j = 0;
     if (!fallback) {
-      int j = 0;
-      while (j < 3 && ex + h[j] < target) {
-        ex += h[j];
-        j++;
-      }
-      b += j;
+      while (j < per - 1 && ex + mine[j] < target) ex += mine[j++];
     } else {
-      int j = 3;
-      while (j > 0 && h[j] == 0) j--;
-      for (int t = 0; t < j; t++) ex += h[t];
-      b += j;
+      int last = per - 1;
+      while (last > 0 && mine[last] == 0) last--;
+      while (j < last) ex += mine[j++];
     }
-    res[0] = (unsigned long long)b;
+    res[0] = (unsigned long long)(lane * per + j);
     res[1] = (unsigned long long)ex;
   }
 }
 
 __global__ __launch_bounds__(SM_THREADS) void sample_kernel(SampleParams p) {
-  __shared__ unsigned long long hist[256];
+  __shared__ unsigned long long hist[SM_BINS0];
   __shared__ unsigned long long res[2];
   __shared__ float redf[SM_WAVES];
   __shared__ unsigned long long red64[SM_WAVES];
@@ -254,13 +249,16 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(SampleParams p) {
   });
   mx = block_max<SM_WAVES>(mx, redf);
 
-  // ---- radix selects, most significant byte first. DESC: by count from the top (top-k);
+  // ---- radix selects, most significant digit first. desc: by count from the top (top-k);
   // otherwise by mass from the bottom over keys >= floor_key (top-p).
-  auto radix_select = [&](bool desc, uint64_t target, uint32_t floor_key) -> uint32_t {
+  auto radix_select = [&](auto desc_tag, uint64_t target, uint32_t floor_key) -> uint32_t {
+    constexpr bool desc = decltype(desc_tag)::value;
     uint32_t prefix = 0;
-    for (int pass = 0; pass < 4; pass++) {
-      const int shift = 24 - 8 * pass;
-      if (tid < 256) hist[tid] = 0;
+    for (int pass = 0; pass < 3; pass++) {
+      const int shift = pass == 0 ? 20 : (pass == 1 ? 10 : 0);
+      const int bits = pass == 0 ? 12 : 10;
+      const int nbins = 1 << bits;
+      for (int i = tid; i < nbins; i += SM_THREADS) hist[i] = 0;
       __syncthreads();
       scan_row(p, row, aligned, groups, [&](const Quad& q, int, bool in) {
 #pragma unroll
@@ -270,24 +268,23 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(SampleParams p) {
           uint64_t w = 1;
           if (valid) {
             key = float_key(q.x[j]);
-            if (pass > 0 && (key >> (shift + 8)) != prefix) valid = false;
-            if (!desc) {
+            if (pass > 0 && (key >> (shift + bits)) != prefix) valid = false;
+            if constexpr (!desc) {
               const float d = q.x[j] - mx;
               if (key < floor_key || !(d >= SM_CUTOFF)) valid = false;
               else w = (uint64_t)(exp32(d) * 4294967296.0f);
             }
           }
-          uint32_t bin = (key >> shift) & 255u;
-          if (desc) bin = 255u - bin;
-          hist_add(hist, valid, bin, w);
+          uint32_t bin = (key >> shift) & (uint32_t)(nbins - 1);
+          if (desc) bin = (uint32_t)(nbins - 1) - bin;
+          hist_add<desc>(hist, valid, bin, w);
         }
       });
       __syncthreads();
       if (!desc && pass == 0) {  // the mass limit needs the total first: L = floor((1 - p) Q), target = L + 1
         if (wave == 0) {
           uint64_t s = 0;
-#pragma unroll
-          for (int j = 0; j < 4; j++) s += hist[4 * lane + j];
+          for (int j = 0; j < nbins / 64; j++) s += hist[lane * (nbins / 64) + j];
           s = wave_sum_u64(s);
           if (lane == 0) red64[0] = s;
         }
@@ -295,21 +292,21 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(SampleParams p) {
         const double lim = (double)(1.0f - p.top_p) * (double)red64[0];
         target = (uint64_t)lim + 1ull;
       }
-      if (wave == 0) pick_bin(hist, target, res);
+      if (wave == 0) pick_bin(hist, nbins, target, res);
       __syncthreads();
       uint32_t b = (uint32_t)res[0];
       target -= res[1];
-      if (desc) b = 255u - b;
-      prefix = (prefix << 8) | b;
+      if (desc) b = (uint32_t)(nbins - 1) - b;
+      prefix = (prefix << bits) | b;
       __syncthreads();
     }
     return prefix;
   };
 
   uint32_t thr = 0;
-  if (p.top_k > 0 && p.top_k < p.V) thr = radix_select(true, (uint64_t)p.top_k, 0u);
+  if (p.top_k > 0 && p.top_k < p.V) thr = radix_select(std::true_type{}, (uint64_t)p.top_k, 0u);
   if (p.top_p < 1.0f) {
-    const uint32_t tp = radix_select(false, 0ull, thr);
+    const uint32_t tp = radix_select(std::false_type{}, 0ull, thr);
     thr = tp > thr ? tp : thr;
   }
 
