@@ -82,6 +82,16 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
 int vx_gemm_bf16_nt_variant(const void* x, const void* w, const void* bias, void* c, int64_t M,
                             int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind,
                             int mt, hipStream_t stream);
+/* Dense SwiGLU: C[M, N] = r16(r16(silu(r16(X Wg^T))) * r16(X Wu^T)) for K-contiguous bf16 X [M, K],
+ * Wg, Wu [N, K] (same pitch ldw): gate_proj, up_proj and act_fn(gate) * up of a dense MLP in one
+ * kernel, bit-identical to two vx_gemm_bf16_nt calls followed by bf16 silu and multiply (the glue
+ * the reference runs in torch between its GEMMs: Qwen3MoeMLP.forward, HF modeling_qwen3_moe.py, which
+ * vexact/models/qwen3_moe/modeling_qwen3_moe.py keeps for the dense layers). kind < 0 chooses the
+ * kernel by M; 0 (with mt = 1 / 2 / 4: 16 mt rows per tile), 1, 3 force the streaming, 128x128 tiled
+ * or 256x256 wide kernel (all give the same bits). */
+int vx_gemm_swiglu_bf16_nt(const void* x, const void* w_gate, const void* w_up, void* c, int64_t M, int64_t N,
+                           int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind, int mt, hipStream_t stream);
+
 /* Batched, fully strided fallback for any dtype code: one thread per output, fp32 FMA chain in
  * ascending k. Covers the layouts / dtypes of matmul_persistent and _bmm_kernel / triton_bmm
  * (batch_invariant_ops.py:484-606) that the fast path rejects. */

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import row_ops as O
-from tests.util import assert_bf16_close, assert_bitwise
+from tests.util import assert_bf16_close, assert_bitwise, bf16_ulp_distance
 
 pytestmark = pytest.mark.gpu
 
@@ -168,3 +168,30 @@ def test_bmm():
     torch.testing.assert_close(got.cpu(), torch.bmm(inv, pos), atol=0, rtol=0)  # single products are exact
     with pytest.raises(AssertionError):
         triton_bmm(a.cuda()[0], b.cuda())
+
+
+@pytest.mark.parametrize("N,K", [(1536, 2048), (6144, 1024), (200, 264)])
+def test_dense_swiglu_equals_unfused_chain_and_is_row_invariant(N, K):
+    g = torch.Generator(device="cuda").manual_seed(N + K)
+    wg = torch.empty(N, K, dtype=torch.bfloat16, device="cuda").normal_(0, 0.03, generator=g)
+    wu = torch.empty(N, K, dtype=torch.bfloat16, device="cuda").normal_(0, 0.03, generator=g)
+    xall = torch.empty(4096, K, dtype=torch.bfloat16, device="cuda").normal_(0, 1.0, generator=g)
+    big = ops.gemm_swiglu(xall, wg, wu)                       # 4096 rows: wide or tiled kernel
+    for M in (1, 7, 64, 65, 300, 384, 385, 2048):
+        print(f"[case] dense swiglu M={M} N={N} K={K}", flush=True)
+        x = xall[:M]
+        got = ops.gemm_swiglu(x, wg, wu)
+        assert_bitwise(got, big[:M], f"rows 0..{M} alone vs inside 4096 rows")
+        gate, up = ops.gemm_nt(x, wg), ops.gemm_nt(x, wu)
+        want = torch.nn.functional.silu(gate) * up            # bf16 silu, bf16 multiply
+        ulp = bf16_ulp_distance(got, want)
+        assert int(ulp.max()) <= 1 and float((ulp == 0).float().mean()) > 0.999, (int(ulp.max()), float((ulp == 0).float().mean()))
+    # every kernel that can run the shape gives the same bits
+    x = xall[:300]
+    ref = ops.gemm_swiglu(x, wg, wu)
+    for kind, mt in ((0, 1), (0, 2), (0, 4), (1, 0)) + (((3, 0),) if K % 64 == 0 else ()):
+        assert_bitwise(ops.gemm_swiglu(x, wg, wu, kind=kind, mt=mt), ref, f"kind {kind} mt {mt}")
+    # and the fused MoE's expert MLP with routing weight 1 is the same arithmetic
+    down = torch.empty(256, N, dtype=torch.bfloat16, device="cuda").normal_(0, 0.03, generator=g)
+    y = ops.swiglu_mlp(x, wg, wu, down)
+    assert_bitwise(y, ops.gemm_nt(ref, down), "swiglu_mlp")

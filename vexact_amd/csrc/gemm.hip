@@ -106,6 +106,54 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
   return launch_status();
 }
 
+// Dense SwiGLU: C[M, N] = r16(r16(silu(r16(X Wg^T))) * r16(X Wu^T)), both projections and the
+// activation in one kernel. kind < 0: automatic; 0 / 1 / 3 force the streaming (mt rows / 16), the
+// 128x128 tiled or the 256x256 wide kernel (for the tests that check they agree bit for bit).
+static int gemm_swiglu_dispatch(const GemmParams& p, int kind, int mt, hipStream_t stream) {
+  const int64_t M = p.M, N = p.N;
+  if (kind < 0) {
+    const int64_t wide_tiles = ((M + WD_BM - 1) / WD_BM) * ((N + 127) / 128);
+    if (M <= 16) { kind = 0; mt = 1; }
+    else if (M <= 32) { kind = 0; mt = 2; }
+    else if (M <= 64) { kind = 0; mt = 4; }
+    else if (M > 384 && wide_tiles >= 64 && p.K % WD_BK == 0) kind = 3;  // measured crossover
+    else kind = 1;
+  }
+  if (kind == 0) {
+    if (mt != 1 && mt != 2 && mt != 4) return VX_ERR_ARG;
+    const int64_t my = (M + 16 * mt - 1) / (16 * mt);
+    if (my > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)my);
+    if (mt == 1) gemm_stream_kernel<1, EPI_SWIGLU, false><<<grid, 256, 0, stream>>>(p);
+    else if (mt == 2) gemm_stream_kernel<2, EPI_SWIGLU, false><<<grid, 256, 0, stream>>>(p);
+    else gemm_stream_kernel<4, EPI_SWIGLU, false><<<grid, 256, 0, stream>>>(p);
+  } else if (kind == 1) {
+    const int64_t my = (M + TL_BM - 1) / TL_BM;
+    if (my > 65535) return VX_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)my);
+    gemm_tiled_kernel<EPI_SWIGLU, false><<<grid, 256, 0, stream>>>(p);
+  } else if (kind == 3) {
+    if (!gemm_wide_swiglu_launch(p, stream)) return VX_ERR_UNSUPPORTED;
+  } else {
+    return VX_ERR_ARG;
+  }
+  return launch_status();
+}
+
+int vx_gemm_swiglu_bf16_nt(const void* x, const void* w_gate, const void* w_up, void* c, int64_t M, int64_t N,
+                           int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int kind, int mt, hipStream_t stream) {
+  if (!x || !w_gate || !w_up || !c || M < 0 || N <= 0 || K <= 0) return VX_ERR_ARG;
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return VX_ERR_ARG;
+  if (!gemm_fast_ok(x, w_gate, K, ldx, ldw) || !gemm_fast_ok(x, w_up, K, ldx, ldw)) return VX_ERR_UNSUPPORTED;
+  if (M == 0) return VX_OK;
+  GemmParams p = {};
+  p.x = (const bf16_t*)x; p.ldx = ldx;
+  p.w = (const bf16_t*)w_gate; p.w2 = (const bf16_t*)w_up; p.ldw = ldw;
+  p.c = (bf16_t*)c; p.ldc = ldc;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  return gemm_swiglu_dispatch(p, kind, mt, stream);
+}
+
 // Forces one kernel regardless of M (kind 0 = streaming with 16*mt rows per tile, mt in {1,2,4};
 // kind 1 = 128x128 tiled; kind 2 = streaming, 16 k-steps in flight; kind 3 = 256x256 wide tiles,
 // needs K % 64 == 0; kind 4 = LDS ring kernel, mt = configuration 0..6). For tests that check

@@ -35,7 +35,7 @@ struct GemmParams {
   const int* tile_row0;   // [m_tiles] first row of the tile (in C / sorted order)
   const int* tile_rows;   // [m_tiles] rows in the tile
   const int* row_src;     // [M] row of x feeding C row i (null = identity)
-  const bf16_t* row_scale;      // EPI_SWIGLU: per-row routing weight, looked up as
+  const bf16_t* row_scale;      // EPI_SWIGLU: per-row routing weight (null = none), looked up as
   const int* row_scale_idx;     //   row_scale[row_scale_idx[i]] (idx null = identity)
 };
 
@@ -203,8 +203,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
     const int64_t orow = row0 + m;
     bf16_t o[4];
     if constexpr (EPI == EPI_SWIGLU) {
-      const int si = p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow;
-      const float wr = bf16_to_f32(p.row_scale[si]);
+      float wr = 1.0f;  // no row scale: the last rounding of swiglu_bf16 is then the identity
+      if (p.row_scale) wr = bf16_to_f32(p.row_scale[p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow]);
 #pragma unroll
       for (int j = 0; j < 4; j++) o[j] = swiglu_bf16(acc[i][j], acc2[i][j], wr);
     } else {
@@ -353,8 +353,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p) {
     if (m >= rows) continue;
     const int64_t orow = row0 + m;
     if constexpr (EPI == EPI_SWIGLU) {
-      const int si = p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow;
-      const float wr = bf16_to_f32(p.row_scale[si]);
+      float wr = 1.0f;  // no row scale: the last rounding of swiglu_bf16 is then the identity
+      if (p.row_scale) wr = bf16_to_f32(p.row_scale[p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow]);
 #pragma unroll
       for (int j = 0; j < 2; j++) {
         const int nc = n0 + 32 * wn + 16 * j + 4 * g;

@@ -234,7 +234,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
         float wr = 0.f;
         if (m < t.rows) {
           const int64_t orow = t.row0 + m;
-          wr = bf16_to_f32(p.row_scale[p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow]);
+          wr = p.row_scale ? bf16_to_f32(p.row_scale[p.row_scale_idx ? p.row_scale_idx[orow] : (int)orow]) : 1.0f;
         }
         bf16_t o[8];
 #pragma unroll
@@ -333,6 +333,12 @@ static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int6
 static inline bool gemm_wide_launch(const GemmParams& p, hipStream_t stream) {
   if (p.M <= 0) return false;
   return gemm_wide_launch_t<EPI_PLAIN, false>(p, ((int64_t)p.M + WD_BM - 1) / WD_BM, p.M, stream);
+}
+
+// dense with the SwiGLU epilogue: C[M, N] = swiglu(X Wg^T, X Wu^T)
+static inline bool gemm_wide_swiglu_launch(const GemmParams& p, hipStream_t stream) {
+  if (p.M <= 0) return false;
+  return gemm_wide_launch_t<EPI_SWIGLU, false>(p, ((int64_t)p.M + WD_BM - 1) / WD_BM, p.M, stream);
 }
 
 // grouped, over a 256-row tile table of max_m_tiles entries

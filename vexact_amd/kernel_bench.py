@@ -7,7 +7,7 @@ out, and the replay is timed with events. Prints time, algorithmic bytes (or flo
 fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
 to run under ``rocprofv3 --pmc``.
 
-    python -m vexact_amd.kernel_bench --what moe,attn,gemm,small,prefill,copy
+    python -m vexact_amd.kernel_bench --what moe,attn,gemm,small,prefill,dense,sampler,copy
 """
 
 from __future__ import annotations
@@ -155,6 +155,23 @@ def main() -> None:
             report(f"prefill gemm {name} M={M} N={N} K={K}", timeit(lambda li: ops.gemm_nt(xx, w_, out=c), n_layers=2),
                    flops=2 * M * N * K)
             del w_, xx, c
+    if "dense" in what:
+        # dense SwiGLU MLP of a Qwen3-8B-shaped layer (hidden 4096, intermediate 12288): fused gate/up, then down
+        Hd, Id = 4096, 12288
+        wg, wu, wd = rnd(Id, Hd), rnd(Id, Hd), rnd(Hd, Id)
+        for M in (256, 8192):
+            xx = rnd(M, Hd, std=1.0)
+            hh = torch.empty(M, Id, dtype=torch.bfloat16, device=dev)
+            yy = torch.empty(M, Hd, dtype=torch.bfloat16, device=dev)
+            t1 = timeit(lambda li: ops.gemm_swiglu(xx, wg, wu, out=hh), n_layers=2)
+            t2 = timeit(lambda li: ops.gemm_nt(hh, wd, out=yy), n_layers=2)
+            if M <= 512:
+                report(f"dense swiglu gate/up M={M}", t1, 2 * Id * Hd * 2 + M * Hd * 2 + M * Id * 2)
+                report(f"dense down M={M}", t2, Id * Hd * 2 + M * Hd * 2 + M * Id * 2)
+            else:
+                report(f"dense swiglu gate/up M={M}", t1, flops=2 * M * 2 * Id * Hd)
+                report(f"dense down M={M}", t2, flops=2 * M * Id * Hd)
+        del wg, wu, wd
     if "prefill" in what:
         # MoE expert GEMMs over a prefill chunk (256-row expert tiles)
         for T in (8192, 32768):

@@ -265,6 +265,30 @@ def gemm_nt_variant(x: torch.Tensor, w_nk: torch.Tensor, kind: int, mt: int = 1,
     return c
 
 
+def gemm_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, out: Optional[torch.Tensor] = None,
+                kind: int = -1, mt: int = 1) -> torch.Tensor:
+    """``silu(x @ w_gate.T) * (x @ w_up.T)`` with every bf16 rounding of the unfused chain, in one
+    kernel. ``x`` [M, K], ``w_gate`` / ``w_up`` [N, K] bf16 with the same row pitch."""
+    _need_gpu("x", x)
+    if not (_fast_ok(x, w_gate) and _fast_ok(x, w_up)) or w_gate.shape != w_up.shape or w_gate.stride(0) != w_up.stride(0):
+        raise ValueError("gemm_swiglu: need K-contiguous, 16-byte aligned bf16 operands; gate and up of one shape and pitch")
+    M, K = x.shape
+    N = w_gate.shape[0]
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    _lib.check(
+        _lib.load().vx_gemm_swiglu_bf16_nt(x.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), out.data_ptr(), M, N, K,
+                                           x.stride(0), w_gate.stride(0), out.stride(0), kind, mt, _stream()),
+        "vx_gemm_swiglu_bf16_nt",
+    )
+    return out
+
+
+def swiglu_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """Dense SwiGLU MLP ``down_proj(act_fn(gate_proj(x)) * up_proj(x))`` in two kernels."""
+    return gemm_nt(gemm_swiglu(x, w_gate, w_up), w_down)
+
+
 def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``a[M,K] @ b[K,N] (+ bias[N])`` with the dtype of ``a``; any strides.
 
