@@ -136,6 +136,32 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
                  int page_size, float softmax_scale, int causal, int mode, int max_seqlen_q,
                  void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
+/* vx_attention that also writes each query row's log-sum-exp, lse [total_q, Hq] fp32 = (m + log2 l) ln 2
+ * as the reference's packed forward saves it (_varlen_attn_fwd_block_kernel,
+ * triton_invariant_attention.py:187-191); +inf for a row without a visible key. Modes 1 and 2 only
+ * (with lse the general kernel is used for every head size; the output bits are the same). */
+int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
+                     const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                     int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                     int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
+                     int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
+                     int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
+                     int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
+/* Backward of causal varlen attention on packed q [Tq, Hq, D], k / v [Tk, Hkv, D] (D = 64 or 128):
+ * dq, dk, dv (bf16) from dout, the forward's out and lse. P and dS are rounded to bf16 before they
+ * enter a matrix product, as in the reference; all sums run in an order fixed by the sequence's own
+ * lengths. strides[16] = token and head strides (elements) of q, k, v, out, dout, dq, dk, dv.
+ * Workspace: vx_attention_bwd_workspace_bytes(total_q, Hq) (the row sums O . dO).
+ * Replaces _varlen_attn_bwd_dq_kernel / _varlen_attn_bwd_dkv_kernel and
+ * _NonpagedFlashAttentionVarlen.backward (triton_invariant_attention.py:193-430, 786-902). */
+int64_t vx_attention_bwd_workspace_bytes(int64_t total_q, int64_t Hq);
+int vx_attention_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                     void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
+                     int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int D,
+                     const int64_t* strides, float softmax_scale, int max_seqlen_q, int max_seqlen_k,
+                     void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
 /* ---- fused MoE ------------------------------------------------------------------------- */
 
 /* softmax(fp32) -> top-k (ties: lower expert first) -> optional renorm -> cast.

@@ -277,3 +277,73 @@ def test_decode_forms_agree_bitwise(qh, kh, dk, dv, page, head_major):
     assert_bitwise(outs["auto"], outs["split"], "auto vs split decode")
     ref = torch.stack([OA.eager_attention(q[i : i + 1].cpu(), k[i], v[i], dk**-0.5)[0] for i in range(len(kv_lens))])
     torch.testing.assert_close(outs["fused"].cpu(), ref, atol=3e-3, rtol=3e-3)
+
+
+def _packed_fwd_bwd(q_seqs, k_seqs, v_seqs, do_seqs):
+    q = torch.cat(q_seqs).cuda().requires_grad_()
+    k = torch.cat(k_seqs).cuda().requires_grad_()
+    v = torch.cat(v_seqs).cuda().requires_grad_()
+    q_lens, kv_lens = [t.shape[0] for t in q_seqs], [t.shape[0] for t in k_seqs]
+    out, _ = flash_attn_varlen_func(q, k, v, cu_seqlens_q=_cu(q_lens).cuda(), cu_seqlens_k=_cu(kv_lens).cuda(),
+                                    max_seqlen_q=max(q_lens), max_seqlen_k=max(kv_lens), causal=True)
+    out.backward(torch.cat(do_seqs).cuda())
+    return out.detach().cpu(), q.grad.cpu(), k.grad.cpu(), v.grad.cpu()
+
+
+@pytest.mark.parametrize(("qh", "kh", "d", "q_lens", "kv_lens"), [
+    (8, 2, 128, [24, 19], [24, 19]),
+    (4, 4, 64, [70, 1, 33], [70, 90, 33]),
+    (8, 1, 128, [130, 5, 64, 1], [130, 200, 64, 65]),
+    (6, 2, 64, [17], [300]),
+])
+def test_packed_backward_matches_autograd_and_is_batch_invariant(qh, kh, d, q_lens, kv_lens):
+    # formulas of the reference's backward kernels (triton_invariant_attention.py:193-430) against
+    # autograd through an fp32 eager attention; P and dS are rounded to bf16 on the GPU
+    print(f"[case] attention backward Hq={qh} Hkv={kh} D={d} q={q_lens} kv={kv_lens}", flush=True)
+    q_seqs, k_seqs, v_seqs = _seqs(q_lens, qh, d, 1), _seqs(kv_lens, kh, d, 2), _seqs(kv_lens, kh, d, 3)
+    do_seqs = _seqs(q_lens, qh, d, 4)
+    out, dq, dk, dv = _packed_fwd_bwd(q_seqs, k_seqs, v_seqs, do_seqs)
+    scale = d ** -0.5
+    o = 0
+    ok = 0
+    for s, (ql, kl) in enumerate(zip(q_lens, kv_lens)):
+        qf, kf, vf = (t.float().requires_grad_() for t in (q_seqs[s], k_seqs[s], v_seqs[s]))
+        g = qh // kh
+        kk, vv = kf.repeat_interleave(g, dim=1), vf.repeat_interleave(g, dim=1)
+        sc = torch.einsum("qhd,khd->hqk", qf, kk) * scale
+        pos = torch.arange(ql) + (kl - ql)
+        mask = torch.arange(kl)[None, :] <= pos[:, None]
+        sc = sc.masked_fill(~mask[None], float("-inf"))
+        ref = torch.einsum("hqk,khd->qhd", torch.softmax(sc, -1), vv)
+        ref.backward(do_seqs[s].float())
+        for name, got, want in (("dq", dq[o : o + ql], qf.grad), ("dk", dk[ok : ok + kl], kf.grad), ("dv", dv[ok : ok + kl], vf.grad)):
+            err = (got.float() - want).abs()
+            tol = 2e-2 * float(want.abs().max())
+            assert float(err.max()) <= tol, f"{name} of sequence {s}: max err {float(err.max()):.4f} > {tol:.4f}"
+            assert float(err.mean()) <= 2e-3 * float(want.abs().max()), f"{name} of sequence {s}: mean err"
+        assert_bf16_close(out[o : o + ql], ref.detach().to(torch.bfloat16), max_ulp=2, atol_frac=3e-3, what=f"out of sequence {s}")
+        # the sequence alone gives the same gradient bits
+        _, dq1, dk1, dv1 = _packed_fwd_bwd(q_seqs[s : s + 1], k_seqs[s : s + 1], v_seqs[s : s + 1], do_seqs[s : s + 1])
+        assert_bitwise(dq1, dq[o : o + ql], f"dq of sequence {s} alone vs in the batch")
+        assert_bitwise(dk1, dk[ok : ok + kl], f"dk of sequence {s} alone vs in the batch")
+        assert_bitwise(dv1, dv[ok : ok + kl], f"dv of sequence {s} alone vs in the batch")
+        o += ql
+        ok += kl
+
+
+def test_packed_forward_with_lse_keeps_the_output_bits():
+    from vexact_amd import ops
+    q_lens, kv_lens = [40, 3, 129], [40, 77, 129]
+    q, k, v = (torch.cat(_seqs(l, h, 128, sd)).cuda() for l, h, sd in ((q_lens, 8, 1), (kv_lens, 2, 2), (kv_lens, 2, 3)))
+    cu_q, cu_k = _cu(q_lens).cuda(), _cu(kv_lens).cuda()
+    plain = ops.packed_attention(q, k, v, cu_q, cu_k, 128 ** -0.5, True, max(q_lens))
+    out, lse = ops.packed_attention(q, k, v, cu_q, cu_k, 128 ** -0.5, True, max(q_lens), return_lse=True)
+    assert_bitwise(out, plain, "output with and without the log-sum-exp")
+    o = ok = 0
+    for ql, kl in zip(q_lens, kv_lens):
+        sc = torch.einsum("qhd,khd->hqk", q[o : o + ql].float().cpu(), k[ok : ok + kl].float().cpu().repeat_interleave(4, dim=1)) * 128 ** -0.5
+        mask = torch.arange(kl)[None, :] <= (torch.arange(ql) + (kl - ql))[:, None]
+        want = torch.logsumexp(sc.masked_fill(~mask[None], float("-inf")), -1).transpose(0, 1)
+        assert float((lse[o : o + ql].cpu() - want).abs().max()) < 2e-3
+        o += ql
+        ok += kl

@@ -2,8 +2,9 @@
 
 Mirrors ``vexact/batch_invariant_ops/triton_invariant_attention.py`` of the reference:
 ``flash_attn_varlen_func`` (:905-979), ``flash_attention_forward`` (:982-1088), the argument checks
-of ``_PagedFlashAttentionVarlen.forward`` (:605-650) and the helpers at :13-44. Forward only: the
-paged path raises on backward like the reference (:694-697); the packed path has no backward here.
+of ``_PagedFlashAttentionVarlen.forward`` (:605-650) and the helpers at :13-44. The paged path raises
+on backward like the reference (:694-697); the packed path has forward and backward
+(``_NonpagedFlashAttentionVarlen``, :700-902).
 """
 
 from __future__ import annotations
@@ -86,6 +87,38 @@ class _PagedAttention(torch.autograd.Function):
         raise NotImplementedError("paged triton flash_attn_varlen_func backward is not implemented")
 
 
+class _PackedAttention(torch.autograd.Function):
+    """Causal varlen attention on packed q/k/v with the HIP forward (log-sum-exp saved) and backward."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, softmax_scale, causal, max_seqlen_q, max_seqlen_k):
+        if q.ndim != 3 or k.ndim != 3 or v.ndim != 3:
+            raise ValueError("non-paged flash_attn_varlen_func expects q/k/v with shape (total_tokens, heads, head_dim)")
+        if q.shape[-1] != k.shape[-1]:
+            raise ValueError(f"q and k head_dim must match, got {q.shape[-1]} and {k.shape[-1]}")
+        if k.shape[-2] != v.shape[-2]:
+            raise ValueError(f"k/v must have the same number of KV heads, got {k.shape[-2]} and {v.shape[-2]}")
+        if q.shape[-2] % k.shape[-2] != 0:
+            raise ValueError(f"query heads ({q.shape[-2]}) must be divisible by KV heads ({k.shape[-2]})")
+        if not causal:
+            raise NotImplementedError("non-paged triton flash_attn_varlen_func only supports causal=True")
+        q, k, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, k, v))
+        out, lse = ops.packed_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, softmax_scale, True, max_seqlen_q,
+                                        return_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k)
+        ctx.softmax_scale, ctx.max_seqlen_q, ctx.max_seqlen_k = softmax_scale, max_seqlen_q, max_seqlen_k
+        return out
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k = ctx.saved_tensors
+        if do.stride(-1) != 1:
+            do = do.contiguous()
+        dq, dk, dv = ops.packed_attention_backward(q, k, v, out, do, lse, cu_seqlens_q, cu_seqlens_k, ctx.softmax_scale,
+                                                   ctx.max_seqlen_q, ctx.max_seqlen_k)
+        return dq, dk, dv, None, None, None, None, None, None
+
+
 def flash_attn_varlen_func(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -129,8 +162,12 @@ def flash_attn_varlen_func(
         _require_cuda("q", q)
         _require_cuda_int32("cu_seqlens_q", cu_seqlens_q)
         _require_cuda_int32("cu_seqlens_k", cu_seqlens_k)
-        if q.requires_grad or k.requires_grad or v.requires_grad:
-            raise NotImplementedError("packed flash_attn_varlen_func is forward-only in this build")
+        if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+            out = _PackedAttention.apply(
+                q, k, v, cu_seqlens_q.contiguous(), cu_seqlens_k.contiguous(), scale, bool(causal),
+                _as_python_int(max_seqlen_q, "max_seqlen_q"), _as_python_int(max_seqlen_k, "max_seqlen_k"),
+            )
+            return out, None
         _as_python_int(max_seqlen_k, "max_seqlen_k")
         out = ops.packed_attention(
             q, k, v, cu_seqlens_q.contiguous(), cu_seqlens_k.contiguous(), scale, bool(causal),

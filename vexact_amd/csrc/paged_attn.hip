@@ -53,6 +53,7 @@ struct AttnParams {
   float* part;
   int64_t img_floats;
   int max_chunks;
+  float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernel only)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -660,6 +661,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw
     if (i >= qlen) continue;
     bf16_t* op = p.o + (int64_t)(q0 + i) * p.sot + (int64_t)head_of[t] * p.soh;
     const bool dead = w.qpos[t] < 0;  // no visible key: define the output as 0
+    // (m + log2 l) ln 2, the form the reference saves for its backward (:187-191); +inf for a dead row
+    // makes every recomputed probability of that row 0
+    if (p.lse && g == 0)
+      p.lse[(int64_t)(q0 + i) * p.Hq + head_of[t]] = dead ? INFINITY : (M[t] + __builtin_amdgcn_logf(L[t])) * 0.6931471824645996f;
 #pragma unroll
     for (int ds = 0; ds < (DV + 127) / 128; ds++)
 #pragma unroll
@@ -993,7 +998,7 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
     while (hpw * 2 <= 4 * QT && G % (hpw * 2) == 0) hpw *= 2;
     const int rpb = 16 * (4 * QT / hpw);
     dim3 grid((rows + rpb - 1) / rpb, p.Hq / hpw, p.num_seqs);
-    if constexpr (DK == 128 && DV == 128) {
+    if constexpr (DK == 128 && DV == 128) if (!p.lse) {
       // K and V through LDS, shared by the 16 query tiles of a block
       int hp = 1;
       while (hp * 2 <= 8 && G % (hp * 2) == 0) hp *= 2;
@@ -1029,6 +1034,14 @@ extern "C" {
 
 int vx_attn_chunk_size() { return ATT_CHUNK; }
 
+int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
+                     const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                     int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                     int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
+                     int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
+                     int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
+                     int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
 // floats of one chunk image: per q-tile (16 heads) and 128-dim set, 8 float4 slots per lane, plus one
 // slot per q-tile for (m, l); 64 lanes x 4 floats per slot
 static inline int64_t part_image_floats(int64_t Hq, int64_t Hkv, int64_t Dv) {
@@ -1054,7 +1067,22 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
                  int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
                  int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
                  int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  return vx_attention_lse(q, k, v, out, nullptr, cu_seqlens_q, seqused_k, cu_seqlens_k, block_table, total_q, num_seqs, Hq,
+                          Hkv, Dk, Dv, sqt, sqh, skb, skp, skh, svb, svp, svh, sot, soh, bt_stride, max_pages, page_size,
+                          softmax_scale, causal, mode, max_seqlen_q, workspace, workspace_bytes, stream);
+}
+
+// vx_attention that also writes the rows' log-sum-exp (lse [total_q, Hq] fp32, natural log; modes 1
+// and 2 only), which the backward needs.
+int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
+                     const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                     int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                     int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
+                     int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
+                     int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
+                     int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (!q || !k || !v || !out || !cu_seqlens_q) return VX_ERR_ARG;
+  if (lse && mode != 1 && mode != 2) return VX_ERR_UNSUPPORTED;
   if (total_q < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return VX_ERR_ARG;
   if (mode < 0 || mode > 4) return VX_ERR_ARG;
   if (mode != 2 && (!seqused_k || !block_table || page_size <= 0 || max_pages <= 0)) return VX_ERR_ARG;
@@ -1083,6 +1111,7 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
   p.Hq = Hq; p.Hkv = Hkv; p.num_seqs = (int)num_seqs;
   p.qk_scale = softmax_scale * 1.44269504f;
   p.causal = causal;
+  p.lse = lse;
   if (decode) {
     const int64_t max_kv = max_pages * (int64_t)page_size;
     const int64_t nch = (max_kv + ATT_CHUNK - 1) / ATT_CHUNK;

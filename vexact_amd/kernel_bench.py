@@ -7,7 +7,7 @@ out, and the replay is timed with events. Prints time, algorithmic bytes (or flo
 fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
 to run under ``rocprofv3 --pmc``.
 
-    python -m vexact_amd.kernel_bench --what moe,attn,gemm,small,prefill,dense,sampler,copy
+    python -m vexact_amd.kernel_bench --what moe,attn,gemm,small,prefill,dense,train,sampler,copy
 """
 
 from __future__ import annotations
@@ -155,6 +155,16 @@ def main() -> None:
             report(f"prefill gemm {name} M={M} N={N} K={K}", timeit(lambda li: ops.gemm_nt(xx, w_, out=c), n_layers=2),
                    flops=2 * M * N * K)
             del w_, xx, c
+    if "train" in what:
+        # training-side attention on packed sequences: forward with log-sum-exp, then backward
+        Hq, Hkv, D, S, Lp = 32, 4, 128, 8, 1024
+        q, kk, vv = rnd(S * Lp, Hq, D, std=1.0), rnd(S * Lp, Hkv, D, std=1.0), rnd(S * Lp, Hkv, D, std=1.0)
+        do = rnd(S * Lp, Hq, D, std=1.0)
+        cu = torch.arange(0, (S + 1) * Lp, Lp, dtype=torch.int32, device=dev)
+        fl = 4 * Hq * D * S * Lp * (Lp + 1) // 2
+        report("packed attention fwd + lse 8 x 1024", timeit(lambda li: ops.packed_attention(q, kk, vv, cu, cu, D**-0.5, True, Lp, return_lse=True), n_layers=2), flops=fl)
+        o, lse = ops.packed_attention(q, kk, vv, cu, cu, D**-0.5, True, Lp, return_lse=True)
+        report("packed attention bwd 8 x 1024", timeit(lambda li: ops.packed_attention_backward(q, kk, vv, o, do, lse, cu, cu, D**-0.5, Lp, Lp), n_layers=2), flops=fl * 5 // 2)
     if "dense" in what:
         # dense SwiGLU MLP of a Qwen3-8B-shaped layer (hidden 4096, intermediate 12288): fused gate/up, then down
         Hd, Id = 4096, 12288

@@ -7,6 +7,7 @@ missing the call raises.
 
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -451,26 +452,62 @@ def packed_attention(
     softmax_scale: float,
     causal: bool,
     max_seqlen_q: int = 0,
-) -> torch.Tensor:
-    """Varlen attention on packed (non-paged) K/V ``[Tk, Hkv, D]``; same arithmetic as the paged path."""
+    return_lse: bool = False,
+):
+    """Varlen attention on packed (non-paged) K/V ``[Tk, Hkv, D]``; same arithmetic as the paged path.
+    ``return_lse`` also returns the rows' fp32 log-sum-exp ``[T, Hq]`` (what the backward needs)."""
     T, Hq, Dk = q.shape
     Hkv, Dv = k.shape[1], v.shape[-1]
     o = torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
+    lse = torch.empty((T, Hq), dtype=torch.float32, device=q.device) if return_lse else None
     if T == 0:
-        return o
+        return (o, lse) if return_lse else o
     if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
         raise ValueError("attention supports bfloat16 q/k/v only")
     B = cu_seqlens_q.numel() - 1
     _lib.check(
-        _lib.load().vx_attention(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), cu_seqlens_q.data_ptr(), None,
+        _lib.load().vx_attention_lse(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(lse), cu_seqlens_q.data_ptr(), None,
             cu_seqlens_k.data_ptr(), None, T, B, Hq, Hkv, Dk, Dv, q.stride(0), q.stride(1),
             0, k.stride(0), k.stride(1), 0, v.stride(0), v.stride(1), o.stride(0), o.stride(1),
             0, 0, 0, float(softmax_scale), 1 if causal else 0, 2, int(max_seqlen_q), None, 0, _stream(),
         ),
         "vx_attention",
     )
-    return o
+    return (o, lse) if return_lse else o
+
+
+def packed_attention_backward(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
+    cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, softmax_scale: float, max_seqlen_q: int, max_seqlen_k: int,
+):
+    """(dq, dk, dv) of causal ``packed_attention`` (bf16, shapes of q, k, v)."""
+    for name, t in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)):
+        _need_gpu(name, t)
+        if t.dtype != torch.bfloat16 or t.dim() != 3 or t.stride(2) != 1:
+            raise ValueError(f"attention backward: {name} must be bf16 [tokens, heads, dim] with a contiguous last dim")
+    T, Hq, D = q.shape
+    Tk, Hkv, Dv = v.shape
+    if D != Dv or k.shape != (Tk, Hkv, D) or D not in (64, 128):
+        raise ValueError(f"attention backward supports equal q/k/v head sizes of 64 or 128, got {D} and {Dv}")
+    if lse.dtype != torch.float32 or lse.shape != (T, Hq) or not lse.is_contiguous():
+        raise ValueError("attention backward: lse must be a contiguous fp32 [tokens, heads] tensor")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if T == 0 or Tk == 0:
+        return dq.zero_(), dk.zero_(), dv.zero_()
+    lib = _lib.load()
+    ws = _workspace(lib.vx_attention_bwd_workspace_bytes(T, Hq), q.device)
+    strides = (ctypes.c_int64 * 16)(*[s for t in (q, k, v, out, dout, dq, dk, dv) for s in (t.stride(0), t.stride(1))])
+    _lib.check(
+        lib.vx_attention_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), dq.data_ptr(),
+            dk.data_ptr(), dv.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), T, Tk,
+            cu_seqlens_q.numel() - 1, Hq, Hkv, D, strides, float(softmax_scale), int(max_seqlen_q), int(max_seqlen_k),
+            ws.data_ptr(), ws.numel(), _stream(),
+        ),
+        "vx_attention_bwd",
+    )
+    return dq, dk, dv
 
 
 # ----------------------------------------------------------------------------- MoE
