@@ -138,8 +138,7 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
 
 /* vx_attention that also writes each query row's log-sum-exp, lse [total_q, Hq] fp32 = (m + log2 l) ln 2
  * as the reference's packed forward saves it (_varlen_attn_fwd_block_kernel,
- * triton_invariant_attention.py:187-191); +inf for a row without a visible key. Modes 1 and 2 only
- * (with lse the general kernel is used for every head size; the output bits are the same). */
+ * triton_invariant_attention.py:187-191); +inf for a row without a visible key. Modes 1 and 2 only. */
 int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
                      const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
                      int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,

@@ -5,7 +5,9 @@ Mirrors ``fused_moe_forward`` of ``vexact/batch_invariant_ops/fused_moe.py:459-4
 (``vexact/models/qwen3_moe/modeling_qwen3_moe.py:89-100``). Arithmetic follows
 ``FusedMoeExpertFunction.forward`` (fused_moe.py:24-102): bf16 gate/up projections, bf16
 ``silu(g) * u``, routing weight applied before the down projection, fp32 sum over a token's slots
-in slot order. Forward only.
+in slot order. The backward (``FusedMoeExpertFunction.backward``, fused_moe.py:126-265) recomputes
+the gate / up projections with the same grouped kernel and runs the dgrad / wgrad products as plain
+per-expert library GEMMs: only the forward has to match the rollout bit for bit.
 """
 
 from __future__ import annotations
@@ -32,6 +34,70 @@ def _split_weights(fc1_1_weight, fc1_2_weight, fc1_1_2_weight):
     return fc1_1_weight, fc1_2_weight
 
 
+class FusedMoeExpertFunction(torch.autograd.Function):
+    """Forward on the HIP kernels (bit-identical to the inference path); backward with the formulas
+    of the reference's ``FusedMoeExpertFunction.backward`` (fused_moe.py:126-265). Gradients for the
+    routing weights, the hidden states and the three expert weights."""
+
+    @staticmethod
+    def forward(ctx, num_experts, routing_weights, selected_experts, hidden_states, gate_w, up_w, down_w):
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
+        out = ops.fused_moe(x, routing_weights.reshape(x.shape[0], -1), selected_experts.reshape(x.shape[0], -1),
+                            gate_w, up_w, down_w, num_experts)
+        ctx.num_experts = num_experts
+        ctx.save_for_backward(routing_weights, selected_experts, hidden_states, gate_w, up_w, down_w)
+        return out.reshape(hidden_states.shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        routing_weights, selected_experts, hidden_states, gate_w, up_w, down_w = ctx.saved_tensors
+        E = ctx.num_experts
+        H = hidden_states.shape[-1]
+        x = hidden_states.reshape(-1, H)
+        T, k = x.shape[0], selected_experts.reshape(x.shape[0], -1).shape[1]
+        dy = grad_output.reshape(-1, H).to(torch.bfloat16)
+        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=False))
+        tok = r.sorted_token.long()                      # token of each expert-sorted row
+        flat = r.sorted_flat.long()                      # (token, slot) flat index of each sorted row
+        # recomputed with the forward's kernels, so these are the values the forward used
+        g = ops.moe_gemm(x, gate_w, r, row_src=r.sorted_token)
+        u = ops.moe_gemm(x, up_w, r, row_src=r.sorted_token)
+        a = torch.ops.aten.silu(g)
+        act = a * u
+        w_sorted = routing_weights.reshape(-1)[flat].unsqueeze(1)
+        hw = act * w_sorted
+        xs, dys = x[tok], dy[tok]
+        cu = r.cu.cpu().tolist()                         # host copy: the products below are per-expert library calls
+        d_hw = torch.empty_like(hw)
+        d_g_w = torch.zeros_like(gate_w) if ctx.needs_input_grad[4] else None
+        d_u_w = torch.zeros_like(up_w) if ctx.needs_input_grad[5] else None
+        d_d_w = torch.zeros_like(down_w) if ctx.needs_input_grad[6] else None
+        for e in range(E):
+            lo, hi = cu[e], cu[e + 1]
+            if hi > lo:
+                d_hw[lo:hi] = dys[lo:hi] @ down_w[e]                               # dgrad of the down projection
+                if d_d_w is not None:
+                    d_d_w[e] = dys[lo:hi].t() @ hw[lo:hi]
+        d_act = d_hw * w_sorted
+        d_w_sorted = torch.sum(act * d_hw, dim=-1)
+        grad_rw = torch.empty_like(d_w_sorted)
+        grad_rw[flat] = d_w_sorted
+        d_a, d_u = d_act * u, a * d_act
+        d_g = torch.ops.aten.silu_backward(d_a, g)
+        d_xs = torch.empty_like(xs)
+        for e in range(E):
+            lo, hi = cu[e], cu[e + 1]
+            if hi > lo:
+                d_xs[lo:hi] = d_g[lo:hi] @ gate_w[e] + d_u[lo:hi] @ up_w[e]
+                if d_g_w is not None:
+                    d_g_w[e] = d_g[lo:hi].t() @ xs[lo:hi]
+                if d_u_w is not None:
+                    d_u_w[e] = d_u[lo:hi].t() @ xs[lo:hi]
+        d_x = ops.moe_gather(d_xs, r.scatter_index)
+        return (None, grad_rw.reshape(routing_weights.shape).to(routing_weights.dtype), None,
+                d_x.reshape(hidden_states.shape), d_g_w, d_u_w, d_d_w)
+
+
 def fused_moe_forward(
     num_experts: int,
     routing_weights: torch.Tensor,
@@ -54,6 +120,9 @@ def fused_moe_forward(
     if down_w.stride(2) != 1:
         down_w = down_w.contiguous()
     shape = hidden_states.shape
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (routing_weights, hidden_states, gate_w, up_w, down_w)):
+        return FusedMoeExpertFunction.apply(num_experts, routing_weights, selected_experts, hidden_states, gate_w, up_w,
+                                            down_w)
     x = hidden_states.reshape(-1, shape[-1])
     out = ops.fused_moe(
         x, routing_weights.reshape(x.shape[0], -1), selected_experts.reshape(x.shape[0], -1), gate_w, up_w, down_w,

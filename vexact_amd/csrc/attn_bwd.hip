@@ -51,26 +51,35 @@ __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnBwdParams p, in
   p.delta[i] = s;
 }
 
-// acc[td] (rows = dims 8 r16' + td, cols = stationary) += (moving rows 0..63, transposed) x pf.
-// rowp(r) = pointer to moving row r of the block (clamped to an existing row; its weight in pf is 0).
+// The moving rows of a 64-row block in the layout the transposed products read: slot idx of half ch
+// holds row 32 ch + 16 (idx / 4) + 4 g + idx % 4, dims 8 r16 .. +8 (16 lanes cover a 256-byte row).
+// rowp(r) = pointer to moving row r of the block, clamped to an existing row (its weight is 0).
 template <int D, class RowPtr>
-__device__ __forceinline__ void bwd_tr_product(RowPtr rowp, const uint4 (&pf)[2], f32x4 (&acc)[8]) {
+__device__ __forceinline__ void bwd_tr_load(RowPtr rowp, uint4 (&rows)[2][8]) {
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const bool dok = 8 * r16 < D;
 #pragma unroll
-  for (int ch = 0; ch < 2; ch++) {
-    uint4 row[8];
+  for (int ch = 0; ch < 2; ch++)
 #pragma unroll
     for (int idx = 0; idx < 8; idx++) {
       const int r = 32 * ch + 16 * (idx >> 2) + 4 * g + (idx & 3);
-      row[idx] = mask16(ldg16_raw(rowp(r) + (dok ? 8 * r16 : 0)), dok);
+      rows[ch][idx] = ldg16_raw(rowp(r) + (dok ? 8 * r16 : 0));
     }
+}
+
+// acc[td] (rows = dims 8 r16' + td, cols = stationary) += (moving rows 0..63, transposed) x pf
+template <int D>
+__device__ __forceinline__ void bwd_tr_product(const uint4 (&rows)[2][8], const uint4 (&pf)[2], f32x4 (&acc)[8]) {
+  const int r16 = threadIdx.x & 15;
+  const bool dok = 8 * r16 < D;
+#pragma unroll
+  for (int ch = 0; ch < 2; ch++) {
 #pragma unroll
     for (int td = 0; td < 8; td++) {
       uint32_t w[4];
 #pragma unroll
       for (int qd = 0; qd < 4; qd++) {
-        const uint4 ra = row[2 * qd], rb = row[2 * qd + 1];
+        const uint4 ra = mask16(rows[ch][2 * qd], dok), rb = mask16(rows[ch][2 * qd + 1], dok);
         const uint32_t a = (td < 2) ? ra.x : (td < 4) ? ra.y : (td < 6) ? ra.z : ra.w;
         const uint32_t b = (td < 2) ? rb.x : (td < 4) ? rb.y : (td < 6) ? rb.z : rb.w;
         w[qd] = (td & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
@@ -148,17 +157,28 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
   const bf16_t* kb_ = p.k + (int64_t)k0 * p.skt + (int64_t)kvh * p.skh;
   const bf16_t* vb_ = p.v + (int64_t)k0 * p.svt + (int64_t)kvh * p.svh;
   for (int kb = 0; kb <= maxpos; kb += 64) {
-    float ds[4][4];
+    // every load of the block is issued before the first is used: one memory round trip per block
+    uint4 kfr[4][KS], vfr[4][KS], rows[2][8];
 #pragma unroll
     for (int tt = 0; tt < 4; tt++) {
       const int64_t kr = min(kb + 16 * tt + r16, kv_len - 1);
       const bf16_t* kp = kb_ + kr * p.skt + 8 * g;
       const bf16_t* vp = vb_ + kr * p.svt + 8 * g;
+#pragma unroll
+      for (int s = 0; s < KS; s++) {
+        kfr[tt][s] = ldg16_raw(kp + 32 * s);
+        vfr[tt][s] = ldg16_raw(vp + 32 * s);
+      }
+    }
+    bwd_tr_load<D>([&](int r) { return kb_ + (int64_t)min(kb + r, kv_len - 1) * p.skt; }, rows);
+    float ds[4][4];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++) {
       f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f}, dp = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < KS; s++) {
-        st = mfma16(ldg16_raw(kp + 32 * s), qf[s], st);
-        dp = mfma16(ldg16_raw(vp + 32 * s), of[s], dp);
+        st = mfma16(kfr[tt][s], qf[s], st);
+        dp = mfma16(vfr[tt][s], of[s], dp);
       }
 #pragma unroll
       for (int r = 0; r < 4; r++) {
@@ -169,7 +189,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
     }
     uint4 pf[2];
     bwd_pack(ds, pf);
-    bwd_tr_product<D>([&](int r) { return kb_ + (int64_t)min(kb + r, kv_len - 1) * p.skt; }, pf, acc);
+    bwd_tr_product<D>(rows, pf, acc);
   }
   if (qok) bwd_store_tile<D>(acc, p.dq + tq * p.sdqt + (int64_t)h * p.sdqh);
 }
@@ -214,35 +234,53 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnBwdParams p) {
       const bf16_t* qb_ = p.q + (int64_t)q0 * p.sqt + (int64_t)h * p.sqh;
       const bf16_t* db_ = p.d_o + (int64_t)q0 * p.sdt + (int64_t)h * p.sdh;
       for (int ib = istart; ib < qlen; ib += 64) {
-        float pr[4][4], ds[4][4];
+        // phase 1: the block's Q and dO rows as A operands plus the rows' lse and delta, all loads first
+        uint4 qfr[4][KS], ofr[4][KS];
+        float lse2[4][4], dl[4][4];
 #pragma unroll
         for (int tt = 0; tt < 4; tt++) {
           const int64_t ir = min(ib + 16 * tt + r16, qlen - 1);
           const bf16_t* qp = qb_ + ir * p.sqt + 8 * g;
           const bf16_t* dp_ = db_ + ir * p.sdt + 8 * g;
+#pragma unroll
+          for (int s = 0; s < KS; s++) {
+            qfr[tt][s] = ldg16_raw(qp + 32 * s);
+            ofr[tt][s] = ldg16_raw(dp_ + 32 * s);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const int64_t tq = q0 + min(ib + 16 * tt + 4 * g + r, qlen - 1);
+            lse2[tt][r] = p.lse[tq * p.Hq + h];
+            dl[tt][r] = p.delta[tq * p.Hq + h];
+          }
+        }
+        float pr[4][4], ds[4][4];
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) {
           f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f}, dp = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int s = 0; s < KS; s++) {
-            st = mfma16(ldg16_raw(qp + 32 * s), kf[s], st);
-            dp = mfma16(ldg16_raw(dp_ + 32 * s), vf[s], dp);
+            st = mfma16(qfr[tt][s], kf[s], st);
+            dp = mfma16(ofr[tt][s], vf[s], dp);
           }
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             const int iq = ib + 16 * tt + 4 * g + r;    // this register's query (moving row)
             const bool ok = iq < qlen && kok && j <= shift + iq;
-            const int64_t tq = q0 + min(iq, qlen - 1);
-            const float lse2 = p.lse[tq * p.Hq + h] * 1.44269504f;
-            const float delta = p.delta[tq * p.Hq + h];
-            const float e = ok ? __builtin_amdgcn_exp2f(st[r] * c2 - lse2) : 0.f;
+            const float e = ok ? __builtin_amdgcn_exp2f(st[r] * c2 - lse2[tt][r] * 1.44269504f) : 0.f;
             pr[tt][r] = e;
-            ds[tt][r] = e * (dp[r] - delta) * p.scale;
+            ds[tt][r] = e * (dp[r] - dl[tt][r]) * p.scale;
           }
         }
+        // phase 2: the same rows in the transposable layout (they are in the cache now)
+        uint4 rows_o[2][8], rows_q[2][8];
+        bwd_tr_load<D>([&](int r) { return db_ + (int64_t)min(ib + r, qlen - 1) * p.sdt; }, rows_o);
+        bwd_tr_load<D>([&](int r) { return qb_ + (int64_t)min(ib + r, qlen - 1) * p.sqt; }, rows_q);
         uint4 pfp[2], pfs[2];
         bwd_pack(pr, pfp);
         bwd_pack(ds, pfs);
-        bwd_tr_product<D>([&](int r) { return db_ + (int64_t)min(ib + r, qlen - 1) * p.sdt; }, pfp, dv);
-        bwd_tr_product<D>([&](int r) { return qb_ + (int64_t)min(ib + r, qlen - 1) * p.sqt; }, pfs, dk);
+        bwd_tr_product<D>(rows_o, pfp, dv);
+        bwd_tr_product<D>(rows_q, pfs, dk);
       }
     }
   }

@@ -53,7 +53,7 @@ struct AttnParams {
   float* part;
   int64_t img_floats;
   int max_chunks;
-  float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernel only)
+  float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernels)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -898,6 +898,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
     if (i >= qlen) continue;
     bf16_t* op = p.o + (int64_t)(q0 + i) * p.sot + (int64_t)head_of[t] * p.soh;
     const bool dead = qpos[t] < 0;
+    if (p.lse && g == 0)
+      p.lse[(int64_t)(q0 + i) * p.Hq + head_of[t]] = dead ? INFINITY : (M[t] + __builtin_amdgcn_logf(L[t])) * 0.6931471824645996f;
 #pragma unroll
     for (int f = 0; f < 8; f++) {
       uint2 pk;
@@ -998,7 +1000,7 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
     while (hpw * 2 <= 4 * QT && G % (hpw * 2) == 0) hpw *= 2;
     const int rpb = 16 * (4 * QT / hpw);
     dim3 grid((rows + rpb - 1) / rpb, p.Hq / hpw, p.num_seqs);
-    if constexpr (DK == 128 && DV == 128) if (!p.lse) {
+    if constexpr (DK == 128 && DV == 128) {
       // K and V through LDS, shared by the 16 query tiles of a block
       int hp = 1;
       while (hp * 2 <= 8 && G % (hp * 2) == 0) hp *= 2;
