@@ -44,11 +44,79 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--seed", type=int, default=5)
+    ap.add_argument("--cpu-configs", action="store_true",
+                    help="time the CPU oracle on the reference's other configurations (op chain, decode attention, "
+                         "chunked prefill, fused MoE) instead of running the GPU benchmark; prints one JSON line")
     return ap.parse_args()
+
+
+def cpu_configs(seed):
+    """CPU legs of the reference configurations C1 - C4: the oracle (torch CPU restatement) timed on this
+    host's cores at the full shapes (chunked prefill: 2 of the 16 sequences, scaled by the work)."""
+    import numpy as np
+    import torch
+
+    from oracle import attention as OA
+    from oracle import moe as OM
+    from oracle.row_ops import hf_rms_norm_ref, log_softmax_ref, matmul_ref
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+
+    def timed(fn, reps=2):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    res = {"cores": cores, "kind": "port"}
+    # C1: RMSNorm -> lm_head -> fp32 log_softmax, H = 2048, V = 151936
+    H, V = 2048, 151936
+    wl, wn = rnd(V, H, std=0.02), (1 + 0.02 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    for M in (1, 64):
+        x = rnd(M, H)
+        res[f"C1 op chain M={M} (s)"] = round(timed(lambda: log_softmax_ref(matmul_ref(hf_rms_norm_ref(x, wn), wl.t()).float())), 4)
+    del wl
+    # C2: decode attention, 64 sequences, context 128..4096, Hq = 16, Hkv = 8, D = 128, page 16
+    rng = np.random.default_rng(2)
+    L = rng.integers(128, 4097, size=64)
+    k_seqs = [rnd(int(n), 8, 128) for n in L]
+    v_seqs = [rnd(int(n), 8, 128) for n in L]
+    kc, vc, table = OA.make_paged_kv_cache(k_seqs, v_seqs, 16)
+    q = rnd(64, 16, 128)
+    cu = torch.arange(65, dtype=torch.int32)
+    used = torch.tensor(L, dtype=torch.int32)
+    res["C2 decode attention B=64 (s)"] = round(timed(lambda: OA.paged_attention_ref(q, kc, vc, cu, used, table, 128 ** -0.5)), 4)
+    del kc, vc, k_seqs, v_seqs
+    # C3: chunked prefill, 512-token chunks on prefixes 0..8192, Hq = 32, Hkv = 8: 2 of 16 sequences
+    prefix = np.random.default_rng(3).integers(0, 8193, size=16)
+    work = lambda P: 512 * P + 512 * 513 // 2  # noqa: E731
+    sub = [int(prefix[0]), int(prefix[1])]
+    qs = [rnd(512, 32, 128) for _ in sub]
+    ks = [rnd(P + 512, 8, 128) for P in sub]
+    vs = [rnd(P + 512, 8, 128) for P in sub]
+    t = timed(lambda: [OA.eager_attention(a, b, c, 128 ** -0.5) for a, b, c in zip(qs, ks, vs)], reps=1)
+    res["C3 chunked prefill 16 x 512 (s, scaled from 2 sequences)"] = round(t * sum(work(int(P)) for P in prefix) / sum(work(P) for P in sub), 3)
+    # C4: fused MoE block, H = 2048, I = 768, 128 experts, top-8
+    E, k, I = 128, 8, 768
+    gw, uw, dw = rnd(E, I, H, std=0.02), rnd(E, I, H, std=0.02), rnd(E, H, I, std=0.02)
+    for T in (1, 64, 256):
+        x = rnd(T, H)
+        w, idx = OM.router_ref(torch.randn(T, E, generator=g), k)
+        res[f"C4 fused MoE T={T} (s)"] = round(timed(lambda: OM.fused_moe_ref(x, w, idx, gw, uw, dw), reps=1), 4)
+    print(json.dumps({"cpu_configs": res}), flush=True)
 
 
 def main():
     args = parse()
+    if args.cpu_configs:
+        cpu_configs(args.seed)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (all pipeline stages collapsed onto one MI355X); "
               "--gpus must be 1", file=sys.stderr)
