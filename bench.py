@@ -239,7 +239,7 @@ def main():
                                    cfg.head_dim, cfg.rms_eps)
             timed("attn_decode", lambda: ops.paged_attention(db.q, dec.key_cache[li], dec.value_cache[li], db.query_start_loc,
                                                              db.context_lens, db.block_tables, scale, 1, out=db.attn,
-                                                             workspace=db.attn_ws))
+                                                             workspace=db.attn_ws, seq_order=db.seq_order))
             timed("o_gemm", lambda: ops.gemm_nt(db.attn.view(B, -1), lw["o"], out=db.o))
             ops.rms_norm(db.o, lw["post_norm"], cfg.rms_eps, hf_two_rounding=True, residual=db.x, sum_out=db.x, out=db.h)
             ops.gemm_nt(db.h, lw["router"], out=db.router_logits)

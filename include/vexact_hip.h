@@ -136,16 +136,20 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
                  int page_size, float softmax_scale, int causal, int mode, int max_seqlen_q,
                  void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
-/* vx_attention that also writes each query row's log-sum-exp, lse [total_q, Hq] fp32 = (m + log2 l) ln 2
- * as the reference's packed forward saves it (_varlen_attn_fwd_block_kernel,
- * triton_invariant_attention.py:187-191); +inf for a row without a visible key. Modes 1 and 2 only. */
-int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
-                     const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
-                     int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
-                     int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
-                     int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
-                     int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
-                     int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+/* vx_attention with two optional extras.
+ * lse [total_q, Hq] fp32 (modes 1 and 2): each query row's log-sum-exp (m + log2 l) ln 2, as the
+ * reference's packed forward saves it (_varlen_attn_fwd_block_kernel,
+ * triton_invariant_attention.py:187-191); +inf for a row without a visible key.
+ * seq_order [num_seqs] int32 (decode modes 0, 3, 4): a permutation of the sequences; workgroup i of
+ * the decode kernels takes sequence seq_order[i]. Longest context first shortens the tail of a batch
+ * with mixed lengths; the results do not depend on it. (No counterpart in the reference.) */
+int vx_attention_ex(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
+                    const int* cu_seqlens_q, const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                    int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                    int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
+                    int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
+                    int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
+                    int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 /* Backward of causal varlen attention on packed q [Tq, Hq, D], k / v [Tk, Hkv, D] (D = 64 or 128):
  * dq, dk, dv (bf16) from dout, the forward's out and lse. P and dS are rounded to bf16 before they
@@ -249,7 +253,9 @@ int vx_sample_tokens(const void* logits, int dtype, int64_t ld, int64_t rows, in
  * Request s has context length num_computed[s] AFTER this step, tokens_this_step[s] query tokens
  * and the block ids block_ids[block_offsets[s] .. block_offsets[s + 1]). Padding: tokens past the
  * step get slot -1 / position 0; sequences past it get query_start_loc = total tokens, context
- * length 0 and an all-zero block-table row; unused entries of real rows are -1.
+ * length 0 and an all-zero block-table row; unused entries of real rows are -1. seq_order [cap_seqs]
+ * (optional) receives the sequences by context length, longest first (ties and padding in index
+ * order), for vx_attention_ex.
  * Replaces _prepare_gen_ctx (vexact/inferencer/inferencer.py:193-291) and the static-buffer padding
  * of prepare_cudagraph_gen_ctx (inferencer.py:306-324) in one pass. VX_ERR_ARG if the step does not
  * fit the bucket or a request's blocks do not cover its context. */
@@ -257,7 +263,7 @@ int vx_host_step_metadata(int64_t num_reqs, const int64_t* num_computed, const i
                           const int32_t* block_ids, const int64_t* block_offsets, int32_t page_size,
                           int64_t max_blocks, int64_t cap_tokens, int64_t cap_seqs, int64_t* positions,
                           int32_t* slot_mapping, int32_t* query_start_loc, int32_t* context_lens,
-                          int32_t* block_tables, int64_t* total_tokens, int32_t* max_seqlen_q);
+                          int32_t* block_tables, int32_t* seq_order, int64_t* total_tokens, int32_t* max_seqlen_q);
 
 /* Block allocator that always hands out the lowest free ids (KVCacheManager,
  * vexact/batch_invariant_ops/kv_cache_context.py:141-217). allocate: the blocks a request holding

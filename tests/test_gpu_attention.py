@@ -275,6 +275,11 @@ def test_decode_forms_agree_bitwise(qh, kh, dk, dv, page, head_major):
             for kind in ("split", "fused", "auto")}
     assert_bitwise(outs["fused"], outs["split"], "fused vs split decode")
     assert_bitwise(outs["auto"], outs["split"], "auto vs split decode")
+    # the order in which the workgroups take the sequences (longest first) does not change a bit
+    order = torch.tensor(sorted(range(len(kv_lens)), key=lambda i: (-kv_lens[i], i)), dtype=torch.int32).cuda()
+    for kind in ("split", "fused"):
+        assert_bitwise(ops.paged_attention(q, kc, vc, cu, used, table.cuda(), dk**-0.5, 1, decode_kernel=kind, seq_order=order),
+                       outs["split"], f"{kind} decode with a sequence order")
     ref = torch.stack([OA.eager_attention(q[i : i + 1].cpu(), k[i], v[i], dk**-0.5)[0] for i in range(len(kv_lens))])
     torch.testing.assert_close(outs["fused"].cpu(), ref, atol=3e-3, rtol=3e-3)
 

@@ -67,6 +67,7 @@ def test_bucket_padding_rules():
     assert np.array_equal(b.context_lens.numpy(), ref["context_lens"])
     assert np.array_equal(b.block_tables.numpy(), ref["block_tables"])
     assert np.array_equal(b.query_start_loc.numpy(), ref["query_start_loc"])
+    assert b.seq_order.tolist() == sorted(range(8), key=lambda s: (-int(ref["context_lens"][s]), s))
     with pytest.raises(ValueError, match="total_tokens exceeds capture_tokens"):
         StepBuffers(cfg, 2, 8, "cpu").load(meta, np.array([1, 2, 3]))
     with pytest.raises(ValueError, match="graph_num_seqs cannot be smaller than num_seqs"):
@@ -95,6 +96,9 @@ def test_native_builder_pads_like_the_two_step_restatement():
         for k in ("slot_mapping", "positions", "context_lens", "block_tables", "query_start_loc"):
             assert np.array_equal(getattr(b, k).numpy(), ref[k]), (n, k)
         assert b.input_ids.tolist() == ids.tolist() + [0] * (cap_t - T)
+        # longest context first, ties and padding in index order
+        lens = ref["context_lens"]
+        assert b.seq_order.tolist() == sorted(range(cap_s), key=lambda s: (-int(lens[s]), s))
 
 
 def test_native_builder_rejects_inconsistent_steps():

@@ -34,9 +34,9 @@ PROTOTYPES = {
         _I,
         [_P] * 8 + [_L, _L, _I, _I, _I, _I] + [_L] * 12 + [_I, _F, _I, _I, _I, _P, _L, _P],
     ),
-    "vx_attention_lse": (
+    "vx_attention_ex": (
         _I,
-        [_P] * 9 + [_L, _L, _I, _I, _I, _I] + [_L] * 12 + [_I, _F, _I, _I, _I, _P, _L, _P],
+        [_P] * 10 + [_L, _L, _I, _I, _I, _I] + [_L] * 12 + [_I, _F, _I, _I, _I, _P, _L, _P],
     ),
     "vx_attention_bwd_workspace_bytes": (_L, [_L, _L]),
     "vx_attention_bwd": (_I, [_P] * 11 + [_L, _L, _L, _I, _I, _I, _P, _F, _I, _I, _P, _L, _P]),
@@ -58,7 +58,7 @@ PROTOTYPES = {
     "vx_embedding": (_I, [_P, _P, _I, _P, _L, _L, _L, _P]),
     "vx_fill_i32": (_I, [_P, _I, _L, _P]),
     "vx_sample_tokens": (_I, [_P, _I, _L, _L, _L, _F, _I, _F, _P, _P, _P, _P]),
-    "vx_host_step_metadata": (_I, [_L, _P, _P, _P, _P, _I, _L, _L, _L] + [_P] * 7),
+    "vx_host_step_metadata": (_I, [_L, _P, _P, _P, _P, _I, _L, _L, _L] + [_P] * 8),
     "vx_kv_allocator_create": (_P, [_L]),
     "vx_kv_allocator_destroy": (None, [_P]),
     "vx_kv_allocator_num_free": (_L, [_P]),

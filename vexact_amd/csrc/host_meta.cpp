@@ -25,6 +25,8 @@ extern "C" {
 // [cap_seqs + 1], context_lens [cap_seqs], block_tables [cap_seqs, max_blocks]. Padding: tokens past
 // the step get slot -1 and position 0; sequences past the step get query_start_loc = total tokens,
 // context length 0 and an all-zero block-table row; unused block-table entries of real rows are -1.
+// seq_order [cap_seqs] (optional) receives the sequences sorted by context length, longest first,
+// ties and padding in index order: the order in which the decode attention kernel should take them.
 // Returns VX_OK and the step's token count / longest query in *total_tokens / *max_seqlen_q, or
 // VX_ERR_ARG when the step does not fit the bucket, a request has too few blocks for its context,
 // or its counts are inconsistent.
@@ -32,7 +34,7 @@ int vx_host_step_metadata(int64_t num_reqs, const int64_t* num_computed, const i
                           const int32_t* block_ids, const int64_t* block_offsets, int32_t page_size,
                           int64_t max_blocks, int64_t cap_tokens, int64_t cap_seqs, int64_t* positions,
                           int32_t* slot_mapping, int32_t* query_start_loc, int32_t* context_lens,
-                          int32_t* block_tables, int64_t* total_tokens, int32_t* max_seqlen_q) {
+                          int32_t* block_tables, int32_t* seq_order, int64_t* total_tokens, int32_t* max_seqlen_q) {
   if (num_reqs < 0 || page_size <= 0 || max_blocks <= 0 || cap_tokens < 0 || cap_seqs < num_reqs) return VX_ERR_ARG;
   if (!positions || !slot_mapping || !query_start_loc || !context_lens || !block_tables) return VX_ERR_ARG;
   if (num_reqs > 0 && (!num_computed || !tokens_this_step || !block_ids || !block_offsets)) return VX_ERR_ARG;
@@ -73,6 +75,11 @@ int vx_host_step_metadata(int64_t num_reqs, const int64_t* num_computed, const i
     query_start_loc[s + 1] = (int32_t)total;
     context_lens[s] = 0;
     std::fill(block_tables + s * max_blocks, block_tables + (s + 1) * max_blocks, 0);
+  }
+  if (seq_order) {
+    for (int64_t s = 0; s < cap_seqs; s++) seq_order[s] = (int32_t)s;
+    std::stable_sort(seq_order, seq_order + cap_seqs,
+                     [&](int32_t a, int32_t b) { return context_lens[a] > context_lens[b]; });
   }
   if (total_tokens) *total_tokens = total;
   if (max_seqlen_q) *max_seqlen_q = (int32_t)maxq;

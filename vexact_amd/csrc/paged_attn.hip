@@ -53,6 +53,7 @@ struct AttnParams {
   float* part;
   int64_t img_floats;
   int max_chunks;
+  const int* seq_order;  // optional [B]: decode kernels take sequence seq_order[i] as their i-th (longest first balances the tail)
   float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernels)
 };
 
@@ -338,7 +339,7 @@ __device__ __forceinline__ KVSource<KIND> make_source(const AttnParams& p, int s
 // ---------------------------------------------------------------------------------------
 template <int DK, int DV, int QT, int KIND>
 __device__ __forceinline__ void attn_decode_split_body(const AttnParams& p) {
-  const int kvh = blockIdx.x, seq = blockIdx.y, chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
+  const int kvh = blockIdx.x, seq = p.seq_order ? p.seq_order[blockIdx.y] : (int)blockIdx.y, chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
@@ -418,7 +419,7 @@ __device__ __forceinline__ void attn_decode_fused_body(const AttnParams& p) {
   float4* racc = img + NW * IMG4;                   // [MAXE] running accumulators
   float2* rml = (float2*)(racc + MAXE);             // [MAXE] running (M, L), one private copy per element
 
-  const int kvh = blockIdx.x, seq = blockIdx.y;
+  const int kvh = blockIdx.x, seq = p.seq_order ? p.seq_order[blockIdx.y] : (int)blockIdx.y;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
@@ -527,7 +528,7 @@ constexpr int fused_lds_bytes() {
 // 128 ds + 32 g + 8 r + (0..7), reads its own slots of every image and writes 16 bytes per (ds, r).
 template <int DV, int QT>
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
-  const int kvh = blockIdx.x, seq = blockIdx.y;
+  const int kvh = blockIdx.x, seq = p.seq_order ? p.seq_order[blockIdx.y] : (int)blockIdx.y;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
@@ -1036,7 +1037,8 @@ extern "C" {
 
 int vx_attn_chunk_size() { return ATT_CHUNK; }
 
-int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
+int vx_attention_ex(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
+                    const int* cu_seqlens_q,
                      const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
                      int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
                      int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
@@ -1069,14 +1071,16 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
                  int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
                  int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
                  int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
-  return vx_attention_lse(q, k, v, out, nullptr, cu_seqlens_q, seqused_k, cu_seqlens_k, block_table, total_q, num_seqs, Hq,
+  return vx_attention_ex(q, k, v, out, nullptr, nullptr, cu_seqlens_q, seqused_k, cu_seqlens_k, block_table, total_q, num_seqs, Hq,
                           Hkv, Dk, Dv, sqt, sqh, skb, skp, skh, svb, svp, svh, sot, soh, bt_stride, max_pages, page_size,
                           softmax_scale, causal, mode, max_seqlen_q, workspace, workspace_bytes, stream);
 }
 
-// vx_attention that also writes the rows' log-sum-exp (lse [total_q, Hq] fp32, natural log; modes 1
-// and 2 only), which the backward needs.
-int vx_attention_lse(const void* q, const void* k, const void* v, void* out, float* lse, const int* cu_seqlens_q,
+// vx_attention with two optional extras: lse [total_q, Hq] fp32 (natural log; modes 1 and 2 only) receives
+// the rows' log-sum-exp, which the backward needs; seq_order [num_seqs] (decode modes) is a permutation
+// of the sequences in which the decode kernels take them, e.g. longest context first.
+int vx_attention_ex(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
+                    const int* cu_seqlens_q,
                      const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
                      int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
                      int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
@@ -1085,6 +1089,7 @@ int vx_attention_lse(const void* q, const void* k, const void* v, void* out, flo
                      int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (!q || !k || !v || !out || !cu_seqlens_q) return VX_ERR_ARG;
   if (lse && mode != 1 && mode != 2) return VX_ERR_UNSUPPORTED;
+  if (seq_order && (mode == 1 || mode == 2)) return VX_ERR_UNSUPPORTED;
   if (total_q < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return VX_ERR_ARG;
   if (mode < 0 || mode > 4) return VX_ERR_ARG;
   if (mode != 2 && (!seqused_k || !block_table || page_size <= 0 || max_pages <= 0)) return VX_ERR_ARG;
@@ -1114,6 +1119,7 @@ int vx_attention_lse(const void* q, const void* k, const void* v, void* out, flo
   p.qk_scale = softmax_scale * 1.44269504f;
   p.causal = causal;
   p.lse = lse;
+  p.seq_order = seq_order;
   if (decode) {
     const int64_t max_kv = max_pages * (int64_t)page_size;
     const int64_t nch = (max_kv + ATT_CHUNK - 1) / ATT_CHUNK;

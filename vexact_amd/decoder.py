@@ -144,7 +144,7 @@ def _flatten_requests(requests: Sequence[dict]):
     return done, n_tok, ids, offs
 
 
-def _native_step_metadata(requests, page_size, max_blocks, cap_tokens, cap_seqs, positions, slot, qsl, lens, bt):
+def _native_step_metadata(requests, page_size, max_blocks, cap_tokens, cap_seqs, positions, slot, qsl, lens, bt, order=None):
     """One call of ``vx_host_step_metadata`` writing into the given host addresses (ints)."""
     from . import _lib
 
@@ -152,7 +152,7 @@ def _native_step_metadata(requests, page_size, max_blocks, cap_tokens, cap_seqs,
     total, maxq = ctypes.c_int64(0), ctypes.c_int32(0)
     rc = _lib.load().vx_host_step_metadata(
         len(requests), done.ctypes.data, n_tok.ctypes.data, ids.ctypes.data, offs.ctypes.data, page_size, max_blocks,
-        cap_tokens, cap_seqs, positions, slot, qsl, lens, bt, ctypes.byref(total), ctypes.byref(maxq))
+        cap_tokens, cap_seqs, positions, slot, qsl, lens, bt, order, ctypes.byref(total), ctypes.byref(maxq))
     if rc != 0:
         # say which of the reference's conditions failed (inferencer.py:306-311), else the generic message
         if len(requests) > cap_seqs:
@@ -210,7 +210,8 @@ class StepBuffers:
         # buffer with the same layout, so that a step costs one host-to-device copy.
         mb = self.max_blocks
         segs = (("positions", i64, (T,)), ("input_ids", i64, (T,)), ("slot_mapping", i32, (T,)),
-                ("query_start_loc", i32, (B + 1,)), ("context_lens", i32, (B,)), ("block_tables", i32, (B, mb)))
+                ("query_start_loc", i32, (B + 1,)), ("context_lens", i32, (B,)), ("seq_order", i32, (B,)),
+                ("block_tables", i32, (B, mb)))
         offs, end = {}, 0
         for name, dt, shape in segs:
             offs[name] = end
@@ -226,6 +227,7 @@ class StepBuffers:
         self._host_ptr = {k: v.ctypes.data for k, v in self._host.items()}
         self._host["slot_mapping"].fill(-1)
         self._host["block_tables"].fill(-1)
+        self._host["seq_order"][:] = np.arange(B)
         self.meta_dev.copy_(self.meta_host)
         H, k = cfg.hidden_size, cfg.top_k
         self.x = z(T, H, dtype=bf)
@@ -274,6 +276,7 @@ class StepBuffers:
         h["block_tables"][:B, :w] = meta["block_tables"][:, :w]
         h["context_lens"][:B] = meta["context_lens"]; h["context_lens"][B:] = 0
         h["query_start_loc"][: B + 1] = meta["query_start_loc"]; h["query_start_loc"][B + 1:] = T
+        h["seq_order"][:] = np.argsort(-h["context_lens"], kind="stable")  # longest context first
         return self._commit(T, B, input_ids)
 
     def load_requests(self, requests: Sequence[dict], input_ids: np.ndarray, page_size: int) -> tuple[int, int, int]:
@@ -282,7 +285,7 @@ class StepBuffers:
         p = self._host_ptr
         T, maxq = _native_step_metadata(requests, page_size, self.max_blocks, self.num_tokens, self.num_seqs,
                                         p["positions"], p["slot_mapping"], p["query_start_loc"], p["context_lens"],
-                                        p["block_tables"])
+                                        p["block_tables"], p["seq_order"])
         if len(input_ids) != T:
             raise ValueError(f"{len(input_ids)} input ids for a step of {T} tokens")
         self._commit(T, len(requests), input_ids)
@@ -332,7 +335,8 @@ class Qwen3MoeDecoder:
                                    b.q, self.key_cache[li], self.value_cache[li], cfg.num_heads, cfg.num_kv_heads,
                                    cfg.head_dim, cfg.rms_eps)
             ops.paged_attention(b.q, self.key_cache[li], self.value_cache[li], b.query_start_loc, b.context_lens,
-                                b.block_tables, scale, max_seqlen_q, out=b.attn, workspace=b.attn_ws)
+                                b.block_tables, scale, max_seqlen_q, out=b.attn, workspace=b.attn_ws,
+                                seq_order=b.seq_order if max_seqlen_q == 1 else None)
             ops.gemm_nt(b.attn.view(b.num_tokens, -1), lw["o"], out=b.o)
             # x <- x + o ; h <- post_norm(x)
             ops.rms_norm(b.o, lw["post_norm"], cfg.rms_eps, hf_two_rounding=True, residual=b.x, sum_out=b.x, out=b.h)

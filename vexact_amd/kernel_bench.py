@@ -131,11 +131,13 @@ def main() -> None:
         q = rnd(B, Hq, D, std=1.0)
         cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
         used = torch.tensor(L, dtype=torch.int32, device=dev)
+        order = torch.tensor(np.argsort(-L, kind="stable").astype(np.int32), device=dev)  # longest first, as the host builder emits
         btd = torch.tensor(bt, device=dev)
         out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
         ws = torch.empty(_lib.load().vx_paged_attn_decode_workspace_bytes(B, Hq, Hkv, D, 4096), dtype=torch.uint8, device=dev)
         report(f"paged decode attention (sum L={int(L.sum())})",
-               timeit(lambda li: ops.paged_attention(q, kc[li], vc[li], cu, used, btd, D**-0.5, 1, out=out, workspace=ws)),
+               timeit(lambda li: ops.paged_attention(q, kc[li], vc[li], cu, used, btd, D**-0.5, 1, out=out, workspace=ws,
+                                                     seq_order=order)),
                int(L.sum()) * 2 * Hkv * D * 2 + 2 * B * Hq * D * 2 + sum(pages) * 4)
     if "gemm" in what:
         for name, N, K in (("qkv", 5120, 2048), ("o", 2048, 4096), ("router", 128, 2048), ("lm_head", 151936, 2048)):
@@ -298,8 +300,9 @@ def main() -> None:
         used = torch.tensor(L, dtype=torch.int32, device=dev)
         btd = torch.tensor(bt, device=dev)
         out = torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev)
+        order = torch.tensor(np.argsort(-L, kind="stable").astype(np.int32), device=dev)  # what the host metadata builder emits
         report(f"C2 decode attention B=64 (sum L={int(L.sum())})",
-               timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, btd, D**-0.5, 1, out=out), n_layers=2),
+               timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, btd, D**-0.5, 1, out=out, seq_order=order), n_layers=2),
                int(L.sum()) * 2 * Hkv * D * 2 + 2 * S * Hq * D * 2 + sum(pages) * 4)
         del kc, vc
         # C4: fused MoE block at T tokens

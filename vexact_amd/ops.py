@@ -406,11 +406,14 @@ def paged_attention(
     out: Optional[torch.Tensor] = None,
     workspace: Optional[torch.Tensor] = None,
     decode_kernel: str = "auto",
+    seq_order: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal paged attention. ``max_seqlen_q == 1`` selects the split-KV decode kernels; any other
     value the general kernel (identical bits per row). ``decode_kernel`` forces one of the two decode
     forms ("split": one wavefront per 256-key chunk plus a combine launch, "fused": chunks folded
-    inside one workgroup per (sequence, kv head)); "auto" picks by batch size. Same bits either way."""
+    inside one workgroup per (sequence, kv head)); "auto" picks by batch size. Same bits either way.
+    ``seq_order`` (int32 permutation of the sequences, decode only) is the order in which the decode
+    workgroups take the sequences; longest first shortens the tail of a batch of mixed lengths."""
     T, Hq, Dk = q.shape
     Hkv, Dv = k_cache.shape[2], v_cache.shape[-1]
     o = out if out is not None else torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
@@ -429,10 +432,13 @@ def paged_attention(
     if mode != 1:
         need = lib.vx_paged_attn_decode_workspace_bytes(B, Hq, Hkv, Dv, max_pages * page)
         ws = workspace if workspace is not None and workspace.numel() * workspace.element_size() >= need else _workspace(need, q.device)
+    if seq_order is not None and (mode == 1 or seq_order.dtype != torch.int32 or seq_order.numel() != B
+                                  or not seq_order.is_contiguous()):
+        raise ValueError("seq_order must be a contiguous int32 permutation of the sequences, for decode steps only")
     _lib.check(
-        lib.vx_attention(
-            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr(), cu_seqlens_q.data_ptr(),
-            seqused_k.data_ptr(), None, page_table.data_ptr(), T, B, Hq, Hkv, Dk, Dv,
+        lib.vx_attention_ex(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr(), None, _ptr(seq_order),
+            cu_seqlens_q.data_ptr(), seqused_k.data_ptr(), None, page_table.data_ptr(), T, B, Hq, Hkv, Dk, Dv,
             q.stride(0), q.stride(1), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
             v_cache.stride(0), v_cache.stride(1), v_cache.stride(2), o.stride(0), o.stride(1),
             page_table.stride(0), max_pages, page, float(softmax_scale), 1, mode, int(max_seqlen_q),
@@ -466,8 +472,8 @@ def packed_attention(
         raise ValueError("attention supports bfloat16 q/k/v only")
     B = cu_seqlens_q.numel() - 1
     _lib.check(
-        _lib.load().vx_attention_lse(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(lse), cu_seqlens_q.data_ptr(), None,
+        _lib.load().vx_attention_ex(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(lse), None, cu_seqlens_q.data_ptr(), None,
             cu_seqlens_k.data_ptr(), None, T, B, Hq, Hkv, Dk, Dv, q.stride(0), q.stride(1),
             0, k.stride(0), k.stride(1), 0, v.stride(0), v.stride(1), o.stride(0), o.stride(1),
             0, 0, 0, float(softmax_scale), 1 if causal else 0, 2, int(max_seqlen_q), None, 0, _stream(),
