@@ -30,25 +30,28 @@ struct AttnBwdParams {
   float scale;
 };
 
-// delta[t, h] = sum_d f32(O[t, h, d]) f32(dO[t, h, d]), ascending d
+// delta[t, h] = sum_d f32(O[t, h, d]) f32(dO[t, h, d]): 16 lanes per (token, head) row, 8 dims each,
+// then a fixed butterfly over the 16 lanes
 template <int D>
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnBwdParams p, int64_t total_q) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= total_q * p.Hq) return;
-  const int64_t t = i / p.Hq;
-  const int h = (int)(i % p.Hq);
-  const bf16_t* op = p.o + t * p.sot + (int64_t)h * p.soh;
-  const bf16_t* dp = p.d_o + t * p.sdt + (int64_t)h * p.sdh;
+  const int64_t i = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int c = threadIdx.x & 15;
+  const bool live = i < total_q * p.Hq;
+  const int64_t ii = live ? i : 0;
+  const int64_t t = ii / p.Hq;
+  const int h = (int)(ii % p.Hq);
   float s = 0.f;
-#pragma unroll
-  for (int d = 0; d < D; d += 8) {
-    const uint4 a = ldg16_raw(op + d), b = ldg16_raw(dp + d);
+  if (8 * c < D) {
+    const uint4 a = ldg16_raw(p.o + t * p.sot + (int64_t)h * p.soh + 8 * c);
+    const uint4 b = ldg16_raw(p.d_o + t * p.sdt + (int64_t)h * p.sdh + 8 * c);
     s += bf16lo(a.x) * bf16lo(b.x); s += bf16hi(a.x) * bf16hi(b.x);
     s += bf16lo(a.y) * bf16lo(b.y); s += bf16hi(a.y) * bf16hi(b.y);
     s += bf16lo(a.z) * bf16lo(b.z); s += bf16hi(a.z) * bf16hi(b.z);
     s += bf16lo(a.w) * bf16lo(b.w); s += bf16hi(a.w) * bf16hi(b.w);
   }
-  p.delta[i] = s;
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+  if (live && c == 0) p.delta[i] = s;
 }
 
 // The moving rows of a 64-row block in the layout the transposed products read: slot idx of half ch
@@ -290,11 +293,288 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnBwdParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Head size 128: the moving side goes through LDS once per workgroup. 8 wavefronts hold 8 stationary
+// tiles (128 queries of one head for dQ); every 64-row block of the two moving arrays (K and V) is
+// brought in by direct-to-LDS loads into one of two 32 KB stages while the previous block is being
+// used. Rows are 256 bytes with 16-byte piece c of row r stored at piece c ^ (r & 15): the 16-byte
+// fragment reads (A operands of the score products) and the transposing 8-byte reads
+// (ds_read_b64_tr_b16, A operands of the products that contract over the moving rows) are both
+// free of bank conflicts, and the transposing reads deliver the rows in the k-slot order in which
+// P / dS sit in the accumulator registers, so there are no register transposes.
+// The accumulator of fragment f holds dims 16 f + 4 g + r of the lane's stationary row.
+// ---------------------------------------------------------------------------------------
+constexpr int BWL_WAVES = 8;
+constexpr int BWL_ARR = 64 * 256;          // one 64-row array
+constexpr int BWL_STAGE = 2 * BWL_ARR;     // two arrays per stage
+constexpr int BWL_LDS = 2 * BWL_STAGE;     // two stages
+typedef short bw_v4s_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* bw_lds_ptr_t;
+
+// wavefront `wave` of NW brings rows [64 / NW * wave, +64 / NW) of a 64-row array into LDS: 4 rows per instruction
+template <int NW = BWL_WAVES>
+__device__ __forceinline__ void bwl_issue_rows(const bf16_t* base, int64_t row_stride, int first_row, int last_row,
+                                               uint32_t lds_arr, int wave) {
+  const int lane = threadIdx.x & 63;
+  constexpr int RPW = 64 / NW;
+#pragma unroll
+  for (int j = 0; j < RPW / 4; j++) {
+    const int row = RPW * wave + 4 * j + (lane >> 4);
+    const int piece = (lane & 15) ^ (row & 15);
+    const bf16_t* src = base + (int64_t)min(first_row + row, last_row) * row_stride + 8 * piece;
+    const uint32_t dst = lds_arr + (RPW * wave + 4 * j) * 256;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+  }
+}
+// A operand of a score product: row 16 tt + r16 of the array, dims 32 s + 8 g .. +8
+__device__ __forceinline__ uint4 bwl_frag(const uint8_t* arr, int tt, int s) {
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int row = 16 * tt + r16;
+  return *(const uint4*)(arr + row * 256 + (((4 * s + g) ^ (row & 15)) * 16));
+}
+// acc[f] (rows = dims 16 f + .., cols = stationary) += (array rows, transposed) x pf
+__device__ __forceinline__ void bwl_tr_product(const uint8_t* arr, const uint4 (&pf)[2], f32x4 (&acc)[8]) {
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int ch = 0; ch < 2; ch++) {
+#pragma unroll
+    for (int f = 0; f < 8; f++) {
+      const int byte = 32 * f + 8 * (r16 & 3);
+      const int row_lo = 32 * ch + 4 * g + (r16 >> 2), row_hi = row_lo + 16;
+      const bw_v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) bw_v4s_t*)(arr + row_lo * 256 + (((byte >> 4) ^ (row_lo & 15)) * 16) + (byte & 15)));
+      const bw_v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) bw_v4s_t*)(arr + row_hi * 256 + (((byte >> 4) ^ (row_hi & 15)) * 16) + (byte & 15)));
+      const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+      acc[f] = mfma16(make_uint4(lo2.x, lo2.y, hi2.x, hi2.y), pf[ch], acc[f]);
+    }
+  }
+}
+// lane (g, c): acc[f][r] = element (dim 16 f + 4 g + r) of stationary row c
+__device__ __forceinline__ void bwl_store_tile(const f32x4 (&acc)[8], bf16_t* rowp) {
+  const int g = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int f = 0; f < 8; f++) {
+    uint2 pk;
+    pk.x = pack_bf16x2(acc[f][0], acc[f][1]);
+    pk.y = pack_bf16x2(acc[f][2], acc[f][3]);
+    *(uint2*)(rowp + 16 * f + 4 * g) = pk;
+  }
+}
+
+// dQ, head size 128: grid (ceil(max_q / 128), Hq, sequences), 512 threads
+__global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwdParams p) {
+  constexpr int KS = 4;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t bw_lds[];
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int q0 = p.cu_q[seq], qlen = p.cu_q[seq + 1] - q0;
+  const int k0 = p.cu_k[seq], kv_len = p.cu_k[seq + 1] - k0;
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i_base = blockIdx.x * (16 * BWL_WAVES);
+  if (i_base >= qlen || kv_len <= 0) return;  // uniform over the block
+  const int kvh = h / (p.Hq / p.Hkv);
+  const int shift = kv_len - qlen;
+  // last key any query of the block sees (uniform): every wavefront walks the blocks up to it
+  const int blk_maxpos = min(shift + min(i_base + 16 * BWL_WAVES, qlen) - 1, kv_len - 1);
+  const int i = i_base + 16 * wave + r16;       // this lane's query
+  const bool qok = i < qlen;
+  const int pos = qok ? shift + i : -1;
+  const int64_t tq = q0 + (qok ? i : qlen - 1);
+  uint4 qf[KS], of[KS];
+  {
+    const bf16_t* qp = p.q + tq * p.sqt + (int64_t)h * p.sqh + 8 * g;
+    const bf16_t* dp = p.d_o + tq * p.sdt + (int64_t)h * p.sdh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      qf[s] = ldg16_raw(qp + 32 * s);
+      of[s] = ldg16_raw(dp + 32 * s);
+    }
+  }
+  const float c2 = p.scale * 1.44269504f;
+  const float lse2 = p.lse[tq * p.Hq + h] * 1.44269504f;
+  const float delta = p.delta[tq * p.Hq + h];
+  int wave_maxpos = pos;  // last key this wavefront's queries see
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) wave_maxpos = max(wave_maxpos, __shfl_xor(wave_maxpos, o, 64));
+  f32x4 acc[8];
+#pragma unroll
+  for (int f = 0; f < 8; f++) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // the registers above must be loaded before the first direct-to-LDS load is counted
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  const bf16_t* kb_ = p.k + (int64_t)k0 * p.skt + (int64_t)kvh * p.skh;
+  const bf16_t* vb_ = p.v + (int64_t)k0 * p.svt + (int64_t)kvh * p.svh;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(bw_lds_ptr_t)bw_lds;
+  auto issue_block = [&](int kb, int stage) {
+    bwl_issue_rows(kb_, p.skt, kb, kv_len - 1, lds0 + stage * BWL_STAGE, wave);
+    bwl_issue_rows(vb_, p.svt, kb, kv_len - 1, lds0 + stage * BWL_STAGE + BWL_ARR, wave);
+  };
+  if (blk_maxpos >= 0) issue_block(0, 0);
+  for (int kb = 0, stage = 0; kb <= blk_maxpos; kb += 64, stage ^= 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // block kb is in LDS for everyone; everyone is done with the other stage
+    if (kb + 64 <= blk_maxpos) issue_block(kb + 64, stage ^ 1);
+    if (kb > wave_maxpos) continue;  // nothing visible to this wavefront any more (it keeps loading and syncing)
+    const uint8_t* ks = bw_lds + stage * BWL_STAGE;
+    const uint8_t* vs = ks + BWL_ARR;
+    float ds[4][4];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++) {
+      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f}, dp = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; s++) {
+        st = mfma16(bwl_frag(ks, tt, s), qf[s], st);
+        dp = mfma16(bwl_frag(vs, tt, s), of[s], dp);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int key = kb + 16 * tt + 4 * g + r;
+        const float pr = (key <= pos) ? __builtin_amdgcn_exp2f(st[r] * c2 - lse2) : 0.f;
+        ds[tt][r] = pr * (dp[r] - delta) * p.scale;
+      }
+    }
+    uint4 pf[2];
+    bwd_pack(ds, pf);
+    bwl_tr_product(ks, pf, acc);
+  }
+  if (qok) bwl_store_tile(acc, p.dq + tq * p.sdqt + (int64_t)h * p.sdqh);
+}
+
+// dK, dV, head size 128: grid (ceil(max_k / (16 NW)), Hkv, sequences), NW wavefronts. The moving side is
+// the queries of the kv head's query heads, one head after the other: Q and dO blocks plus the
+// 64 rows' lse and delta per stage.
+constexpr int BWK_STAGE = 2 * BWL_ARR + 1024;  // Q, dO, then 64 lse and 64 delta values
+constexpr int BWK_LDS = 2 * BWK_STAGE;
+constexpr int BWK_WAVES = 8;  // 128 keys per workgroup (64-key workgroups measured slower: 470 vs 404 us on 8 x 1024 tokens)
+
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams p) {
+  constexpr int KS = 4;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t bw_lds[];
+  const int seq = blockIdx.z, kvh = blockIdx.y;
+  const int q0 = p.cu_q[seq], qlen = p.cu_q[seq + 1] - q0;
+  const int k0 = p.cu_k[seq], kv_len = p.cu_k[seq + 1] - k0;
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j_base = blockIdx.x * (16 * NW);
+  if (j_base >= kv_len) return;  // uniform over the block
+  const int G = p.Hq / p.Hkv;
+  const int shift = kv_len - qlen;
+  const int j0 = j_base + 16 * wave;            // first key of this wavefront's tile
+  const int j = j0 + r16;                       // this lane's key
+  const bool kok = j < kv_len;
+  const int64_t tk = k0 + (kok ? j : kv_len - 1);
+  uint4 kf[KS], vf[KS];
+  {
+    const bf16_t* kp = p.k + tk * p.skt + (int64_t)kvh * p.skh + 8 * g;
+    const bf16_t* vp = p.v + tk * p.svt + (int64_t)kvh * p.svh + 8 * g;
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+      kf[s] = ldg16_raw(kp + 32 * s);
+      vf[s] = ldg16_raw(vp + 32 * s);
+    }
+  }
+  const float c2 = p.scale * 1.44269504f;
+  f32x4 dk[8], dv[8];
+#pragma unroll
+  for (int f = 0; f < 8; f++) {
+    dk[f] = f32x4{0.f, 0.f, 0.f, 0.f};
+    dv[f] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // first query that sees the block's first key; the moving blocks start there
+  const int ib0 = max(0, j_base - shift);
+  const int nblk = qlen > ib0 ? (qlen - ib0 + 63) / 64 : 0;
+  const int nsteps = nblk * G;  // query heads one after the other
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(bw_lds_ptr_t)bw_lds;
+  auto issue_step = [&](int step, int stage) {
+    const int h = kvh * G + step / nblk, ib = ib0 + 64 * (step % nblk);
+    const uint32_t sb = lds0 + stage * BWK_STAGE;
+    bwl_issue_rows<NW>(p.q + (int64_t)q0 * p.sqt + (int64_t)h * p.sqh, p.sqt, ib, qlen - 1, sb, wave);
+    bwl_issue_rows<NW>(p.d_o + (int64_t)q0 * p.sdt + (int64_t)h * p.sdh, p.sdt, ib, qlen - 1, sb + BWL_ARR, wave);
+    if (wave < 2) {  // 64 lse values (wavefront 0) and 64 delta values (wavefront 1), one dword per lane
+      const float* src = (wave == 0 ? p.lse : p.delta) + (int64_t)(q0 + min(ib + lane, qlen - 1)) * p.Hq + h;
+      const uint32_t dst = sb + 2 * BWL_ARR + wave * 256;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+    }
+  };
+  if (nsteps > 0) issue_step(0, 0);
+  for (int step = 0, stage = 0; step < nsteps; step++, stage ^= 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // this step's rows are in LDS for everyone; everyone is done with the other stage
+    if (step + 1 < nsteps) issue_step(step + 1, stage ^ 1);
+    const int ib = ib0 + 64 * (step % nblk);
+    if (ib + 63 + shift < j0) continue;  // none of the block's queries sees any key of this wavefront's tile
+    const uint8_t* qs = bw_lds + stage * BWK_STAGE;
+    const uint8_t* os = qs + BWL_ARR;
+    const float* lse_s = (const float*)(os + BWL_ARR);
+    const float* del_s = lse_s + 64;
+    float pr[4][4], ds[4][4];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++) {
+      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f}, dp = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; s++) {
+        st = mfma16(bwl_frag(qs, tt, s), kf[s], st);
+        dp = mfma16(bwl_frag(os, tt, s), vf[s], dp);
+      }
+      const float4 l4 = *(const float4*)(lse_s + 16 * tt + 4 * g);
+      const float4 d4 = *(const float4*)(del_s + 16 * tt + 4 * g);
+      const float lr[4] = {l4.x, l4.y, l4.z, l4.w}, dr[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int iq = ib + 16 * tt + 4 * g + r;  // this register's query (moving row)
+        const bool ok = iq < qlen && kok && j <= shift + iq;
+        const float e = ok ? __builtin_amdgcn_exp2f(st[r] * c2 - lr[r] * 1.44269504f) : 0.f;
+        pr[tt][r] = e;
+        ds[tt][r] = e * (dp[r] - dr[r]) * p.scale;
+      }
+    }
+    uint4 pfp[2], pfs[2];
+    bwd_pack(pr, pfp);
+    bwd_pack(ds, pfs);
+    bwl_tr_product(os, pfp, dv);
+    bwl_tr_product(qs, pfs, dk);
+  }
+  if (kok) {
+    bwl_store_tile(dk, p.dk + tk * p.sdkt + (int64_t)kvh * p.sdkh);
+    bwl_store_tile(dv, p.dv + tk * p.sdvt + (int64_t)kvh * p.sdvh);
+  }
+}
+
 template <int D>
 static int launch_attn_bwd(const AttnBwdParams& p, int64_t total_q, int num_seqs, int max_q, int max_k, hipStream_t stream) {
-  attn_bwd_delta_kernel<D><<<(unsigned)((total_q * p.Hq + 255) / 256), 256, 0, stream>>>(p, total_q);
-  attn_bwd_dq_kernel<D><<<dim3((unsigned)((max_q + 63) / 64), (unsigned)p.Hq, (unsigned)num_seqs), 256, 0, stream>>>(p);
-  attn_bwd_dkv_kernel<D><<<dim3((unsigned)((max_k + 63) / 64), (unsigned)p.Hkv, (unsigned)num_seqs), 256, 0, stream>>>(p);
+  attn_bwd_delta_kernel<D><<<(unsigned)((total_q * p.Hq + 15) / 16), 256, 0, stream>>>(p, total_q);
+  if constexpr (D == 128) {
+    static bool attr_set = false;
+    if (!attr_set) {
+      if (hipFuncSetAttribute((const void*)attn_bwd_dq_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, BWL_LDS) != hipSuccess) {
+        (void)hipGetLastError();
+        return VX_ERR_LAUNCH;
+      }
+      attr_set = true;
+    }
+    attn_bwd_dq_lds_kernel<<<dim3((unsigned)((max_q + 16 * BWL_WAVES - 1) / (16 * BWL_WAVES)), (unsigned)p.Hq, (unsigned)num_seqs),
+                             64 * BWL_WAVES, BWL_LDS, stream>>>(p);
+  } else {
+    attn_bwd_dq_kernel<D><<<dim3((unsigned)((max_q + 63) / 64), (unsigned)p.Hq, (unsigned)num_seqs), 256, 0, stream>>>(p);
+  }
+  if constexpr (D == 128) {
+    static bool attr_set2 = false;
+    if (!attr_set2) {
+      if (hipFuncSetAttribute((const void*)attn_bwd_dkv_lds_kernel<BWK_WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, BWK_LDS) != hipSuccess) {
+        (void)hipGetLastError();
+        return VX_ERR_LAUNCH;
+      }
+      attr_set2 = true;
+    }
+    attn_bwd_dkv_lds_kernel<BWK_WAVES><<<dim3((unsigned)((max_k + 16 * BWK_WAVES - 1) / (16 * BWK_WAVES)), (unsigned)p.Hkv, (unsigned)num_seqs),
+                                         64 * BWK_WAVES, BWK_LDS, stream>>>(p);
+  } else {
+    attn_bwd_dkv_kernel<D><<<dim3((unsigned)((max_k + 63) / 64), (unsigned)p.Hkv, (unsigned)num_seqs), 256, 0, stream>>>(p);
+  }
   return launch_status();
 }
 
@@ -322,7 +602,7 @@ int vx_attention_bwd(const void* q, const void* k, const void* v, const void* ou
        (uintptr_t)dv) % 16 != 0)
     return VX_ERR_UNSUPPORTED;
   if (!workspace || workspace_bytes < total_q * Hq * 4 || ((uintptr_t)workspace & 15)) return VX_ERR_WORKSPACE;
-  if (total_q * Hq > 0x7fffffffLL * 256) return VX_ERR_ARG;
+  if (total_q * Hq > 0x7fffffffLL * 16) return VX_ERR_ARG;
   AttnBwdParams p = {};
   p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.o = (const bf16_t*)out;
   p.d_o = (const bf16_t*)dout; p.lse = lse; p.delta = (float*)workspace;
