@@ -189,6 +189,6 @@ const char* vx_status_string(int code) {
   }
 }
 
-int vx_abi_version() { return 2; }
+int vx_abi_version() { return 3; }
 
 }  // extern "C"

@@ -59,6 +59,11 @@ struct AttnParams {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// sequence handled by decode workgroup i (clamped: a bad order entry must not become a wild address)
+__device__ __forceinline__ int decode_seq(const AttnParams& p, unsigned i) {
+  return p.seq_order ? min(max(p.seq_order[i], 0), p.num_seqs - 1) : (int)i;
+}
+
 // Where a sequence's keys and values live. SRC_FAST: paged, page size a power of two >= 16, so a
 // 16-key tile lies inside one page and its page id is wave-uniform. SRC_GENERIC: paged, any page
 // size (one table lookup per key). SRC_PACKED: contiguous rows [Tk, Hkv, D].
@@ -339,7 +344,7 @@ __device__ __forceinline__ KVSource<KIND> make_source(const AttnParams& p, int s
 // ---------------------------------------------------------------------------------------
 template <int DK, int DV, int QT, int KIND>
 __device__ __forceinline__ void attn_decode_split_body(const AttnParams& p) {
-  const int kvh = blockIdx.x, seq = p.seq_order ? p.seq_order[blockIdx.y] : (int)blockIdx.y, chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
+  const int kvh = blockIdx.x, seq = decode_seq(p, blockIdx.y), chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
@@ -419,7 +424,7 @@ __device__ __forceinline__ void attn_decode_fused_body(const AttnParams& p) {
   float4* racc = img + NW * IMG4;                   // [MAXE] running accumulators
   float2* rml = (float2*)(racc + MAXE);             // [MAXE] running (M, L), one private copy per element
 
-  const int kvh = blockIdx.x, seq = p.seq_order ? p.seq_order[blockIdx.y] : (int)blockIdx.y;
+  const int kvh = blockIdx.x, seq = decode_seq(p, blockIdx.y);
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
@@ -528,7 +533,7 @@ constexpr int fused_lds_bytes() {
 // 128 ds + 32 g + 8 r + (0..7), reads its own slots of every image and writes 16 bytes per (ds, r).
 template <int DV, int QT>
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
-  const int kvh = blockIdx.x, seq = p.seq_order ? p.seq_order[blockIdx.y] : (int)blockIdx.y;
+  const int kvh = blockIdx.x, seq = decode_seq(p, blockIdx.y);
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = p.seqused_k[seq];
