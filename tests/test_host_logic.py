@@ -207,3 +207,21 @@ def test_ops_refuse_cpu_tensors_and_bad_arguments():
         matmul_persistent(torch.zeros(2, 3), torch.zeros(3, 5, dtype=torch.bfloat16))
     with pytest.raises(AssertionError, match="Expected 3D tensors"):
         triton_bmm(torch.zeros(2, 3), torch.zeros(3, 5))
+
+
+def test_sampler_argument_errors_need_no_gpu():
+    # the reference's error cases (tests/test_inferencer_sampling.py:88-130) are raised before any device work
+    from vexact_amd.inferencer.sampler import Sampler
+
+    def cfg(**kw):
+        c = types.SimpleNamespace(do_sample=True, temperature=1.0, top_k=4, top_p=1.0)
+        c.__dict__.update(kw)
+        return c
+
+    s, logits = Sampler(), torch.randn(2, 16)
+    with pytest.raises(ValueError, match="every request in the batch"):
+        s.batch_sample_token(logits, [cfg(seed=1234), cfg()], torch.arange(2))
+    with pytest.raises(ValueError, match="sampling_positions must be set"):
+        s.batch_sample_token(logits, [cfg(seed=1), cfg(seed=2)])
+    with pytest.raises(AssertionError, match="top_p must be set"):
+        s.batch_sample_token(logits, [cfg(top_p=None)] * 2)
