@@ -122,29 +122,28 @@ template <int NACC>
 __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float c, int qpos, float& m, float& l,
                                                   f32x4 (&acc)[NACC], uint4 (&pf)[2], bool all_visible = false) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
+  // The block maximum is taken over the raw scores and scaled once: x -> fl(x c) is monotone for
+  // c > 0, so fl(max(s) c) = max(fl(s c)); the exponent argument is then one fused multiply-add.
   float bm = -INFINITY;
   if (all_visible) {  // wave-uniform: every key of the block is visible to every row of the tile
 #pragma unroll
     for (int tt = 0; tt < 4; tt++)
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        st[tt][r] = st[tt][r] * c;
-        bm = fmaxf(bm, st[tt][r]);
-      }
+      for (int r = 0; r < 4; r++) bm = fmaxf(bm, st[tt][r]);
   } else {
 #pragma unroll
     for (int tt = 0; tt < 4; tt++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const int key = kb + 16 * tt + 4 * g + r;
-        float tv = st[tt][r] * c;
-        tv = (key <= qpos) ? tv : -INFINITY;
+        const float tv = (key <= qpos) ? st[tt][r] : -INFINITY;  // exp2(fma(-inf, c, .)) = 0 below
         st[tt][r] = tv;
         bm = fmaxf(bm, tv);
       }
   }
   bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
   bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+  bm = bm * c;
   const float mn = fmaxf(m, bm);
   const float ms = (mn == -INFINITY) ? 0.f : mn;  // fully masked so far: everything stays 0
   const float alpha = fast_exp2(m - ms);
@@ -154,10 +153,11 @@ __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float 
   for (int tt = 0; tt < 4; tt++) {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-      // two probabilities rounded to bf16 at once; the row sum adds the rounded values
-      const uint32_t pk = pack_bf16x2(fast_exp2(st[tt][2 * h] - ms), fast_exp2(st[tt][2 * h + 1] - ms));
-      rs += bf16lo(pk);
-      rs += bf16hi(pk);
+      // two probabilities rounded to bf16 at once; the row sum adds the rounded values (one
+      // v_dot2c_f32_bf16 with a pair of ones adds both halves)
+      const uint32_t pk = pack_bf16x2(fast_exp2(__builtin_fmaf(st[tt][2 * h], c, -ms)),
+                                      fast_exp2(__builtin_fmaf(st[tt][2 * h + 1], c, -ms)));
+      rs = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), rs, false);
       pw[tt][h] = pk;
     }
   }
