@@ -352,3 +352,27 @@ def test_packed_forward_with_lse_keeps_the_output_bits():
         assert float((lse[o : o + ql].cpu() - want).abs().max()) < 2e-3
         o += ql
         ok += kl
+
+
+def test_decode_forms_agree_bitwise_with_many_workgroups():
+    """256 sequences x 4 kv heads = 1024 workgroups: the fused kernel then runs with 4 wavefronts per
+    workgroup (several rounds for the longer sequences); same bits as one wavefront per chunk."""
+    from vexact_amd import ops
+
+    g = torch.Generator().manual_seed(21)
+    kv_lens = torch.randint(1, 1500, (256,), generator=g).tolist()
+    kv_lens[:4] = [2049, 1, 256, 1025]
+    k = [(torch.randn(n, 4, 128, generator=g) * 0.3).to(torch.bfloat16) for n in kv_lens]
+    v = [(torch.randn(n, 4, 128, generator=g) * 0.3).to(torch.bfloat16) for n in kv_lens]
+    q = (torch.randn(len(kv_lens), 32, 128, generator=g) * 0.3).to(torch.bfloat16).cuda()
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, 16)
+    kc, vc = k_cache.cuda(), v_cache.cuda()
+    cu = torch.arange(len(kv_lens) + 1, dtype=torch.int32).cuda()
+    used = torch.tensor(kv_lens, dtype=torch.int32).cuda()
+    order = torch.tensor(sorted(range(len(kv_lens)), key=lambda i: (-kv_lens[i], i)), dtype=torch.int32).cuda()
+    split = ops.paged_attention(q, kc, vc, cu, used, table.cuda(), 128**-0.5, 1, decode_kernel="split")
+    for kw in (dict(decode_kernel="fused"), dict(decode_kernel="auto"), dict(decode_kernel="fused", seq_order=order)):
+        assert_bitwise(ops.paged_attention(q, kc, vc, cu, used, table.cuda(), 128**-0.5, 1, **kw), split, str(kw))
+    for i in (0, 1, 2, 3, 100):
+        ref = OA.eager_attention(q[i : i + 1].cpu(), k[i], v[i], 128**-0.5)[0]
+        torch.testing.assert_close(split[i].cpu(), ref, atol=3e-3, rtol=3e-3)

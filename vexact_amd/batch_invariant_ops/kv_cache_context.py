@@ -114,7 +114,10 @@ class KVCacheManager:
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:
-            self._lib.vx_kv_allocator_destroy(h)
+            try:
+                self._lib.vx_kv_allocator_destroy(h)
+            except Exception:  # interpreter shutdown: the library may already be gone
+                pass
 
     def _num_blocks_needed(self, num_tokens: int) -> int:
         return (num_tokens + self.cache_config.page_size - 1) // self.cache_config.page_size

@@ -945,7 +945,7 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
     // decode: chunks folded inside one workgroup per (sequence, kv head) when that fills the machine
     // (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3). Same bits.
     const int G = p.Hq / p.Hkv;
-    constexpr int NW1 = 8, NW2 = 4;  // wavefronts per block for one / two q-tiles (LDS: 84 / 96 KB at Dv = 128)
+    constexpr int NW1 = 8, NW1S = 4, NW2 = 4;  // wavefronts per block for one (many / very many workgroups) / two q-tiles
     if (G > 32) return VX_ERR_UNSUPPORTED;
     const bool fits = (G <= 16 ? fused_lds_bytes<DV, 1, NW1>() : fused_lds_bytes<DV, 2, NW2>()) <= 160 * 1024;
     if (mode == 4 && !fits) return VX_ERR_UNSUPPORTED;
@@ -968,7 +968,13 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
   } while (0)
       if (G <= 16) {
         if constexpr (DK <= 128 && DV <= 128) {
-          if (fast) VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_FAST, NW1);
+          // With >= 1024 workgroups, 4 wavefronts each: two workgroups then share a CU and one's set-up
+          // and fold overlap the other's streaming (measured 121.5 vs 124.8 us at 256 sequences x 4 kv
+          // heads; with 512 workgroups of long sequences 8 wavefronts are faster, 115 vs 125 us).
+          if ((int64_t)p.num_seqs * p.Hkv >= 1024) {
+            if (fast) VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_FAST, NW1S);
+            else VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_GENERIC, NW1S);
+          } else if (fast) VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_FAST, NW1);
           else VX_FUSED(attn_decode_fused_kernel_occ2, 1, SRC_GENERIC, NW1);
         } else {
           if (fast) VX_FUSED(attn_decode_fused_kernel, 1, SRC_FAST, NW1);
