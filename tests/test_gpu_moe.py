@@ -93,8 +93,9 @@ def test_routing_integers_exact(T, E, k, bm):
     sel = torch.randint(0, E, (T, k), generator=g)
     if T == 700:
         sel[:, :] = 3  # everything on one expert
-    for dt in (torch.int64, torch.int32):
-        r = ops.moe_route(sel.to(dt).cuda(), E, bm=bm)
+    # chunked: three launches over 1024-entry chunks from 8192 entries on; otherwise one workgroup
+    for dt, chunked in ((torch.int64, True), (torch.int32, True), (torch.int32, False)):
+        r = ops.moe_route(sel.to(dt).cuda(), E, bm=bm, chunked=chunked)
         ref = OM.routing_integers_ref(sel, E)
         assert np.array_equal(r.splits.cpu().numpy(), ref["splits"])
         assert np.array_equal(r.cu.cpu().numpy(), ref["cu"])

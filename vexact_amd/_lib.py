@@ -43,6 +43,8 @@ PROTOTYPES = {
     "vx_router_topk": (_I, [_P, _P, _P, _L, _I, _I, _L, _I, _I, _I, _I, _P]),
     "vx_moe_max_tiles": (_L, [_L, _I, _I]),
     "vx_moe_route": (_I, [_P, _I, _L, _I, _I, _I] + [_P] * 8 + [_L, _P]),
+    "vx_moe_route_workspace_bytes": (_L, [_L, _I]),
+    "vx_moe_route_ws": (_I, [_P, _I, _L, _I, _I, _I] + [_P] * 8 + [_L, _P, _L, _P]),
     "vx_moe_gemm": (
         _I,
         [_P, _L, _P, _P, _L, _L, _P, _L, _L, _L, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _P],

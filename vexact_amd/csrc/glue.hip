@@ -12,8 +12,10 @@
 
 namespace vx {
 
-// grid = (ceil(T*(Hq+2Hkv)/4)); one wavefront per (token, head). Lane l < D/4 owns elements
-// 4l .. 4l+3. qkv row layout: [q heads | k heads | v heads], each head D wide.
+// grid = (ceil(T*(Hq+2Hkv)/8)); half a wavefront per (token, head): 32 lanes, lane l < D/4 of the
+// half owns elements 4l .. 4l+3. qkv row layout: [q heads | k heads | v heads], each head D wide.
+// The sum of squares is a 5-step butterfly inside the half: the same additions, in the same order, as a
+// 64-lane butterfly whose upper 32 lanes hold zeros.
 template <int D, typename PosT>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     const bf16_t* __restrict__ qkv, int64_t ld, const bf16_t* __restrict__ qw,
@@ -22,11 +24,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
     bf16_t* __restrict__ k_out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int64_t T,
     int Hq, int Hkv, float eps, int64_t max_pos, int page_size, int64_t csb, int64_t csp, int64_t csh) {
   const int HT = Hq + 2 * Hkv;
-  const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t wid = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);  // (token, head) item of this half wavefront
   if (wid >= T * HT) return;
   const int64_t t = wid / HT;
   const int h = (int)(wid % HT);
-  const int lane = threadIdx.x & 63;
+  const int lane = threadIdx.x & 31;          // lane inside the half
+  const int half_base = threadIdx.x & 32;     // first lane of the half inside the wavefront
   const bool own = lane < D / 4;
   const bf16_t* src = qkv + t * ld + (int64_t)h * D;
   uint2 raw = make_uint2(0, 0);
@@ -56,7 +59,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
 #pragma unroll
     for (int c = 0; c < 4; c++) acc += x[c] * x[c];
   }
-  const float tot = wave_sum(acc);
+  float tot = acc;
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) tot += __shfl_xor(tot, o, 64);
   const float inv = 1.0f / sqrtf(tot / (float)D + eps);
   float y[4], cs[4], sn[4];
   if (own) {
@@ -78,7 +83,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   float o[4];
 #pragma unroll
   for (int c = 0; c < 4; c++) {
-    const float partner = __shfl(y[c], first ? lane + HL : lane - HL, 64);
+    const float partner = __shfl(y[c], half_base + (first ? lane + HL : lane - HL), 64);
     const float rot = first ? -partner : partner;
     const float a = bf16_to_f32(f32_to_bf16(y[c] * cs[c]));
     const float b = bf16_to_f32(f32_to_bf16(rot * sn[c]));
@@ -139,8 +144,8 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
     page_size = 1;
   }
   if (T == 0) return VX_OK;
-  const int64_t waves = T * (Hq + 2 * Hkv);
-  const int64_t blocks = (waves + 3) / 4;
+  const int64_t items = T * (Hq + 2 * Hkv);
+  const int64_t blocks = (items + 7) / 8;
   if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
 #define VX_QK(DD, PT)                                                                          \
   qk_norm_rope_store_kernel<DD, PT><<<(unsigned)blocks, 256, 0, stream>>>(                     \

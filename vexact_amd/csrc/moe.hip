@@ -170,28 +170,19 @@ __global__ __launch_bounds__(256) void router_topk_bf16_kernel(const bf16_t* __r
 constexpr int RB_THREADS = 1024;
 
 template <bool IDX64>
-__global__ __launch_bounds__(RB_THREADS) void moe_route_kernel(
-    const void* __restrict__ idx, int64_t n, int k, int E, int bm, int* __restrict__ splits,
-    int* __restrict__ cu, int* __restrict__ scatter_index, int* __restrict__ sorted_token,
-    int* __restrict__ sorted_flat, int* __restrict__ tile_group, int* __restrict__ tile_row0,
-    int* __restrict__ tile_rows, int max_tiles) {
-  extern __shared__ int sm[];
-  int* hist = sm;             // [E]
-  int* running = sm + E;      // [E]  next free position per expert
-  int* tstart = sm + 2 * E;   // [E]  first tile of expert
-  int* wavecnt = sm + 3 * E;  // [16][E]
+__device__ __forceinline__ int route_expert_of(const void* idx, int64_t f, int E) {
+  int e;
+  if constexpr (IDX64) e = (int)((const int64_t*)idx)[f];
+  else e = ((const int*)idx)[f];
+  return min(max(e, 0), E - 1);  // keeps later address arithmetic in range
+}
+
+// From the per-expert counts in hist (LDS): splits, cu, running[e] = cu[e], first tile of each expert,
+// and the tile table. Called by a whole 1024-thread block; ends with the results visible to the block.
+__device__ __forceinline__ void route_scan_and_tiles(const int* hist, int* running, int* tstart, int E, int bm,
+                                                     int* splits, int* cu, int* tile_group, int* tile_row0,
+                                                     int* tile_rows, int max_tiles) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  auto expert_of = [&](int64_t f) {
-    int e;
-    if constexpr (IDX64) e = (int)((const int64_t*)idx)[f];
-    else e = ((const int*)idx)[f];
-    return min(max(e, 0), E - 1);  // keeps later address arithmetic in range
-  };
-  for (int e = tid; e < E; e += RB_THREADS) hist[e] = 0;
-  for (int t = tid; t < max_tiles; t += RB_THREADS) { tile_group[t] = -1; tile_row0[t] = 0; tile_rows[t] = 0; }
-  __syncthreads();
-  for (int64_t f = tid; f < n; f += RB_THREADS) atomicAdd(&hist[expert_of(f)], 1);
-  __syncthreads();
   // exclusive scans by wave 0: lane owns experts [lane*per, lane*per+per)
   if (wave == 0) {
     const int per = (E + 63) / 64;
@@ -221,7 +212,6 @@ __global__ __launch_bounds__(RB_THREADS) void moe_route_kernel(
     if (lane == 63) cu[E] = ci;
   }
   __syncthreads();
-  // tile table
   for (int e = tid; e < E; e += RB_THREADS) {
     const int cnt = hist[e], r0 = running[e];
     int t = tstart[e];
@@ -233,43 +223,132 @@ __global__ __launch_bounds__(RB_THREADS) void moe_route_kernel(
       }
     }
   }
-  // stable ranks, 1024 entries at a time
+}
+
+// Stable ranks of the (at most 1024) entries [base, base + 1024) given running[e] = position of the
+// next entry of expert e; advances running. wavecnt is [16][E] of LDS. Called by a whole block.
+template <bool IDX64>
+__device__ __forceinline__ void route_rank_chunk(const void* idx, int64_t base, int64_t n, int k, int E, int ebits,
+                                                 int* running, int* wavecnt, int* scatter_index, int* sorted_token,
+                                                 int* sorted_flat) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 16 * E; i += RB_THREADS) wavecnt[i] = 0;
+  __syncthreads();
+  const int64_t f = base + tid;
+  const bool live = f < n;
+  const int e = live ? route_expert_of<IDX64>(idx, f, E) : 0;
+  // lanes of this wave with the same expert
+  uint64_t same = __ballot(live);
+  for (int b = 0; b < ebits; b++) {
+    const uint64_t bal = __ballot((e >> b) & 1);
+    same &= ((e >> b) & 1) ? bal : ~bal;
+  }
+  if (!live) same = 0;
+  const int rank_in_wave = __popcll(same & ((1ull << lane) - 1ull));
+  if (live && rank_in_wave == 0) wavecnt[wave * E + e] = __popcll(same);
+  __syncthreads();
+  for (int ee = tid; ee < E; ee += RB_THREADS) {
+    int r = running[ee];
+    for (int w = 0; w < 16; w++) {
+      const int c = wavecnt[w * E + ee];
+      wavecnt[w * E + ee] = r;
+      r += c;
+    }
+    running[ee] = r;
+  }
+  __syncthreads();
+  if (live) {
+    const int pos = wavecnt[wave * E + e] + rank_in_wave;
+    scatter_index[f] = pos;
+    sorted_flat[pos] = (int)f;
+    sorted_token[pos] = (int)(f / k);
+  }
+  __syncthreads();
+}
+
+template <bool IDX64>
+__global__ __launch_bounds__(RB_THREADS) void moe_route_kernel(
+    const void* __restrict__ idx, int64_t n, int k, int E, int bm, int* __restrict__ splits,
+    int* __restrict__ cu, int* __restrict__ scatter_index, int* __restrict__ sorted_token,
+    int* __restrict__ sorted_flat, int* __restrict__ tile_group, int* __restrict__ tile_row0,
+    int* __restrict__ tile_rows, int max_tiles) {
+  extern __shared__ int sm[];
+  int* hist = sm;             // [E]
+  int* running = sm + E;      // [E]  next free position per expert
+  int* tstart = sm + 2 * E;   // [E]  first tile of expert
+  int* wavecnt = sm + 3 * E;  // [16][E]
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += RB_THREADS) hist[e] = 0;
+  for (int t = tid; t < max_tiles; t += RB_THREADS) { tile_group[t] = -1; tile_row0[t] = 0; tile_rows[t] = 0; }
+  __syncthreads();
+  for (int64_t f = tid; f < n; f += RB_THREADS) atomicAdd(&hist[route_expert_of<IDX64>(idx, f, E)], 1);
+  __syncthreads();
+  route_scan_and_tiles(hist, running, tstart, E, bm, splits, cu, tile_group, tile_row0, tile_rows, max_tiles);
   int ebits = 0;
   while ((1 << ebits) < E) ebits++;
-  for (int64_t base = 0; base < n; base += RB_THREADS) {
-    for (int i = tid; i < 16 * E; i += RB_THREADS) wavecnt[i] = 0;
-    __syncthreads();
-    const int64_t f = base + tid;
-    const bool live = f < n;
-    const int e = live ? expert_of(f) : 0;
-    // lanes of this wave with the same expert
-    uint64_t same = __ballot(live);
-    for (int b = 0; b < ebits; b++) {
-      const uint64_t bal = __ballot((e >> b) & 1);
-      same &= ((e >> b) & 1) ? bal : ~bal;
-    }
-    if (!live) same = 0;
-    const int rank_in_wave = __popcll(same & ((1ull << lane) - 1ull));
-    if (live && rank_in_wave == 0) wavecnt[wave * E + e] = __popcll(same);
-    __syncthreads();
-    for (int ee = tid; ee < E; ee += RB_THREADS) {
-      int r = running[ee];
-      for (int w = 0; w < 16; w++) {
-        const int c = wavecnt[w * E + ee];
-        wavecnt[w * E + ee] = r;
-        r += c;
-      }
-      running[ee] = r;
-    }
-    __syncthreads();
-    if (live) {
-      const int pos = wavecnt[wave * E + e] + rank_in_wave;
-      scatter_index[f] = pos;
-      sorted_flat[pos] = (int)f;
-      sorted_token[pos] = (int)(f / k);
-    }
-    __syncthreads();
+  for (int64_t base = 0; base < n; base += RB_THREADS)
+    route_rank_chunk<IDX64>(idx, base, n, k, E, ebits, running, wavecnt, scatter_index, sorted_token, sorted_flat);
+}
+
+// ---- the same routing integers for many entries (prefill): three launches over chunks of 1024 entries.
+// counts [chunks][E] (global): first the chunk's expert counts, then (after the scan) the position of the
+// chunk's first entry of each expert.
+template <bool IDX64>
+__global__ __launch_bounds__(RB_THREADS) void moe_route_count_kernel(const void* __restrict__ idx, int64_t n, int E,
+                                                                     int* __restrict__ counts) {
+  extern __shared__ int sm[];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += RB_THREADS) sm[e] = 0;
+  __syncthreads();
+  const int64_t f = (int64_t)blockIdx.x * RB_THREADS + tid;
+  if (f < n) atomicAdd(&sm[route_expert_of<IDX64>(idx, f, E)], 1);
+  __syncthreads();
+  for (int e = tid; e < E; e += RB_THREADS) counts[(int64_t)blockIdx.x * E + e] = sm[e];
+}
+
+__global__ __launch_bounds__(RB_THREADS) void moe_route_scan_kernel(int* __restrict__ counts, int chunks, int E, int bm,
+                                                                    int* __restrict__ splits, int* __restrict__ cu,
+                                                                    int* __restrict__ tile_group, int* __restrict__ tile_row0,
+                                                                    int* __restrict__ tile_rows, int max_tiles) {
+  extern __shared__ int sm[];
+  int* hist = sm;
+  int* running = sm + E;
+  int* tstart = sm + 2 * E;
+  const int tid = threadIdx.x;
+  for (int t = tid; t < max_tiles; t += RB_THREADS) { tile_group[t] = -1; tile_row0[t] = 0; tile_rows[t] = 0; }
+  for (int e = tid; e < E; e += RB_THREADS) {
+    int tot = 0;
+    for (int c = 0; c < chunks; c++) tot += counts[(int64_t)c * E + e];
+    hist[e] = tot;
   }
+  __syncthreads();
+  route_scan_and_tiles(hist, running, tstart, E, bm, splits, cu, tile_group, tile_row0, tile_rows, max_tiles);
+  __syncthreads();
+  for (int e = tid; e < E; e += RB_THREADS) {  // counts -> first position of the chunk's entries of expert e
+    int base = running[e];
+    for (int c = 0; c < chunks; c++) {
+      const int t = counts[(int64_t)c * E + e];
+      counts[(int64_t)c * E + e] = base;
+      base += t;
+    }
+  }
+}
+
+template <bool IDX64>
+__global__ __launch_bounds__(RB_THREADS) void moe_route_rank_kernel(const void* __restrict__ idx, int64_t n, int k, int E,
+                                                                    const int* __restrict__ counts,
+                                                                    int* __restrict__ scatter_index,
+                                                                    int* __restrict__ sorted_token,
+                                                                    int* __restrict__ sorted_flat) {
+  extern __shared__ int sm[];
+  int* running = sm;       // [E]
+  int* wavecnt = sm + E;   // [16][E]
+  for (int e = threadIdx.x; e < E; e += RB_THREADS) running[e] = counts[(int64_t)blockIdx.x * E + e];
+  int ebits = 0;
+  while ((1 << ebits) < E) ebits++;
+  __syncthreads();
+  route_rank_chunk<IDX64>(idx, (int64_t)blockIdx.x * RB_THREADS, n, k, E, ebits, running, wavecnt, scatter_index,
+                          sorted_token, sorted_flat);
 }
 
 template <bool IDX64>
@@ -443,9 +522,18 @@ int64_t vx_moe_max_tiles(int64_t n_entries, int E, int bm) {
   return a + n_entries / bm;
 }
 
-int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,
-                 int* cu, int* scatter_index, int* sorted_token, int* sorted_flat, int* tile_group,
-                 int* tile_row0, int* tile_rows, int64_t max_tiles, hipStream_t stream) {
+// Entries from which the chunked three-launch routing is used when a workspace is given
+constexpr int64_t RB_CHUNKED_FROM = 8192;
+
+int64_t vx_moe_route_workspace_bytes(int64_t n_entries, int E) {
+  if (n_entries < RB_CHUNKED_FROM || E <= 0) return 0;
+  return (n_entries + RB_THREADS - 1) / RB_THREADS * (int64_t)E * 4;
+}
+
+int vx_moe_route_ws(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,
+                    int* cu, int* scatter_index, int* sorted_token, int* sorted_flat, int* tile_group,
+                    int* tile_row0, int* tile_rows, int64_t max_tiles, void* workspace, int64_t workspace_bytes,
+                    hipStream_t stream) {
   if (!expert_idx || !splits || !cu || !scatter_index || !sorted_token || !sorted_flat ||
       !tile_group || !tile_row0 || !tile_rows)
     return VX_ERR_ARG;
@@ -454,6 +542,23 @@ int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, i
   const int64_t n = T * k;
   if (n > 0x7fffffffLL) return VX_ERR_ARG;
   if (max_tiles < vx_moe_max_tiles(n, E, bm) || max_tiles > 0x7fffffffLL) return VX_ERR_WORKSPACE;
+  const int64_t need = vx_moe_route_workspace_bytes(n, E);
+  if (need > 0 && workspace && workspace_bytes >= need && ((uintptr_t)workspace & 3) == 0) {
+    const int64_t chunks = (n + RB_THREADS - 1) / RB_THREADS;
+    int* counts = (int*)workspace;
+    if (idx_i64) moe_route_count_kernel<true><<<(unsigned)chunks, RB_THREADS, (size_t)E * 4, stream>>>(expert_idx, n, E, counts);
+    else moe_route_count_kernel<false><<<(unsigned)chunks, RB_THREADS, (size_t)E * 4, stream>>>(expert_idx, n, E, counts);
+    moe_route_scan_kernel<<<1, RB_THREADS, (size_t)3 * E * 4, stream>>>(counts, (int)chunks, E, bm, splits, cu, tile_group,
+                                                                       tile_row0, tile_rows, (int)max_tiles);
+    const size_t lds = (size_t)(1 + 16) * E * 4;
+    if (idx_i64)
+      moe_route_rank_kernel<true><<<(unsigned)chunks, RB_THREADS, lds, stream>>>(expert_idx, n, k, E, counts, scatter_index,
+                                                                                sorted_token, sorted_flat);
+    else
+      moe_route_rank_kernel<false><<<(unsigned)chunks, RB_THREADS, lds, stream>>>(expert_idx, n, k, E, counts, scatter_index,
+                                                                                 sorted_token, sorted_flat);
+    return launch_status();
+  }
   const size_t lds = (size_t)(3 + 16) * E * sizeof(int);
   if (idx_i64)
     moe_route_kernel<true><<<1, RB_THREADS, lds, stream>>>(expert_idx, n, k, E, bm, splits, cu,
@@ -466,6 +571,13 @@ int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, i
                                                             tile_group, tile_row0, tile_rows,
                                                             (int)max_tiles);
   return launch_status();
+}
+
+int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,
+                 int* cu, int* scatter_index, int* sorted_token, int* sorted_flat, int* tile_group,
+                 int* tile_row0, int* tile_rows, int64_t max_tiles, hipStream_t stream) {
+  return vx_moe_route_ws(expert_idx, idx_i64, T, k, E, bm, splits, cu, scatter_index, sorted_token, sorted_flat,
+                         tile_group, tile_row0, tile_rows, max_tiles, nullptr, 0, stream);
 }
 
 // Grouped GEMM over a tile table: C[rows of tile] = X[row_src[rows]] * W[group]^T.

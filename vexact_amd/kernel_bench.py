@@ -195,6 +195,8 @@ def main() -> None:
             dn = rnd(E, H, I)
             hw = torch.empty(T * k, I, dtype=torch.bfloat16, device=dev)
             eo = torch.empty(T * k, H, dtype=torch.bfloat16, device=dev)
+            report(f"prefill moe route T={T}", timeit(lambda li: ops.moe_route(idx, E, bm=ops.moe_tile_rows(T)), n_layers=2), T * k * 16)
+            report(f"prefill moe route T={T}, one workgroup", timeit(lambda li: ops.moe_route(idx, E, bm=ops.moe_tile_rows(T), chunked=False), n_layers=2), T * k * 16)
             report(f"prefill moe gate/up T={T}",
                    timeit(lambda li: ops.moe_gemm(x, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=w,
                                                   row_scale_idx=r.sorted_flat, out=hw), n_layers=2),
@@ -202,6 +204,20 @@ def main() -> None:
             report(f"prefill moe down T={T}", timeit(lambda li: ops.moe_gemm(hw, dn, r, out=eo), n_layers=2),
                    flops=2 * T * k * H * I)
             del x, logits, gu, dn, hw, eo
+        # q/k norm + rotary + cache store over a prefill chunk
+        Hq_, Hkv_, D_, page_ = 32, 4, 128, 16
+        for T in (8192,):
+            qkv = rnd(T, (Hq_ + 2 * Hkv_) * D_, std=1.0)
+            qn, kn = rnd(D_, std=1.0), rnd(D_, std=1.0)
+            cos_t, sin_t = rnd(16384, D_, std=1.0), rnd(16384, D_, std=1.0)
+            pos = torch.arange(T, dtype=torch.int64, device=dev)
+            slots = torch.randperm(T, device=dev).to(torch.int32)
+            kcache = rnd(T // page_, Hkv_, page_, D_).permute(0, 2, 1, 3)
+            vcache = rnd(T // page_, Hkv_, page_, D_).permute(0, 2, 1, 3)
+            qo = torch.empty(T, Hq_, D_, dtype=torch.bfloat16, device=dev)
+            report(f"prefill q/k norm + rope + store T={T}",
+                   timeit(lambda li: ops.qk_norm_rope_store(qkv, qn, kn, cos_t, sin_t, pos, slots, qo, kcache, vcache, Hq_, Hkv_, D_, 1e-6), n_layers=2),
+                   T * (Hq_ + 2 * Hkv_) * D_ * 2 * 2 + T * D_ * 4)
         # causal attention over whole prompts: 8 sequences of 1024 tokens, paged cache
         Hq, Hkv, D, page, S, Lp = 32, 4, 128, 16, 8, 1024
         npg = S * Lp // page

@@ -563,7 +563,10 @@ class MoeRouting:
                  "tile_rows", "max_tiles", "bm", "T", "k", "E")
 
 
-def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int] = None, buffers=None) -> MoeRouting:
+def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int] = None, buffers=None,
+              chunked: bool = True) -> MoeRouting:
+    """Routing integers of ``selected_experts [T, k]``. From 8192 entries on the work is spread over many
+    workgroups (needs a small workspace); ``chunked=False`` keeps the one-workgroup kernel (same integers)."""
     _need_gpu("selected_experts", selected_experts)
     assert selected_experts.dtype in (torch.int32, torch.int64)
     idx = selected_experts.contiguous()
@@ -588,11 +591,14 @@ def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int
     r.tile_group = ints[o : o + max_tiles]; o += max_tiles
     r.tile_row0 = ints[o : o + max_tiles]; o += max_tiles
     r.tile_rows = ints[o : o + max_tiles]; o += max_tiles
+    need = lib.vx_moe_route_workspace_bytes(n, num_experts) if chunked else 0
+    ws = _workspace(need, dev) if need > 0 else None
     _lib.check(
-        lib.vx_moe_route(
+        lib.vx_moe_route_ws(
             idx.data_ptr(), int(idx.dtype == torch.int64), T, k, num_experts, bm, r.splits.data_ptr(),
             r.cu.data_ptr(), r.scatter_index.data_ptr(), r.sorted_token.data_ptr(), r.sorted_flat.data_ptr(),
-            r.tile_group.data_ptr(), r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), max_tiles, _stream(),
+            r.tile_group.data_ptr(), r.tile_row0.data_ptr(), r.tile_rows.data_ptr(), max_tiles, _ptr(ws),
+            ws.numel() * ws.element_size() if ws is not None else 0, _stream(),
         ),
         "vx_moe_route",
     )
