@@ -66,7 +66,8 @@ def test_wide_kernel_agrees_bitwise(M, N, K, bias):
         assert_bitwise(ops.gemm_nt(ag[1000:1003], wg, bias=bg), full[1000:1003], "3 rows alone vs inside a chunk")
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 640, 2048), (100, 200, 64), (77, 333, 192), (130, 70, 320), (512, 128, 768)])
+@pytest.mark.parametrize("M,N,K", [(256, 640, 2048), (100, 200, 64), (77, 333, 192), (130, 70, 320), (512, 128, 768),
+                                   (3000, 128, 512)])  # the last: many rows, few columns -> ring by dispatch
 def test_ring_kernel_agrees_bitwise(M, N, K):
     a = _gen((M, K), 16)
     w = _gen((N, K), 17, scale=0.05)

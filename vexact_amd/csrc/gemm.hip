@@ -98,6 +98,9 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
     // many rows: 256x256 tiles once they fill at least half the chip, else 128x128 tiles
     const int64_t wide_tiles = ((M + WD_BM - 1) / WD_BM) * ((N + WD_BN - 1) / WD_BN);
     if (wide_tiles >= 128 && gemm_wide_launch(p, stream)) return launch_status();
+    // many rows but few columns (router logits over a prefill chunk): the 64x64 ring kernel yields four
+    // times the workgroups of the 128x128 tiles
+    if (N <= 256 && ((M + 127) / 128) * ((N + 127) / 128) < 256 && gemm_ring_launch(p, 0, stream)) return launch_status();
     const int64_t mtl = (M + TL_BM - 1) / TL_BM;
     if (mtl > 65535) return VX_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)((N + TL_BN - 1) / TL_BN), (unsigned)mtl);

@@ -149,7 +149,7 @@ def main() -> None:
                    2 * (N * K + B * K + B * N))
             del ws_
     if "prefill" in what:
-        for name, M, N, K in (("qkv", 8192, 5120, 2048), ("o", 8192, 2048, 4096), ("lm_head", 4096, 151936, 2048),
+        for name, M, N, K in (("router", 8192, 128, 2048), ("qkv", 8192, 5120, 2048), ("o", 8192, 2048, 4096), ("lm_head", 4096, 151936, 2048),
                               ("square", 8192, 8192, 8192)):
             w_ = rnd(N, K)
             xx = rnd(M, K, std=1.0)
