@@ -28,6 +28,8 @@ fused_moe_ref          k=1,w=1 => plain SwiGLU MLP; all tokens on one expert => 
                        fp64 brute force on tiny shapes; HF-eager form within bf16 tolerance
 prepare_gen_ctx_ref    hand-worked example; vectorised numpy twin
 BlockAllocatorRef      scan restatement of the reference allocator; hand-worked sequence
+attention_backward_ref autograd through the fp32 eager attention; one visible key => dV = dO, dQ = dK = 0
+fused_moe_backward_ref autograd through an fp32 restatement of the expert MLPs
 sampler.philox4x32     Random123 known-answer vectors
 sampler.exp32 / log    numpy exp / log within 4e-7 / 2e-6
 sampler.kept_mask_spec the reference's sort + cumsum rule (apply_top_k_top_p_ref) on tie-free rows

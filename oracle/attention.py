@@ -84,3 +84,36 @@ def paged_attention_ref(q, k_cache, v_cache, cu_seqlens_q, seqused_k, page_table
         v = gather_paged(v_cache, page_table[s], n)
         outs.append(eager_attention(q[q0:q1], k, v, softmax_scale))
     return torch.cat(outs, dim=0) if outs else q.new_zeros((0, q.shape[1], v_cache.shape[-1]))
+
+
+def attention_backward_ref(q_seq, k_seq, v_seq, do_seq, softmax_scale):
+    """Backward of causal attention for one sequence with the reference's roundings
+    (_varlen_attn_bwd_dq_kernel / _varlen_attn_bwd_dkv_kernel, triton_invariant_attention.py:193-430):
+    ``P = exp(scale s - lse)``, ``dP = dO V^T``, ``delta = rowsum(O * dO)`` with ``O`` the bf16 forward
+    output, ``dS = P (dP - delta) scale``; P and dS are rounded to the input dtype before
+    ``dV = P^T dO``, ``dQ = dS K``, ``dK = dS^T Q``; fp32 accumulation, results in the input dtype.
+    ``q_seq/do_seq [Q,Hq,D]``, ``k_seq/v_seq [K,Hkv,D]`` -> (dq, dk, dv)."""
+    dt = q_seq.dtype
+    ql, kl = q_seq.shape[0], k_seq.shape[0]
+    g = q_seq.shape[1] // k_seq.shape[1]
+    q, do = q_seq.float().transpose(0, 1), do_seq.float().transpose(0, 1)            # [Hq, Q, D]
+    k = k_seq.float().transpose(0, 1).repeat_interleave(g, dim=0)                     # [Hq, K, D]
+    v = v_seq.float().transpose(0, 1).repeat_interleave(g, dim=0)
+    s = torch.matmul(q, k.transpose(-1, -2)) * softmax_scale
+    mask = torch.arange(kl).unsqueeze(0) <= (torch.arange(ql) + (kl - ql)).unsqueeze(1)
+    s = s.masked_fill(~mask.unsqueeze(0), float("-inf"))
+    lse = torch.logsumexp(s, dim=-1, keepdim=True)
+    p = torch.where(mask.unsqueeze(0), torch.exp(s - lse), torch.zeros(()))
+    p = torch.nan_to_num(p, nan=0.0)                                                  # rows without a visible key
+    out = eager_attention(q_seq, k_seq, v_seq, softmax_scale).float().transpose(0, 1)  # bf16 forward output
+    delta = (out * do).sum(-1, keepdim=True)
+    dp = torch.matmul(do, v.transpose(-1, -2))
+    ds = p * (dp - delta) * softmax_scale
+    p16, ds16 = p.to(dt).float(), ds.to(dt).float()
+    dq = torch.matmul(ds16, k)
+    dk = torch.matmul(ds16.transpose(-1, -2), q)
+    dv = torch.matmul(p16.transpose(-1, -2), do)
+    hkv = k_seq.shape[1]
+    dk = dk.reshape(hkv, g, kl, -1).sum(1)                                            # heads of a group, ascending
+    dv = dv.reshape(hkv, g, kl, -1).sum(1)
+    return dq.transpose(0, 1).to(dt), dk.transpose(0, 1).to(dt), dv.transpose(0, 1).to(dt)

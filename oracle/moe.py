@@ -113,3 +113,42 @@ def hf_eager_moe_ref(hidden, routing_weights, selected_experts, gate_w, up_w, do
         o = _bf(o.float() * _bf(routing_weights)[tok, slot].float().unsqueeze(1))
         out.index_add_(0, tok, o)
     return out
+
+
+def fused_moe_backward_ref(hidden, routing_weights, selected_experts, gate_w, up_w, down_w, grad_out):
+    """Backward of the fused expert MLPs with the reference's formulas and bf16 intermediates
+    (FusedMoeExpertFunction.backward, vexact/batch_invariant_ops/fused_moe.py:126-265): per
+    (token, slot) row of expert ``e``: ``g = x Wg^T``, ``u = x Wu^T``, ``a = silu(g)``, ``act = a u``,
+    ``hw = act w``; ``d_hw = dY Wd``, ``dWd += dY^T hw``, ``d_act = d_hw w``, ``dw = sum(act d_hw)``,
+    ``d_a = d_act u``, ``d_u = a d_act``, ``d_g = silu'(g) d_a``, ``dx += d_g Wg + d_u Wu``,
+    ``dWg += d_g^T x``, ``dWu += d_u^T x``. Returns (d_routing_weights, d_hidden, dWg, dWu, dWd)."""
+    x, w, dy = _bf(hidden), _bf(routing_weights), _bf(grad_out)
+    T, k = selected_experts.shape
+    sel = selected_experts.to(torch.int64)
+    d_w = torch.zeros(T, k, dtype=torch.float32)
+    d_x_slots = torch.zeros(T, k, x.shape[1], dtype=torch.float32)
+    d_g_w, d_u_w, d_d_w = (torch.zeros_like(t, dtype=torch.float32) for t in (gate_w, up_w, down_w))
+    for e in torch.unique(sel).tolist():
+        tok, slot = torch.nonzero(sel == e, as_tuple=True)
+        xe, dye = x[tok].float(), dy[tok].float()
+        g = _bf(xe @ gate_w[e].float().t())
+        u = _bf(xe @ up_w[e].float().t())
+        a = _bf(F.silu(g.float()))
+        act = _bf(a.float() * u.float())
+        ws = w[tok, slot].float().unsqueeze(1)
+        hw = _bf(act.float() * ws)
+        d_hw = _bf(dye @ down_w[e].float())
+        d_d_w[e] = dye.t() @ hw.float()
+        d_act = _bf(d_hw.float() * ws)
+        d_w[tok, slot] = _bf((act.float() * d_hw.float()).sum(-1)).float()
+        d_a = _bf(d_act.float() * u.float())
+        d_u = _bf(a.float() * d_act.float())
+        sg = torch.sigmoid(g.float())
+        d_g = _bf(d_a.float() * sg * (1 + g.float() * (1 - sg)))
+        d_x_slots[tok, slot] = _bf(d_g.float() @ gate_w[e].float()).float() + _bf(d_u.float() @ up_w[e].float()).float()
+        d_g_w[e] = d_g.float().t() @ xe
+        d_u_w[e] = d_u.float().t() @ xe
+    d_x = torch.zeros(T, x.shape[1], dtype=torch.float32)
+    for i in range(k):
+        d_x = d_x + _bf(d_x_slots[:, i]).float()
+    return _bf(d_w), _bf(d_x), _bf(d_g_w), _bf(d_u_w), _bf(d_d_w)

@@ -327,6 +327,13 @@ def test_packed_backward_matches_autograd_and_is_batch_invariant(qh, kh, d, q_le
             assert float(err.max()) <= tol, f"{name} of sequence {s}: max err {float(err.max()):.4f} > {tol:.4f}"
             assert float(err.mean()) <= 2e-3 * float(want.abs().max()), f"{name} of sequence {s}: mean err"
         assert_bf16_close(out[o : o + ql], ref.detach().to(torch.bfloat16), max_ulp=2, atol_frac=3e-3, what=f"out of sequence {s}")
+        # and against the restatement with the same bf16 roundings of P and dS (tighter)
+        odq, odk, odv = OA.attention_backward_ref(q_seqs[s], k_seqs[s], v_seqs[s], do_seqs[s], scale)
+        for name, got, want in (("dq", dq[o : o + ql], odq), ("dk", dk[ok : ok + kl], odk), ("dv", dv[ok : ok + kl], odv)):
+            err = (got.float() - want.float()).abs()
+            top = float(want.float().abs().max())
+            assert float(err.max()) <= 1e-2 * top and float(err.mean()) <= 1e-3 * top, (
+                f"{name} of sequence {s} vs the CPU restatement: max {float(err.max()):.4g}, mean {float(err.mean()):.4g}, scale {top:.4g}")
         # the sequence alone gives the same gradient bits
         _, dq1, dk1, dv1 = _packed_fwd_bwd(q_seqs[s : s + 1], k_seqs[s : s + 1], v_seqs[s : s + 1], do_seqs[s : s + 1])
         assert_bitwise(dq1, dq[o : o + ql], f"dq of sequence {s} alone vs in the batch")

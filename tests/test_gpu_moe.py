@@ -263,3 +263,10 @@ def test_fused_moe_backward_matches_autograd():
         scale = float(want.grad.abs().max())
         assert float(err.max()) <= 3e-2 * scale, f"grad of {name}: max err {float(err.max()):.4g} vs scale {scale:.4g}"
         assert float(err.mean()) <= 4e-3 * scale, f"grad of {name}: mean err"
+    # and against the CPU restatement with the same bf16 intermediates
+    for name, got, want in zip(("routing weights", "hidden states", "gate", "up", "down"), leaves,
+                               OM.fused_moe_backward_ref(x, w, sel, gw, uw, dw, dy)):
+        err = (got.grad.float().cpu() - want.float()).abs()
+        scale = float(want.float().abs().max())
+        assert float(err.max()) <= 2e-2 * scale and float(err.mean()) <= 2e-3 * scale, (
+            f"grad of {name} vs the CPU restatement: max {float(err.max()):.4g} mean {float(err.mean()):.4g} scale {scale:.4g}")

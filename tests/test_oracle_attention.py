@@ -85,3 +85,30 @@ def test_paged_attention_ref_equals_eager_on_gathered_keys():
     got = OA.paged_attention_ref(torch.cat(qs), kc, vc, cu, used, table, 0.25)
     want = torch.cat([OA.eager_attention(a, b, c, 0.25) for a, b, c in zip(qs, ks, vs)])
     assert torch.equal(got, want)
+
+
+def test_attention_backward_restatement_matches_autograd():
+    # the reference's backward formulas (with bf16 P and dS) against autograd through the fp32 eager
+    # attention; a single visible key makes P = 1 exactly: dV = dO, dQ = dK = 0
+    g = torch.Generator().manual_seed(3)
+    for (ql, kl, hq, hkv, d) in ((9, 9, 4, 2, 32), (5, 23, 6, 2, 64), (1, 40, 2, 2, 32)):
+        q = torch.randn(ql, hq, d, generator=g).to(torch.bfloat16)
+        k = torch.randn(kl, hkv, d, generator=g).to(torch.bfloat16)
+        v = torch.randn(kl, hkv, d, generator=g).to(torch.bfloat16)
+        do = torch.randn(ql, hq, d, generator=g).to(torch.bfloat16)
+        dq, dk, dv = OA.attention_backward_ref(q, k, v, do, d ** -0.5)
+        qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+        grp = hq // hkv
+        s = torch.einsum("qhd,khd->hqk", qf, kf.repeat_interleave(grp, dim=1)) * d ** -0.5
+        mask = torch.arange(kl)[None, :] <= (torch.arange(ql) + (kl - ql))[:, None]
+        o = torch.einsum("hqk,khd->qhd", torch.softmax(s.masked_fill(~mask[None], float("-inf")), -1), vf.repeat_interleave(grp, dim=1))
+        o.backward(do.float())
+        for name, got, want in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+            err = (got.float() - want).abs().max()
+            assert float(err) <= 2e-2 * float(want.abs().max()), (name, ql, kl, float(err))
+    q = torch.randn(1, 2, 32, generator=g).to(torch.bfloat16)
+    k = torch.randn(1, 2, 32, generator=g).to(torch.bfloat16)
+    v = torch.randn(1, 2, 32, generator=g).to(torch.bfloat16)
+    do = torch.randn(1, 2, 32, generator=g).to(torch.bfloat16)
+    dq, dk, dv = OA.attention_backward_ref(q, k, v, do, 0.3)
+    assert torch.equal(dv, do) and float(dq.abs().max()) < 1e-2 and float(dk.abs().max()) < 1e-2

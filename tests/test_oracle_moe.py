@@ -89,3 +89,27 @@ def test_fused_moe_ref_special_cases():
     assert (got3 - want).abs().max() <= 3e-2 * want.abs().max()
     hf = OM.hf_eager_moe_ref(x, w3, sel3, gate, up, down).double()
     assert (hf - want).abs().max() <= 3e-2 * want.abs().max()
+
+
+def test_moe_backward_restatement_matches_autograd():
+    # the reference's backward formulas (bf16 intermediates) against autograd through an fp32 restatement
+    T, H, I, E, k = 24, 32, 16, 4, 2
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    gw, uw = ((torch.randn(E, I, H, generator=g) * 0.2).to(torch.bfloat16) for _ in range(2))
+    dw = (torch.randn(E, H, I, generator=g) * 0.2).to(torch.bfloat16)
+    w, sel = torch.topk(torch.softmax(torch.randn(T, E, generator=g), -1), k)
+    w = (w / w.sum(-1, keepdim=True)).to(torch.bfloat16)
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    got = OM.fused_moe_backward_ref(x, w, sel, gw, uw, dw, dy)
+    leaves = [t.float().requires_grad_() for t in (w, x, gw, uw, dw)]
+    rw, rx, rg, ru, rd = leaves
+    ref = torch.zeros(T, H)
+    for i in range(k):
+        e = sel[:, i]
+        h = torch.nn.functional.silu(torch.einsum("th,tih->ti", rx, rg[e])) * torch.einsum("th,tih->ti", rx, ru[e])
+        ref = ref + rw[:, i : i + 1] * torch.einsum("ti,thi->th", h, rd[e])
+    ref.backward(dy.float())
+    for name, a, b in zip(("routing weights", "hidden", "gate", "up", "down"), got, leaves):
+        err = (a.float() - b.grad).abs()
+        assert float(err.max()) <= 3e-2 * float(b.grad.abs().max()), (name, float(err.max()), float(b.grad.abs().max()))
