@@ -270,3 +270,42 @@ def test_fused_moe_backward_matches_autograd():
         scale = float(want.float().abs().max())
         assert float(err.max()) <= 2e-2 * scale and float(err.mean()) <= 2e-3 * scale, (
             f"grad of {name} vs the CPU restatement: max {float(err.max()):.4g} mean {float(err.mean()):.4g} scale {scale:.4g}")
+
+
+def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
+    # Qwen3MoeSparseMoeBlock after apply_qwen3_moe_patches: router + fused experts on the GPU against the CPU
+    # restatements; a token alone gives the bits it gives in the batch; one expert called directly == dense MLP
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeConfig, Qwen3MoeSparseMoeBlock
+
+    from oracle.row_ops import matmul_ref
+    from vexact_amd.batch_invariant_ops import set_batch_invariant_mode
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches
+
+    apply_qwen3_moe_patches()
+    cfg = Qwen3MoeConfig(hidden_size=256, moe_intermediate_size=128, num_experts=16, num_experts_per_tok=4, norm_topk_prob=True,
+                         num_hidden_layers=1, vocab_size=100, intermediate_size=64, num_attention_heads=2, num_key_value_heads=1)
+    torch.manual_seed(3)
+    blk = Qwen3MoeSparseMoeBlock(cfg).to(torch.bfloat16)
+    with torch.no_grad():
+        blk.gate.weight.normal_(0, 0.5)
+        blk.experts.gate_up_proj.normal_(0, 0.06)
+        blk.experts.down_proj.normal_(0, 0.06)
+    x = torch.randn(1, 40, 256).to(torch.bfloat16)
+    gpu = blk.to("cuda")
+    with torch.no_grad(), set_batch_invariant_mode(True):
+        y = gpu(x.cuda())
+        y1 = gpu(x[:, 7:8].cuda())
+        one = gpu.experts(x[0, :5].cuda(), expert_idx=3)
+    assert_bitwise(y1, y[:, 7:8], "token 7 alone vs in the batch")
+    cpu = blk.to("cpu")
+    logits = matmul_ref(x[0], cpu.gate.weight.detach().t())
+    w, idx = OM.router_ref(logits, 4)
+    got_w, got_idx = ops.router_topk(logits.cuda(), 4)
+    assert torch.equal(got_idx.cpu(), idx)
+    gu, dn = cpu.experts.gate_up_proj.detach(), cpu.experts.down_proj.detach()
+    ref = OM.fused_moe_ref(x[0], w, idx, gu[:, :128], gu[:, 128:], dn)
+    assert_bf16_close(y[0], ref, max_ulp=2, atol_frac=2e-3, what="patched block vs oracle")
+    g = matmul_ref(x[0, :5], gu[3, :128].t())
+    u = matmul_ref(x[0, :5], gu[3, 128:].t())
+    dense = matmul_ref((torch.nn.functional.silu(g.float()).to(torch.bfloat16).float() * u.float()).to(torch.bfloat16), dn[3].t())
+    assert_bf16_close(one, dense, max_ulp=2, atol_frac=2e-3, what="single expert as a dense MLP")

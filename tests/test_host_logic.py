@@ -225,3 +225,26 @@ def test_sampler_argument_errors_need_no_gpu():
         s.batch_sample_token(logits, [cfg(seed=1), cfg(seed=2)])
     with pytest.raises(AssertionError, match="top_p must be set"):
         s.batch_sample_token(logits, [cfg(top_p=None)] * 2)
+
+
+def test_qwen3_moe_patch_points():
+    # apply_qwen3_moe_patches (vexact/models/qwen3_moe/modeling_qwen3_moe.py:291-302): idempotent, fused experts
+    # container with the reference's parameter names and layout, a plain linear router
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeConfig, Qwen3MoeSparseMoeBlock
+
+    from vexact_amd.models.qwen3_moe import Qwen3MoeExperts, apply_qwen3_moe_patches, moe_block_forward
+
+    apply_qwen3_moe_patches()
+    apply_qwen3_moe_patches()
+    cfg = Qwen3MoeConfig(hidden_size=64, moe_intermediate_size=32, num_experts=8, num_experts_per_tok=2, norm_topk_prob=True,
+                         num_hidden_layers=1, vocab_size=100, intermediate_size=64, num_attention_heads=2, num_key_value_heads=1)
+    blk = Qwen3MoeSparseMoeBlock(cfg)
+    assert isinstance(blk.experts, Qwen3MoeExperts) and isinstance(blk.gate, torch.nn.Linear) and blk.gate.bias is None
+    assert dict(blk.named_parameters()).keys() == {"gate.weight", "experts.gate_up_proj", "experts.down_proj"}
+    assert blk.experts.gate_up_proj.shape == (8, 64, 64) and blk.experts.down_proj.shape == (8, 64, 32)
+    assert (blk.top_k, blk.num_experts, blk.norm_topk_prob) == (2, 8, True)
+    blk.experts = torch.nn.ModuleList()
+    with pytest.raises(AssertionError, match="experts are not fused"):
+        moe_block_forward(blk, torch.zeros(1, 2, 64))
+    with pytest.raises(ValueError, match="silu"):
+        Qwen3MoeExperts(types.SimpleNamespace(num_experts=2, hidden_size=8, moe_intermediate_size=8, hidden_act="gelu"))
