@@ -717,6 +717,7 @@ constexpr int PFL_LDS = PFL_NS * PFL_STAGE + PFL_SLOTS * 16 * 256;         // st
 template <int KIND>
 __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnParams p, int hpw) {
   constexpr int D = 128, QT = PFL_QT, KS = D / 32;
+  constexpr int KPW = ATT_BLOCK / PFL_WAVES;  // keys of a block that one wavefront brings in
   extern __shared__ __attribute__((aligned(1024))) uint8_t pf_lds[];
 
   const int seq = blockIdx.z;
@@ -795,14 +796,14 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   auto issue_block = [&](int kb, int stage) {
     const typename KVSource<KIND>::Tiles tl = src.tiles(kb);
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const int row = 8 * wave + 4 * j + (lane >> 4);  // key row inside the block
+    for (int j = 0; j < KPW / 4; j++) {
+      const int row = KPW * wave + 4 * j + (lane >> 4);  // key row inside the block
       const int tt = row >> 4, within = row & 15;
       const bool ok = kb + row < kv_len;
       const int piece = (lane & 15) ^ (row & 15);
       const bf16_t* kp = src.krow(tl, kb, tt, ok ? within : 0) + 8 * piece;
       const bf16_t* vp = src.vrow(tl, kb, tt, ok ? within : 0) + 8 * piece;
-      const uint32_t dst = lds0 + stage * PFL_STAGE + (8 * wave + 4 * j) * 256;
+      const uint32_t dst = lds0 + stage * PFL_STAGE + (KPW * wave + 4 * j) * 256;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                    :: "s"(dst), "v"(kp) : "memory", "m0");
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
@@ -858,12 +859,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   };
 
   const int nblk = blk_maxpos / ATT_BLOCK + 1;
-#pragma unroll
-  for (int i = 0; i < PFL_NS; i++)
-    if (i < nblk) issue_block(i * ATT_BLOCK, i);
-  int stage = 0;
-  for (int b = 0; b < nblk; b++) {
-    const int kb = b * ATT_BLOCK;
+  auto chunk_reset = [&](int kb) {
     if ((kb & (ATT_CHUNK - 1)) == 0) {
 #pragma unroll
       for (int t = 0; t < QT; t++) {
@@ -872,16 +868,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
         for (int i = 0; i < 8; i++) acc[t][i] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
     }
-    // block b has landed; the 4 loads each of up to PFL_NS - 1 later blocks may still be in flight
-    const int ahead = min(PFL_NS - 1, nblk - 1 - b);
-    if (ahead >= 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if (ahead == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    block_compute(kb, stage);
-    __syncthreads();  // everyone is done with this stage
-    if (b + PFL_NS < nblk) issue_block(kb + PFL_NS * ATT_BLOCK, stage);
-    stage = stage + 1 == PFL_NS ? 0 : stage + 1;
+  };
+  auto chunk_fold = [&](int kb, int b) {
     if (((kb + ATT_BLOCK) & (ATT_CHUNK - 1)) == 0 || b + 1 == nblk) {
 #pragma unroll
       for (int t = 0; t < QT; t++) {
@@ -895,6 +883,28 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
         M[t] = Mn;
       }
     }
+  };
+  // one barrier per block: passing it says that block b has landed for everyone and that everyone
+  // is done with block b - 1, whose stage then takes block b + PFL_NS - 1
+#pragma unroll
+  for (int i = 0; i < PFL_NS - 1; i++)
+    if (i < nblk) issue_block(i * ATT_BLOCK, i);
+  int stage = 0;
+  for (int b = 0; b < nblk; b++) {
+    const int kb = b * ATT_BLOCK;
+    chunk_reset(kb);
+    // KPW / 2 loads per block and wavefront; the next block's may still be in flight
+    if (b + 1 < nblk) {
+      static_assert(KPW == 8, "the wait below counts 4 loads per block and wavefront");
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    if (b + PFL_NS - 1 < nblk) issue_block(kb + (PFL_NS - 1) * ATT_BLOCK, stage == 0 ? PFL_NS - 1 : stage - 1);
+    block_compute(kb, stage);
+    stage = stage + 1 == PFL_NS ? 0 : stage + 1;
+    chunk_fold(kb, b);
   }
 
   // lane (r16 = query row, g) holds dims 16 f + 4 g + r of fragment f
