@@ -272,6 +272,53 @@ def test_fused_moe_backward_matches_autograd():
             f"grad of {name} vs the CPU restatement: max {float(err.max()):.4g} mean {float(err.mean()):.4g} scale {scale:.4g}")
 
 
+@pytest.mark.parametrize("T,k,E,N,K,bm", [(300, 2, 8, 128, 64, 32), (257, 4, 16, 200, 264, 128), (4096, 2, 8, 768, 256, 128),
+                                          (5, 1, 8, 8, 8, 64)])
+def test_grouped_backward_products_match_per_expert_matmuls(T, k, E, N, K, bm):
+    # data gradient C = A W_e (two accumulated products, gathered rows) and weight gradient dW_e = dY_e^T X_e
+    # against fp32 matmuls per expert; ragged expert sizes, experts without rows, ragged N and K
+    gen = torch.Generator().manual_seed(T + N)
+    sel = torch.randint(0, E - 1, (T, k), generator=gen)          # the last expert never gets a row
+    if T > 100:
+        sel[sel == 2] = 3                                        # nor does expert 2
+    r = ops.moe_route(sel.cuda(), E, bm=bm)
+    n = T * k
+    cu, tok = r.cu.cpu().tolist(), r.sorted_token.cpu().long()
+    a = torch.randn(T, K, generator=gen).to(torch.bfloat16)       # gathered through sorted_token
+    a2 = torch.randn(n, 40, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(E, K, N, generator=gen) * 0.1).to(torch.bfloat16)
+    w2 = (torch.randn(E, 40, N, generator=gen) * 0.1).to(torch.bfloat16)
+    print(f"[case] nn T={T} k={k} E={E} N={N} K={K} bm={bm}", flush=True)
+    one = ops.moe_gemm_nn(a.cuda(), w.cuda(), r, a_src=r.sorted_token)
+    two = ops.moe_gemm_nn(a.cuda(), w.cuda(), r, a_src=r.sorted_token, a2=a2.cuda(), w2=w2.cuda())
+    plain = ops.moe_gemm_nn(a[tok].cuda(), w.cuda(), r)
+    assert_bitwise(plain, one, "row gather inside the kernel vs gathered beforehand")
+    ref1, ref2 = torch.zeros(n, N), torch.zeros(n, N)
+    for e in range(E):
+        lo, hi = cu[e], cu[e + 1]
+        ref1[lo:hi] = a[tok[lo:hi]].float() @ w[e].float()
+        ref2[lo:hi] = ref1[lo:hi] + a2[lo:hi].float() @ w2[e].float()
+    assert_bf16_close(one, ref1.to(torch.bfloat16), max_ulp=1, atol_frac=1e-3, what="grouped A W")
+    assert_bf16_close(two, ref2.to(torch.bfloat16), max_ulp=1, atol_frac=1e-3, what="grouped A W + A2 W2")
+
+    print(f"[case] tn T={T} k={k} E={E} N={N} K={K}", flush=True)
+    dy = torch.randn(n, N, generator=gen).to(torch.bfloat16)
+    dyt = torch.randn(T, N, generator=gen).to(torch.bfloat16)
+    x = torch.randn(T, K, generator=gen).to(torch.bfloat16)
+    got = ops.moe_gemm_tn(dy.cuda(), x.cuda(), r.cu, E, x_src=r.sorted_token)
+    got2 = ops.moe_gemm_tn(dyt.cuda(), a2.cuda(), r.cu, E, dy_src=r.sorted_token)
+    ref, refb = torch.zeros(E, N, K), torch.zeros(E, N, 40)
+    for e in range(E):
+        lo, hi = cu[e], cu[e + 1]
+        ref[e] = dy[lo:hi].float().t() @ x[tok[lo:hi]].float()
+        refb[e] = dyt[tok[lo:hi]].float().t() @ a2[lo:hi].float()
+    assert_bf16_close(got, ref.to(torch.bfloat16), max_ulp=1, atol_frac=1e-3, what="grouped dY^T X")
+    assert_bf16_close(got2, refb.to(torch.bfloat16), max_ulp=1, atol_frac=1e-3, what="grouped dY^T X, gathered dY")
+    assert float(got[E - 1].abs().max()) == 0.0, "an expert without rows gets zeros"
+    # deterministic: a second launch gives the same bits
+    assert_bitwise(ops.moe_gemm_tn(dy.cuda(), x.cuda(), r.cu, E, x_src=r.sorted_token), got, "second launch")
+
+
 def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
     # Qwen3MoeSparseMoeBlock after apply_qwen3_moe_patches: router + fused experts on the GPU against the CPU
     # restatements; a token alone gives the bits it gives in the batch; one expert called directly == dense MLP

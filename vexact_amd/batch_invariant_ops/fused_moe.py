@@ -57,7 +57,6 @@ class FusedMoeExpertFunction(torch.autograd.Function):
         T, k = x.shape[0], selected_experts.reshape(x.shape[0], -1).shape[1]
         dy = grad_output.reshape(-1, H).to(torch.bfloat16)
         r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=False))
-        tok = r.sorted_token.long()                      # token of each expert-sorted row
         flat = r.sorted_flat.long()                      # (token, slot) flat index of each sorted row
         # recomputed with the forward's kernels, so these are the values the forward used
         g = ops.moe_gemm(x, gate_w, r, row_src=r.sorted_token)
@@ -66,33 +65,18 @@ class FusedMoeExpertFunction(torch.autograd.Function):
         act = a * u
         w_sorted = routing_weights.reshape(-1)[flat].unsqueeze(1)
         hw = act * w_sorted
-        xs, dys = x[tok], dy[tok]
-        cu = r.cu.cpu().tolist()                         # host copy: the products below are per-expert library calls
-        d_hw = torch.empty_like(hw)
-        d_g_w = torch.zeros_like(gate_w) if ctx.needs_input_grad[4] else None
-        d_u_w = torch.zeros_like(up_w) if ctx.needs_input_grad[5] else None
-        d_d_w = torch.zeros_like(down_w) if ctx.needs_input_grad[6] else None
-        for e in range(E):
-            lo, hi = cu[e], cu[e + 1]
-            if hi > lo:
-                d_hw[lo:hi] = dys[lo:hi] @ down_w[e]                               # dgrad of the down projection
-                if d_d_w is not None:
-                    d_d_w[e] = dys[lo:hi].t() @ hw[lo:hi]
+        # grouped products on the HIP kernels; the row gathers x[tok], dy[tok] happen inside them
+        d_hw = ops.moe_gemm_nn(dy, down_w, r, a_src=r.sorted_token)                # dgrad of the down projection
+        d_d_w = ops.moe_gemm_tn(dy, hw, r.cu, E, dy_src=r.sorted_token) if ctx.needs_input_grad[6] else None
         d_act = d_hw * w_sorted
         d_w_sorted = torch.sum(act * d_hw, dim=-1)
         grad_rw = torch.empty_like(d_w_sorted)
         grad_rw[flat] = d_w_sorted
         d_a, d_u = d_act * u, a * d_act
         d_g = torch.ops.aten.silu_backward(d_a, g)
-        d_xs = torch.empty_like(xs)
-        for e in range(E):
-            lo, hi = cu[e], cu[e + 1]
-            if hi > lo:
-                d_xs[lo:hi] = d_g[lo:hi] @ gate_w[e] + d_u[lo:hi] @ up_w[e]
-                if d_g_w is not None:
-                    d_g_w[e] = d_g[lo:hi].t() @ xs[lo:hi]
-                if d_u_w is not None:
-                    d_u_w[e] = d_u[lo:hi].t() @ xs[lo:hi]
+        d_xs = ops.moe_gemm_nn(d_g, gate_w, r, a2=d_u, w2=up_w)
+        d_g_w = ops.moe_gemm_tn(d_g, x, r.cu, E, x_src=r.sorted_token) if ctx.needs_input_grad[4] else None
+        d_u_w = ops.moe_gemm_tn(d_u, x, r.cu, E, x_src=r.sorted_token) if ctx.needs_input_grad[5] else None
         d_x = ops.moe_gather(d_xs, r.scatter_index)
         return (None, grad_rw.reshape(routing_weights.shape).to(routing_weights.dtype), None,
                 d_x.reshape(hidden_states.shape), d_g_w, d_u_w, d_d_w)

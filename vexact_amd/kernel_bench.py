@@ -167,6 +167,26 @@ def main() -> None:
         report("packed attention fwd + lse 8 x 1024", timeit(lambda li: ops.packed_attention(q, kk, vv, cu, cu, D**-0.5, True, Lp, return_lse=True), n_layers=2), flops=fl)
         o, lse = ops.packed_attention(q, kk, vv, cu, cu, D**-0.5, True, Lp, return_lse=True)
         report("packed attention bwd 8 x 1024", timeit(lambda li: ops.packed_attention_backward(q, kk, vv, o, do, lse, cu, cu, D**-0.5, Lp, Lp), n_layers=2), flops=fl * 5 // 2)
+        # fused-MoE backward products at the model's expert shapes, 8192 tokens (128-row expert tiles)
+        T = 8192
+        x = rnd(T, H, std=1.0)
+        logits = torch.randn(T, E, generator=g, device=dev)
+        w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
+        r = ops.moe_route(idx, E, bm=128)
+        gu, dn = rnd(E, 2 * I, H), rnd(E, H, I)
+        dyt, dg, du = rnd(T, H, std=1.0), rnd(T * k, I, std=1.0), rnd(T * k, I, std=1.0)
+        o_i = torch.empty(T * k, I, dtype=torch.bfloat16, device=dev)
+        o_h = torch.empty(T * k, H, dtype=torch.bfloat16, device=dev)
+        o_dn, o_g = torch.empty_like(dn), torch.empty(E, I, H, dtype=torch.bfloat16, device=dev)
+        report("moe bwd dgrad down (dY Wd) T=8192", timeit(lambda li: ops.moe_gemm_nn(dyt, dn, r, a_src=r.sorted_token, out=o_i), n_layers=2),
+               flops=2 * T * k * H * I)
+        report("moe bwd dgrad gate+up T=8192", timeit(lambda li: ops.moe_gemm_nn(dg, gu[:, :I], r, a2=du, w2=gu[:, I:], out=o_h), n_layers=2),
+               flops=2 * T * k * 2 * I * H)
+        report("moe bwd wgrad down T=8192", timeit(lambda li: ops.moe_gemm_tn(dyt, dg, r.cu, E, dy_src=r.sorted_token, out=o_dn), n_layers=2),
+               flops=2 * T * k * H * I)
+        report("moe bwd wgrad gate T=8192", timeit(lambda li: ops.moe_gemm_tn(dg, x, r.cu, E, x_src=r.sorted_token, out=o_g), n_layers=2),
+               flops=2 * T * k * H * I)
+        del gu, dn, o_dn, o_g
     if "dense" in what:
         # dense SwiGLU MLP of a Qwen3-8B-shaped layer (hidden 4096, intermediate 12288): fused gate/up, then down
         Hd, Id = 4096, 12288

@@ -631,6 +631,61 @@ def moe_gemm(
     return c
 
 
+def moe_gemm_nn(
+    a: torch.Tensor, w: torch.Tensor, routing: MoeRouting, *, a_src: Optional[torch.Tensor] = None,
+    a2: Optional[torch.Tensor] = None, w2: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Grouped data gradient: ``C[rows of e] = A[a_src[rows]] @ w[e] (+ A2[rows] @ w2[e])`` with ``w [E, K, N]``
+    (N contiguous). ``routing`` must have been built with at most 128 rows per tile."""
+    E, K, N = w.shape
+    n_rows = routing.T * routing.k
+    assert a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.stride(1) == 1 and w.stride(2) == 1
+    assert a.shape[1] == K and (a_src is not None or a.shape[0] == n_rows)
+    assert (a2 is None) == (w2 is None)
+    K2 = 0
+    if a2 is not None:
+        K2 = w2.shape[1]
+        assert a2.dtype == torch.bfloat16 and w2.dtype == torch.bfloat16 and a2.stride(1) == 1 and w2.stride(2) == 1
+        assert a2.shape == (n_rows, K2) and w2.shape[0] == E and w2.shape[2] == N
+    if a_src is not None:
+        assert a_src.dtype == torch.int32 and a_src.is_contiguous() and a_src.numel() == n_rows
+    c = out if out is not None else torch.empty((n_rows, N), dtype=torch.bfloat16, device=a.device)
+    _lib.check(
+        _lib.load().vx_moe_gemm_nn(
+            a.data_ptr(), a.stride(0), _ptr(a_src), w.data_ptr(), w.stride(1), w.stride(0), K,
+            _ptr(a2), a2.stride(0) if a2 is not None else 0, _ptr(w2), w2.stride(1) if w2 is not None else 0,
+            w2.stride(0) if w2 is not None else 0, K2, c.data_ptr(), c.stride(0), N,
+            routing.tile_group.data_ptr(), routing.tile_row0.data_ptr(), routing.tile_rows.data_ptr(),
+            routing.max_tiles, routing.bm, _stream(),
+        ),
+        "vx_moe_gemm_nn",
+    )
+    return c
+
+
+def moe_gemm_tn(
+    dy: torch.Tensor, x: torch.Tensor, cu: torch.Tensor, num_experts: int, *, dy_src: Optional[torch.Tensor] = None,
+    x_src: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Grouped weight gradient: ``dW[e] = dY[dy_src[r]]^T @ X[x_src[r]]`` summed over the sorted rows
+    ``cu[e] <= r < cu[e + 1]``; returns ``[E, N, K]`` (zeros for an expert without rows)."""
+    N, K = dy.shape[1], x.shape[1]
+    assert dy.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and dy.stride(1) == 1 and x.stride(1) == 1
+    assert cu.dtype == torch.int32 and cu.is_contiguous() and cu.numel() == num_experts + 1
+    for src in (dy_src, x_src):
+        assert src is None or (src.dtype == torch.int32 and src.is_contiguous())
+    dw = out if out is not None else torch.empty((num_experts, N, K), dtype=torch.bfloat16, device=dy.device)
+    assert dw.shape == (num_experts, N, K) and dw.stride(2) == 1
+    _lib.check(
+        _lib.load().vx_moe_gemm_tn(
+            dy.data_ptr(), dy.stride(0), _ptr(dy_src), x.data_ptr(), x.stride(0), _ptr(x_src), dw.data_ptr(),
+            dw.stride(1), dw.stride(0), N, K, cu.data_ptr(), num_experts, _stream(),
+        ),
+        "vx_moe_gemm_tn",
+    )
+    return dw
+
+
 def expert_histogram(idx: torch.Tensor, num_bins: int) -> torch.Tensor:
     assert idx.is_cuda
     assert idx.dtype == torch.int32 or idx.dtype == torch.int64
