@@ -273,7 +273,7 @@ def test_fused_moe_backward_matches_autograd():
 
 
 @pytest.mark.parametrize("T,k,E,N,K,bm", [(300, 2, 8, 128, 64, 32), (257, 4, 16, 200, 264, 128), (4096, 2, 8, 768, 256, 128),
-                                          (5, 1, 8, 8, 8, 64)])
+                                          (5, 1, 8, 8, 8, 64), (1000, 2, 8, 328, 520, 128)])
 def test_grouped_backward_products_match_per_expert_matmuls(T, k, E, N, K, bm):
     # data gradient C = A W_e (two accumulated products, gathered rows) and weight gradient dW_e = dY_e^T X_e
     # against fp32 matmuls per expert; ragged expert sizes, experts without rows, ragged N and K

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnBwdParams p) {
 // Head size 128: the moving side goes through LDS once per workgroup. 8 wavefronts hold 8 stationary
 // tiles (128 queries of one head for dQ); every 64-row block of the two moving arrays (K and V) is
 // brought in by direct-to-LDS loads into one of two 32 KB stages while the previous block is being
-// used. Rows are 256 bytes with 16-byte piece c of row r stored at piece c ^ (r & 15): the 16-byte
+// used. Rows are 256 bytes with 16-byte piece c of row r stored at piece c ^ bwl_swz(r): the 16-byte
 // fragment reads (A operands of the score products) and the transposing 8-byte reads
 // (ds_read_b64_tr_b16, A operands of the products that contract over the moving rows) are both
 // free of bank conflicts, and the transposing reads deliver the rows in the k-slot order in which
@@ -310,6 +310,10 @@ constexpr int BWL_STAGE = 2 * BWL_ARR;     // two arrays per stage
 constexpr int BWL_LDS = 2 * BWL_STAGE;     // two stages
 typedef short bw_v4s_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void* bw_lds_ptr_t;
+// A 16-byte fragment read takes one piece from each of 16 consecutive rows: the swizzle term must differ over
+// them. A transposing read takes two adjacent pieces from each of 8 consecutive rows at a time: the term
+// without its lowest bit must differ over those.
+__device__ __forceinline__ int bwl_swz(int row) { return ((row & 7) << 1) | ((row >> 3) & 1); }
 
 // wavefront `wave` of NW brings rows [64 / NW * wave, +64 / NW) of a 64-row array into LDS: 4 rows per instruction
 template <int NW = BWL_WAVES>
@@ -320,7 +324,7 @@ __device__ __forceinline__ void bwl_issue_rows(const bf16_t* base, int64_t row_s
 #pragma unroll
   for (int j = 0; j < RPW / 4; j++) {
     const int row = RPW * wave + 4 * j + (lane >> 4);
-    const int piece = (lane & 15) ^ (row & 15);
+    const int piece = (lane & 15) ^ bwl_swz(row);
     const bf16_t* src = base + (int64_t)min(first_row + row, last_row) * row_stride + 8 * piece;
     const uint32_t dst = lds_arr + (RPW * wave + 4 * j) * 256;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
@@ -330,7 +334,7 @@ __device__ __forceinline__ void bwl_issue_rows(const bf16_t* base, int64_t row_s
 __device__ __forceinline__ uint4 bwl_frag(const uint8_t* arr, int tt, int s) {
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int row = 16 * tt + r16;
-  return *(const uint4*)(arr + row * 256 + (((4 * s + g) ^ (row & 15)) * 16));
+  return *(const uint4*)(arr + row * 256 + (((4 * s + g) ^ bwl_swz(row)) * 16));
 }
 // acc[f] (rows = dims 16 f + .., cols = stationary) += (array rows, transposed) x pf
 __device__ __forceinline__ void bwl_tr_product(const uint8_t* arr, const uint4 (&pf)[2], f32x4 (&acc)[8]) {
@@ -342,9 +346,9 @@ __device__ __forceinline__ void bwl_tr_product(const uint8_t* arr, const uint4 (
       const int byte = 32 * f + 8 * (r16 & 3);
       const int row_lo = 32 * ch + 4 * g + (r16 >> 2), row_hi = row_lo + 16;
       const bw_v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) bw_v4s_t*)(arr + row_lo * 256 + (((byte >> 4) ^ (row_lo & 15)) * 16) + (byte & 15)));
+          (__attribute__((address_space(3))) bw_v4s_t*)(arr + row_lo * 256 + (((byte >> 4) ^ bwl_swz(row_lo)) * 16) + (byte & 15)));
       const bw_v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) bw_v4s_t*)(arr + row_hi * 256 + (((byte >> 4) ^ (row_hi & 15)) * 16) + (byte & 15)));
+          (__attribute__((address_space(3))) bw_v4s_t*)(arr + row_hi * 256 + (((byte >> 4) ^ bwl_swz(row_hi)) * 16) + (byte & 15)));
       const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
       acc[f] = mfma16(make_uint4(lo2.x, lo2.y, hi2.x, hi2.y), pf[ch], acc[f]);
     }

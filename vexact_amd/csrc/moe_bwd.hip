@@ -19,10 +19,12 @@ typedef short v4s_t __attribute__((ext_vector_type(4)));
 constexpr int NN_ROWS = 64;  // per k-step of the data-gradient kernel (its LDS use is one operand only)
 constexpr int TN_ROWS = 32;  // of the weight-gradient kernel: measured faster than 64 (more workgroups per CU, shorter ragged tails)
 
-// 16-byte piece c of row r lives at piece c ^ (r & 15): the four rows of one transposing read then fall
-// into different banks
+// A transposing read takes two adjacent 16-byte pieces from each of the rows 8 g .. 8 g + 3 (or + 4 .. + 7) of
+// two lane groups g at a time: 16-byte piece c of row r lives at piece c ^ gb_swz(r), whose pair index
+// differs over those eight rows, so they fall into different banks
+__device__ __forceinline__ int gb_swz(int row) { return ((row & 3) | ((row >> 1) & 4)) << 1; }
 __device__ __forceinline__ int gb_off(int row, int byte) {
-  return row * 256 + ((((byte >> 4) ^ (row & 15)) << 4) | (byte & 15));
+  return row * 256 + ((((byte >> 4) ^ gb_swz(row)) << 4) | (byte & 15));
 }
 
 // columns col0 .. col0 + 15, rows row0 .. row0 + 31 of the tile as an MFMA operand: lane (r16, g) gets column
@@ -174,7 +176,7 @@ struct MoeTnParams {
   const int* x_src;
   bf16_t* dw;
   int64_t lddw, dw_gstride;
-  int N, K;
+  int N, K, E;
   const int* cu;
 };
 
@@ -259,6 +261,122 @@ __global__ __launch_bounds__(256) void moe_gemm_tn_kernel(MoeTnParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// The same product on 256 x 256 output tiles: 8 wavefronts as 2 (n halves of 128) x 4 (k quarters of 64),
+// LDS tiles of 32 rows x 256 columns (512-byte rows). Half the operand traffic per output element of the
+// 128 x 128 kernel, which is what bounds that one; two steps of global loads are in flight in registers
+// because only one workgroup fits a CU.
+// ---------------------------------------------------------------------------------------
+constexpr int TW_ROWS = 32, TW_TILE = TW_ROWS * 512;
+
+__device__ __forceinline__ int tw_off(int row, int byte) {
+  return row * 512 + ((((byte >> 4) ^ gb_swz(row)) << 4) | (byte & 15));
+}
+__device__ __forceinline__ uint4 tw_frag(const uint8_t* tile, int col0, int r16, int g) {
+  const int byte = 2 * col0 + 8 * (r16 & 3);
+  const int row_lo = 8 * g + (r16 >> 2), row_hi = row_lo + 4;
+  const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t*)(tile + tw_off(row_lo, byte)));
+  const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t*)(tile + tw_off(row_hi, byte)));
+  const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+  return make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+}
+
+__global__ __launch_bounds__(512) void moe_gemm_tn_wide_kernel(MoeTnParams p) {
+  __shared__ __attribute__((aligned(1024))) uint8_t yt[2][TW_TILE];
+  __shared__ __attribute__((aligned(1024))) uint8_t xt[2][TW_TILE];
+  // Consecutive workgroup ids go to different XCDs (id % 8), each with its own L2: XCD x takes the experts
+  // e = x (mod 8), all output tiles of one expert in a row, so an expert's rows are fetched into one L2.
+  const int tiles_k = (p.K + 255) >> 8, tiles = tiles_k * ((p.N + 255) >> 8);
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int e = (slot / tiles) * 8 + xcd;
+  if (e >= p.E) return;  // uniform
+  const int tile = slot % tiles;
+  const int lo = p.cu[e], hi = p.cu[e + 1];
+  const int k0 = (tile % tiles_k) * 256, n0 = (tile / tiles_k) * 256;
+  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+  const int wave = threadIdx.x >> 6, wn = wave >> 2, wk = wave & 3;
+
+  f32x4 acc[4][8];  // [k tile][n tile]
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int f = 0; f < 8; f++) acc[i][f] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // piece q = tid + 512 j of a tile: row q / 32, 16-byte piece q % 32. The (gathered) row numbers of a
+  // step are fetched one step before its data, so that the two dependent loads do not add their latencies.
+  auto load_rows = [&](int r0, int (&ry)[2], int (&rx)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int r = r0 + ((threadIdx.x + 512 * j) >> 5);
+      const bool ok = r < hi;
+      ry[j] = ok ? (p.dy_src ? p.dy_src[r] : r) : -1;
+      rx[j] = ok ? (p.x_src ? p.x_src[r] : r) : -1;
+    }
+  };
+  auto load_tiles = [&](const int (&ry)[2], const int (&rx)[2], uint4 (&yr)[2], uint4 (&xr)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int pc = (threadIdx.x + 512 * j) & 31;
+      const bool oky = ry[j] >= 0 && n0 + 8 * pc < p.N, okx = rx[j] >= 0 && k0 + 8 * pc < p.K;
+      yr[j] = ldg16(oky ? (const void*)(p.dy + (int64_t)ry[j] * p.lddy + n0 + 8 * pc) : (const void*)p.dy, oky);
+      xr[j] = ldg16(okx ? (const void*)(p.x + (int64_t)rx[j] * p.ldx + k0 + 8 * pc) : (const void*)p.x, okx);
+    }
+  };
+
+  const int steps = (hi - lo + TW_ROWS - 1) / TW_ROWS;
+  uint4 yr[2][2], xr[2][2];  // register set (s & 1) holds step s
+  int ry[2], rx[2];          // row numbers of the next step to be loaded
+  load_rows(lo, ry, rx);
+  if (steps > 0) load_tiles(ry, rx, yr[0], xr[0]);
+  load_rows(lo + TW_ROWS, ry, rx);
+  if (steps > 1) load_tiles(ry, rx, yr[1], xr[1]);
+  load_rows(lo + 2 * TW_ROWS, ry, rx);
+  auto step = [&](int s, int buf, uint4 (&yrs)[2], uint4 (&xrs)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int q = threadIdx.x + 512 * j;
+      const int off = tw_off(q >> 5, 16 * (q & 31));
+      *(uint4*)(yt[buf] + off) = yrs[j];
+      *(uint4*)(xt[buf] + off) = xrs[j];
+    }
+    __syncthreads();  // also: everyone is done reading the other buffer's previous contents
+    if (s + 2 < steps) {
+      load_tiles(ry, rx, yrs, xrs);
+      load_rows(lo + (s + 3) * TW_ROWS, ry, rx);
+    }
+    uint4 yf[8], xf[4];
+#pragma unroll
+    for (int f = 0; f < 8; f++) yf[f] = tw_frag(yt[buf], 128 * wn + 16 * f, r16, g);
+#pragma unroll
+    for (int i = 0; i < 4; i++) xf[i] = tw_frag(xt[buf], 64 * wk + 16 * i, r16, g);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int f = 0; f < 8; f++) acc[i][f] = mfma16(xf[i], yf[f], acc[i][f]);
+  };
+#pragma unroll 1
+  for (int s = 0; s < steps; s += 2) {
+    step(s, 0, yr[0], xr[0]);
+    if (s + 1 < steps) step(s + 1, 1, yr[1], xr[1]);
+  }
+
+  bf16_t* dwe = p.dw + (int64_t)e * p.dw_gstride;
+#pragma unroll
+  for (int f = 0; f < 8; f++) {
+    const int n = n0 + 128 * wn + 16 * f + r16;
+    if (n >= p.N) continue;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int k = k0 + 64 * wk + 16 * i + 4 * g;
+      if (k >= p.K) continue;
+      uint2 pk;
+      pk.x = pack_bf16x2(acc[i][f][0], acc[i][f][1]);
+      pk.y = pack_bf16x2(acc[i][f][2], acc[i][f][3]);
+      *(uint2*)(dwe + (int64_t)n * p.lddw + k) = pk;
+    }
+  }
+}
+
 static inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace vx
@@ -307,8 +425,14 @@ int vx_moe_gemm_tn(const void* dy, int64_t lddy, const int* dy_src, const void* 
   p.dy = (const bf16_t*)dy; p.lddy = lddy; p.dy_src = dy_src;
   p.x = (const bf16_t*)x; p.ldx = ldx; p.x_src = x_src;
   p.dw = (bf16_t*)dw; p.lddw = lddw; p.dw_gstride = dw_gstride;
-  p.N = (int)N; p.K = (int)K; p.cu = cu;
-  moe_gemm_tn_kernel<TN_ROWS><<<dim3((unsigned)((K + 127) / 128), (unsigned)gy, (unsigned)num_experts), 256, 0, stream>>>(p);
+  p.N = (int)N; p.K = (int)K; p.E = (int)num_experts; p.cu = cu;
+  if (N >= 256 && K >= 256) {
+    const int64_t wg = 8 * ((num_experts + 7) / 8) * ((K + 255) / 256) * ((N + 255) / 256);
+    if (wg > 0x7fffffffLL) return VX_ERR_UNSUPPORTED;
+    moe_gemm_tn_wide_kernel<<<dim3((unsigned)wg), 512, 0, stream>>>(p);
+  } else {
+    moe_gemm_tn_kernel<TN_ROWS><<<dim3((unsigned)((K + 127) / 128), (unsigned)gy, (unsigned)num_experts), 256, 0, stream>>>(p);
+  }
   return launch_status();
 }
 

@@ -791,7 +791,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   const KVSource<KIND> src = make_source<KIND>(p, seq, kvh, k0, kv_len);
   // ---- loads: wavefront v brings in keys [8 v, 8 v + 8) of a block, K and V, 4 keys (1 KB) per
   // instruction; lane l writes slot l % 16 of its key row and therefore fetches logical piece
-  // (l % 16) ^ (row & 15)
+  // (l % 16) ^ (row & 15) of K. A transposing read of V touches two adjacent pieces in each of its rows, so
+  // there the pair index must differ between the rows read together: V uses (l % 16) ^ 2 (row & 7).
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)pf_lds;
   auto issue_block = [&](int kb, int stage) {
     const typename KVSource<KIND>::Tiles tl = src.tiles(kb);
@@ -801,8 +802,9 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
       const int tt = row >> 4, within = row & 15;
       const bool ok = kb + row < kv_len;
       const int piece = (lane & 15) ^ (row & 15);
+      const int vpiece = (lane & 15) ^ ((row & 7) << 1);
       const bf16_t* kp = src.krow(tl, kb, tt, ok ? within : 0) + 8 * piece;
-      const bf16_t* vp = src.vrow(tl, kb, tt, ok ? within : 0) + 8 * piece;
+      const bf16_t* vp = src.vrow(tl, kb, tt, ok ? within : 0) + 8 * vpiece;
       const uint32_t dst = lds0 + stage * PFL_STAGE + (KPW * wave + 4 * j) * 256;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                    :: "s"(dst), "v"(kp) : "memory", "m0");
@@ -847,9 +849,9 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
         const int byte = 32 * f + 8 * (r16 & 3);
         const int row_lo = 32 * ch + 4 * g + (r16 >> 2), row_hi = row_lo + 16;
         const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) v4s_t*)(vs + row_lo * 256 + (((byte >> 4) ^ (row_lo & 15)) * 16) + (byte & 15)));
+            (__attribute__((address_space(3))) v4s_t*)(vs + row_lo * 256 + (((byte >> 4) ^ ((row_lo & 7) << 1)) * 16) + (byte & 15)));
         const v4s_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) v4s_t*)(vs + row_hi * 256 + (((byte >> 4) ^ (row_hi & 15)) * 16) + (byte & 15)));
+            (__attribute__((address_space(3))) v4s_t*)(vs + row_hi * 256 + (((byte >> 4) ^ ((row_hi & 7) << 1)) * 16) + (byte & 15)));
         const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
         const uint4 vf = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
 #pragma unroll
