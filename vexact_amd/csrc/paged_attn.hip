@@ -776,7 +776,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
     int v = qpos[t];
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
-    qpos_min[t] = v;
+    qpos_min[t] = __builtin_amdgcn_readfirstlane(v);  // a scalar register
   }
 
   float m[QT], l[QT], M[QT], L[QT];
