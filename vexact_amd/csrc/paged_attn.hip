@@ -118,6 +118,25 @@ struct KVSource {
 // kb + 16 tt + 4 g + r of query column r16) of the 64-key block at kb: masks keys past qpos, updates
 // the running max m and sum l, rescales the NACC accumulators and packs P (rounded to bf16; the sum
 // uses the rounded values) as the two B operands of the P V MFMAs. Shared by every attention kernel.
+// op(x, x of lane ^ 16) and op(x, x of lane ^ 32) for a commutative op, through the row-swap instructions
+// (v_permlane16_swap / v_permlane32_swap: the odd 16-lane rows of the first register trade places with the
+// even rows of the second, resp. rows 2, 3 with rows 0, 1). With both registers holding x, the two results
+// hold the lane's own row pair member and its partner's: no LDS round trip as with a general shuffle.
+// Written as asm: through the builtins the compiler used the first result for both (seen in the generated
+// code of this toolchain). The s_nop covers the wait states between a vector write of an operand and the swap.
+__device__ __forceinline__ void swap16(float x, float& a, float& b) {
+  a = x; b = x;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap32(float x, float& a, float& b) {
+  a = x; b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float max_xor16(float x) { float a, b; swap16(x, a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float max_xor32(float x) { float a, b; swap32(x, a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float add_xor16(float x) { float a, b; swap16(x, a, b); return a + b; }
+__device__ __forceinline__ float add_xor32(float x) { float a, b; swap32(x, a, b); return a + b; }
+
 template <int NACC>
 __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float c, int qpos, float& m, float& l,
                                                   f32x4 (&acc)[NACC], uint4 (&pf)[2], bool all_visible = false) {
@@ -141,8 +160,8 @@ __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float 
         bm = fmaxf(bm, tv);
       }
   }
-  bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
-  bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+  bm = max_xor16(bm);
+  bm = max_xor32(bm);
   bm = bm * c;
   const float mn = fmaxf(m, bm);
   const float ms = (mn == -INFINITY) ? 0.f : mn;  // fully masked so far: everything stays 0
@@ -161,8 +180,8 @@ __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float 
       pw[tt][h] = pk;
     }
   }
-  rs += __shfl_xor(rs, 16, 64);
-  rs += __shfl_xor(rs, 32, 64);
+  rs = add_xor16(rs);
+  rs = add_xor32(rs);
   l = l * alpha + rs;
   m = mn;
   // multiplying by exactly 1 changes nothing: skip the rescale when no lane's maximum moved
