@@ -41,7 +41,8 @@ struct AttnParams {
   bf16_t* o;  // [T, Hq, DV]
   int64_t sot, soh;
   const int* cu_q;       // [B+1]
-  const int* seqused_k;  // paged: [B] kv lengths
+  const int* seqused_k;  // paged: [B] kv lengths (clamped to max_kv: a wrong length must not walk off the block table)
+  int max_kv;            // paged: keys a block-table row can address
   const int* cu_k;       // packed: [B+1]
   const int* block_table;  // [B, bt_stride]
   int64_t bt_stride;
@@ -366,7 +367,7 @@ __device__ __forceinline__ void attn_decode_split_body(const AttnParams& p) {
   const int kvh = blockIdx.x, seq = decode_seq(p, blockIdx.y), chunk = blockIdx.z;  // chunk slowest: late chunks, mostly empty, are dispatched last
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
-  const int kv_len = p.seqused_k[seq];
+  const int kv_len = min(p.seqused_k[seq], p.max_kv);
   if (qlen <= 0 || kv_len <= 0) return;
   const int kstart = chunk * ATT_CHUNK;
   if (kstart >= kv_len) return;
@@ -446,7 +447,7 @@ __device__ __forceinline__ void attn_decode_fused_body(const AttnParams& p) {
   const int kvh = blockIdx.x, seq = decode_seq(p, blockIdx.y);
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
-  const int kv_len = p.seqused_k[seq];
+  const int kv_len = min(p.seqused_k[seq], p.max_kv);
   if (qlen <= 0 || kv_len <= 0) return;  // uniform over the block
   const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = tid >> 6;
@@ -555,7 +556,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
   const int kvh = blockIdx.x, seq = decode_seq(p, blockIdx.y);
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
-  const int kv_len = p.seqused_k[seq];
+  const int kv_len = min(p.seqused_k[seq], p.max_kv);
   if (qlen <= 0 || kv_len <= 0) return;
   const int nch = (kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
@@ -621,7 +622,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   int kv_len, k0 = 0;
-  if constexpr (KIND != SRC_PACKED) kv_len = p.seqused_k[seq];
+  if constexpr (KIND != SRC_PACKED) kv_len = min(p.seqused_k[seq], p.max_kv);
   else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int rows_per_block = 16 * (4 * QT / hpw);
@@ -743,7 +744,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   int kv_len, k0 = 0;
-  if constexpr (KIND != SRC_PACKED) kv_len = p.seqused_k[seq];
+  if constexpr (KIND != SRC_PACKED) kv_len = min(p.seqused_k[seq], p.max_kv);
   else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1162,6 +1163,10 @@ int vx_attention_ex(const void* q, const void* k, const void* v, void* out, floa
   p.causal = causal;
   p.lse = lse;
   p.seq_order = seq_order;
+  {
+    const int64_t mk = mode != 2 ? max_pages * (int64_t)page_size : 0;
+    p.max_kv = (int)(mk > 0x7fffffff ? 0x7fffffff : mk);
+  }
   if (decode) {
     const int64_t max_kv = max_pages * (int64_t)page_size;
     const int64_t nch = (max_kv + ATT_CHUNK - 1) / ATT_CHUNK;
