@@ -64,6 +64,7 @@ __global__ __launch_bounds__(256) void moe_gemm_nn_kernel(MoeNnParams p) {
   const int e = p.tile_group[t];
   if (e < 0) return;  // uniform over the block
   const int row0 = p.tile_row0[t], rows = p.tile_rows[t];
+  if (rows <= 0) return;
   const int n0 = blockIdx.x * 128;
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = threadIdx.x >> 6, wr = wave >> 1, wn = wave & 1;
