@@ -129,12 +129,16 @@ def test_scatter_gather_helpers():
     assert_bitwise(ga, acc.to(torch.bfloat16), "moe_gather")
 
 
-@pytest.mark.parametrize("T,H,I,E,k", [(1, 256, 128, 8, 2), (40, 256, 128, 8, 2), (64, 2048, 768, 128, 8), (300, 512, 256, 16, 4)])
+@pytest.mark.parametrize("T,H,I,E,k", [(1, 256, 128, 8, 2), (40, 256, 128, 8, 2), (64, 2048, 768, 128, 8), (300, 512, 256, 16, 4),
+                                       (33, 7168, 256, 256, 8),     # DeepSeek-V3-like: 256 experts, hidden 7168
+                                       (20, 4096, 1536, 16, 8)])    # Qwen3-235B-like expert shape
 def test_fused_moe_matches_fused_order_oracle(T, H, I, E, k):
     x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=11)
     out = fused_moe_forward(E, w.cuda(), sel.cuda(), x.cuda(), gate.cuda(), up.cuda(), down.cuda())
     ref = OM.fused_moe_ref(x, w, sel, gate, up, down)
-    assert_bf16_close(out, ref, max_ulp=2, atol_frac=2e-3, what="fused MoE vs fused-order oracle")
+    # an intermediate that lands on the other side of a bf16 rounding boundary (the GEMMs agree with the oracle to
+    # 2 ulp, not bit for bit) moves an output by ~2^-8 of one product: the absolute floor grows with the width I
+    assert_bf16_close(out, ref, max_ulp=2, atol_frac=2e-3 if I <= 768 else 5e-3, what="fused MoE vs fused-order oracle")
     # fused gate_up layout [E, 2I, H] (the form the Qwen3-MoE patch passes)
     gu = torch.cat([gate, up], dim=1).cuda()
     out2 = fused_moe_forward(num_experts=E, routing_weights=w.cuda(), selected_experts=sel.cuda(), hidden_states=x.cuda(),
