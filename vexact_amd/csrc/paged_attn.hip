@@ -30,6 +30,7 @@ namespace vx {
 
 constexpr int ATT_CHUNK = 256;  // keys per split chunk (absolute positions)
 constexpr int ATT_BLOCK = 64;   // keys per online-softmax block
+constexpr float ATT_LAZY = 8.f; // log2 headroom before a row's reference maximum moves
 
 struct AttnParams {
   const bf16_t* q;  // [T, Hq, DK]
@@ -164,7 +165,11 @@ __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float 
   bm = max_xor16(bm);
   bm = max_xor32(bm);
   bm = bm * c;
-  const float mn = fmaxf(m, bm);
+  // m is the reference point of the row's exponents, not necessarily its maximum: it moves only when the
+  // block's maximum exceeds it by more than ATT_LAZY (then probabilities stay below 2^ATT_LAZY, harmless
+  // in bf16 / fp32), so most blocks leave the accumulators unscaled. A function of the row's own scores
+  // only, hence the same in every kernel and for every batch.
+  const float mn = (bm > m + ATT_LAZY) ? bm : m;
   const float ms = (mn == -INFINITY) ? 0.f : mn;  // fully masked so far: everything stays 0
   const float alpha = fast_exp2(m - ms);
   float rs = 0.f;
@@ -184,9 +189,11 @@ __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float 
   rs = add_xor16(rs);
   rs = add_xor32(rs);
   l = l * alpha + rs;
+  const bool had_keys = m != -INFINITY;
   m = mn;
-  // multiplying by exactly 1 changes nothing: skip the rescale when no lane's maximum moved
-  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+  // multiplying by exactly 1 changes nothing, and a row that had seen no key holds exact zeros: skip the
+  // rescale unless some lane's reference moved away from a finite value
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f && had_keys) != 0) {
 #pragma unroll
     for (int i = 0; i < NACC; i++) {
       acc[i][0] *= alpha; acc[i][1] *= alpha; acc[i][2] *= alpha; acc[i][3] *= alpha;
@@ -332,6 +339,12 @@ struct AttnWave {
     }
   }
 };
+
+// running = running * A + chunk * B, the same expression (one product, one fused multiply-add) wherever chunk
+// states are folded, so that every kernel gives the same bits
+__device__ __forceinline__ float fold_add(float running, float A, float chunk, float B) {
+  return __builtin_fmaf(running, A, chunk * B);
+}
 
 // fold a chunk state into the running state; exact no-op for an all-masked chunk
 __device__ __forceinline__ void fold_scales(float M, float mc, float& Mn, float& A, float& B) {
@@ -511,11 +524,11 @@ __device__ __forceinline__ void attn_decode_fused_body(const AttnParams& p) {
         const float4 a = img[j * IMG4 + sl * 64 + ln];
         float Mn, A, B;
         fold_scales(M, ml.x, Mn, A, B);
-        L = L * A + ml.y * B;
-        A4.x = A4.x * A + a.x * B;
-        A4.y = A4.y * A + a.y * B;
-        A4.z = A4.z * A + a.z * B;
-        A4.w = A4.w * A + a.w * B;
+        L = fold_add(L, A, ml.y, B);
+        A4.x = fold_add(A4.x, A, a.x, B);
+        A4.y = fold_add(A4.y, A, a.y, B);
+        A4.z = fold_add(A4.z, A, a.z, B);
+        A4.w = fold_add(A4.w, A, a.w, B);
         M = Mn;
       }
       racc[e] = A4;
@@ -577,16 +590,16 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(AttnParams p) {
       const float4 ml = ip[(NI + t) * 64];
       float Mn, A, B;
       fold_scales(M, ml.x, Mn, A, B);
-      L = L * A + ml.y * B;
+      L = fold_add(L, A, ml.y, B);
 #pragma unroll
       for (int i = 0; i < NDV * 8; i++) {
         const int ds = i >> 3, r = (i >> 1) & 3;
         if (128 * ds + 32 * g + 8 * r >= DV) continue;
         const float4 a = ip[(t * NDV * 8 + i) * 64];
-        ACC[i].x = ACC[i].x * A + a.x * B;
-        ACC[i].y = ACC[i].y * A + a.y * B;
-        ACC[i].z = ACC[i].z * A + a.z * B;
-        ACC[i].w = ACC[i].w * A + a.w * B;
+        ACC[i].x = fold_add(ACC[i].x, A, a.x, B);
+        ACC[i].y = fold_add(ACC[i].y, A, a.y, B);
+        ACC[i].z = fold_add(ACC[i].z, A, a.z, B);
+        ACC[i].w = fold_add(ACC[i].w, A, a.w, B);
       }
       M = Mn;
     }
@@ -672,11 +685,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw
     for (int t = 0; t < QT; t++) {
       float Mn, A, B;
       fold_scales(M[t], w.m[t], Mn, A, B);
-      L[t] = L[t] * A + w.l[t] * B;
+      L[t] = fold_add(L[t], A, w.l[t], B);
 #pragma unroll
       for (int i = 0; i < AttnWave<DK, DV, QT>::NACC; i++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) ACC[t][i][r] = ACC[t][i][r] * A + w.acc[t][i][r] * B;
+        for (int r = 0; r < 4; r++) ACC[t][i][r] = fold_add(ACC[t][i][r], A, w.acc[t][i][r], B);
       M[t] = Mn;
     }
   }
@@ -814,22 +827,59 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   // (l % 16) ^ (row & 15) of K. A transposing read of V touches two adjacent pieces in each of its rows, so
   // there the pair index must differ between the rows read together: V uses (l % 16) ^ 2 (row & 7).
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)pf_lds;
+  // The 8 keys a wavefront brings in lie in one 16-key tile (tile wave / 2). For the paged-by-tile and the
+  // packed sources the address is therefore a wave-uniform base (scalar registers) plus a small per-lane byte
+  // offset, which keeps 64-bit per-lane address arithmetic out of the loop.
+  static_assert(KPW == 8, "a wavefront's keys must stay inside one 16-key tile");
+  const int ld_tt = wave >> 1;
   auto issue_block = [&](int kb, int stage) {
-    const typename KVSource<KIND>::Tiles tl = src.tiles(kb);
+    const uint32_t dst0 = lds0 + stage * PFL_STAGE + KPW * wave * 256;
+    if constexpr (KIND == SRC_GENERIC) {
+      const typename KVSource<KIND>::Tiles tl = src.tiles(kb);
 #pragma unroll
-    for (int j = 0; j < KPW / 4; j++) {
-      const int row = KPW * wave + 4 * j + (lane >> 4);  // key row inside the block
-      const int tt = row >> 4, within = row & 15;
-      const bool ok = kb + row < kv_len;
-      const int piece = (lane & 15) ^ (row & 15);
-      const int vpiece = (lane & 15) ^ ((row & 7) << 1);
-      const bf16_t* kp = src.krow(tl, kb, tt, ok ? within : 0) + 8 * piece;
-      const bf16_t* vp = src.vrow(tl, kb, tt, ok ? within : 0) + 8 * vpiece;
-      const uint32_t dst = lds0 + stage * PFL_STAGE + (KPW * wave + 4 * j) * 256;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                   :: "s"(dst), "v"(kp) : "memory", "m0");
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                   :: "s"(dst + ATT_BLOCK * 256), "v"(vp) : "memory", "m0");
+      for (int j = 0; j < KPW / 4; j++) {
+        const int row = KPW * wave + 4 * j + (lane >> 4);  // key row inside the block
+        const bool ok = kb + row < kv_len;
+        const bf16_t* kp = src.krow(tl, kb, ld_tt, ok ? (row & 15) : 0) + 8 * ((lane & 15) ^ (row & 15));
+        const bf16_t* vp = src.vrow(tl, kb, ld_tt, ok ? (row & 15) : 0) + 8 * ((lane & 15) ^ ((row & 7) << 1));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(dst0 + 4 * j * 256), "v"(kp) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(dst0 + 4 * j * 256 + ATT_BLOCK * 256), "v"(vp) : "memory", "m0");
+      }
+    } else {
+      // first key of the wavefront's tile, clamped like every key address: a tile that starts past the end
+      // is read from the sequence's key 0 (never used), keys past the end inside a tile re-read the last key
+      const int tile_key = kb + 16 * ld_tt;
+      int key0;
+      const bf16_t *kt, *vt;
+      if constexpr (KIND == SRC_FAST) {
+        key0 = tile_key <= src.last ? tile_key : 0;
+        const int pg = src.bt[key0 >> src.shift];
+        const int off = key0 & (src.ps - 1);
+        kt = src.kbase + (int64_t)pg * src.skb + (int64_t)off * src.skp;
+        vt = src.vbase + (int64_t)pg * src.svb + (int64_t)off * src.svp;
+      } else {
+        key0 = min(tile_key, src.last);
+        kt = src.kbase + (int64_t)key0 * src.skp;
+        vt = src.vbase + (int64_t)key0 * src.svp;
+      }
+      const uint64_t kb64 = (uint64_t)kt, vb64 = (uint64_t)vt;
+      const uint64_t ksb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(kb64 >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)kb64);
+      const uint64_t vsb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(vb64 >> 32)) << 32) |
+                           (uint32_t)__builtin_amdgcn_readfirstlane((int)vb64);
+#pragma unroll
+      for (int j = 0; j < KPW / 4; j++) {
+        const int row = KPW * wave + 4 * j + (lane >> 4);
+        const int dk = tile_key <= src.last ? min(kb + row, src.last) - key0 : 0;  // 0 .. 15
+        const uint32_t koff = (uint32_t)dk * (uint32_t)(src.skp * 2) + 16u * (uint32_t)((lane & 15) ^ (row & 15));
+        const uint32_t voff = (uint32_t)dk * (uint32_t)(src.svp * 2) + 16u * (uint32_t)((lane & 15) ^ ((row & 7) << 1));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(dst0 + 4 * j * 256), "v"(koff), "s"(ksb) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(dst0 + 4 * j * 256 + ATT_BLOCK * 256), "v"(voff), "s"(vsb) : "memory", "m0");
+      }
     }
   };
 
@@ -897,11 +947,11 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
       for (int t = 0; t < QT; t++) {
         float Mn, A, B;
         fold_scales(M[t], m[t], Mn, A, B);
-        L[t] = L[t] * A + l[t] * B;
+        L[t] = fold_add(L[t], A, l[t], B);
 #pragma unroll
         for (int i = 0; i < 8; i++)
 #pragma unroll
-          for (int r = 0; r < 4; r++) ACC[t][i][r] = ACC[t][i][r] * A + acc[t][i][r] * B;
+          for (int r = 0; r < 4; r++) ACC[t][i][r] = fold_add(ACC[t][i][r], A, acc[t][i][r], B);
         M[t] = Mn;
       }
     }
