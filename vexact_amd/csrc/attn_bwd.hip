@@ -321,13 +321,18 @@ __device__ __forceinline__ void bwl_issue_rows(const bf16_t* base, int64_t row_s
                                                uint32_t lds_arr, int wave) {
   const int lane = threadIdx.x & 63;
   constexpr int RPW = 64 / NW;
+  // wave-uniform base (scalar registers) + 32-bit lane offset: rows past the end re-read the last row
+  const int r0 = min(first_row, last_row);
+  const uint64_t b64 = (uint64_t)(base + (int64_t)r0 * row_stride);
+  const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b64 >> 32)) << 32) |
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)b64);
 #pragma unroll
   for (int j = 0; j < RPW / 4; j++) {
     const int row = RPW * wave + 4 * j + (lane >> 4);
     const int piece = (lane & 15) ^ bwl_swz(row);
-    const bf16_t* src = base + (int64_t)min(first_row + row, last_row) * row_stride + 8 * piece;
+    const uint32_t voff = (uint32_t)(min(first_row + row, last_row) - r0) * (uint32_t)(row_stride * 2) + 16u * (uint32_t)piece;
     const uint32_t dst = lds_arr + (RPW * wave + 4 * j) * 256;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(voff), "s"(sb) : "memory", "m0");
   }
 }
 // A operand of a score product: row 16 tt + r16 of the array, dims 32 s + 8 g .. +8
