@@ -92,20 +92,38 @@ __global__ __launch_bounds__(256) void moe_gemm_nn_kernel(MoeNnParams p) {
       ap[rt] = a + (int64_t)r * lda + 8 * g;
     }
     // this thread's two 16-byte pieces of a weight tile: piece q = tid + 256 j -> row q / 16, piece q % 16
+    // A step that lies fully inside K (and a column tile fully inside N) is loaded without masks: the masks
+    // cost four selects per load, as many vector instructions as the products they feed.
+    const bool full_n = n0 + 128 <= p.N;  // uniform
     auto load_w = [&](int k0, uint4 (&wreg)[GB_PIECES]) {
+      if (full_n && k0 + GB_ROWS <= K) {
 #pragma unroll
-      for (int j = 0; j < GB_PIECES; j++) {
-        const int q = threadIdx.x + 256 * j, row = q >> 4, pc = q & 15;
-        const bool ok = k0 + row < K && n0 + 8 * pc < p.N;
-        wreg[j] = ldg16(ok ? (const void*)(w + (int64_t)(k0 + row) * ldw + n0 + 8 * pc) : (const void*)w, ok);
+        for (int j = 0; j < GB_PIECES; j++) {
+          const int q = threadIdx.x + 256 * j;
+          wreg[j] = ldg16_raw(w + (int64_t)(k0 + (q >> 4)) * ldw + n0 + 8 * (q & 15));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < GB_PIECES; j++) {
+          const int q = threadIdx.x + 256 * j, row = q >> 4, pc = q & 15;
+          const bool ok = k0 + row < K && n0 + 8 * pc < p.N;
+          wreg[j] = ldg16(ok ? (const void*)(w + (int64_t)(k0 + row) * ldw + n0 + 8 * pc) : (const void*)w, ok);
+        }
       }
     };
     auto load_a = [&](int k0, uint4 (&af)[GB_ROWS / 32][4]) {
+      if (k0 + GB_ROWS <= K) {
 #pragma unroll
-      for (int kc = 0; kc < GB_ROWS / 32; kc++) {
-        const bool ok = k0 + 32 * kc + 8 * g < K;
+        for (int kc = 0; kc < GB_ROWS / 32; kc++)
 #pragma unroll
-        for (int rt = 0; rt < 4; rt++) af[kc][rt] = ldg16(ok ? ap[rt] + k0 + 32 * kc : a, ok);
+          for (int rt = 0; rt < 4; rt++) af[kc][rt] = ldg16_raw(ap[rt] + k0 + 32 * kc);
+      } else {
+#pragma unroll
+        for (int kc = 0; kc < GB_ROWS / 32; kc++) {
+          const bool ok = k0 + 32 * kc + 8 * g < K;
+#pragma unroll
+          for (int rt = 0; rt < 4; rt++) af[kc][rt] = ldg16(ok ? ap[rt] + k0 + 32 * kc : a, ok);
+        }
       }
     };
     const int steps = (K + GB_ROWS - 1) / GB_ROWS;
@@ -314,13 +332,24 @@ __global__ __launch_bounds__(512) void moe_gemm_tn_wide_kernel(MoeTnParams p) {
       rx[j] = ok ? (p.x_src ? p.x_src[r] : r) : -1;
     }
   };
-  auto load_tiles = [&](const int (&ry)[2], const int (&rx)[2], uint4 (&yr)[2], uint4 (&xr)[2]) {
+  // `full` (uniform): every row of the step exists and the output tile lies inside N x K: no masks
+  const bool full_nk = n0 + 256 <= p.N && k0 + 256 <= p.K;
+  auto load_tiles = [&](bool full, const int (&ry)[2], const int (&rx)[2], uint4 (&yr)[2], uint4 (&xr)[2]) {
+    if (full) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const int pc = (threadIdx.x + 512 * j) & 31;
-      const bool oky = ry[j] >= 0 && n0 + 8 * pc < p.N, okx = rx[j] >= 0 && k0 + 8 * pc < p.K;
-      yr[j] = ldg16(oky ? (const void*)(p.dy + (int64_t)ry[j] * p.lddy + n0 + 8 * pc) : (const void*)p.dy, oky);
-      xr[j] = ldg16(okx ? (const void*)(p.x + (int64_t)rx[j] * p.ldx + k0 + 8 * pc) : (const void*)p.x, okx);
+      for (int j = 0; j < 2; j++) {
+        const int pc = (threadIdx.x + 512 * j) & 31;
+        yr[j] = ldg16_raw(p.dy + (int64_t)ry[j] * p.lddy + n0 + 8 * pc);
+        xr[j] = ldg16_raw(p.x + (int64_t)rx[j] * p.ldx + k0 + 8 * pc);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int pc = (threadIdx.x + 512 * j) & 31;
+        const bool oky = ry[j] >= 0 && n0 + 8 * pc < p.N, okx = rx[j] >= 0 && k0 + 8 * pc < p.K;
+        yr[j] = ldg16(oky ? (const void*)(p.dy + (int64_t)ry[j] * p.lddy + n0 + 8 * pc) : (const void*)p.dy, oky);
+        xr[j] = ldg16(okx ? (const void*)(p.x + (int64_t)rx[j] * p.ldx + k0 + 8 * pc) : (const void*)p.x, okx);
+      }
     }
   };
 
@@ -328,9 +357,9 @@ __global__ __launch_bounds__(512) void moe_gemm_tn_wide_kernel(MoeTnParams p) {
   uint4 yr[2][2], xr[2][2];  // register set (s & 1) holds step s
   int ry[2], rx[2];          // row numbers of the next step to be loaded
   load_rows(lo, ry, rx);
-  if (steps > 0) load_tiles(ry, rx, yr[0], xr[0]);
+  if (steps > 0) load_tiles(full_nk && lo + TW_ROWS <= hi, ry, rx, yr[0], xr[0]);
   load_rows(lo + TW_ROWS, ry, rx);
-  if (steps > 1) load_tiles(ry, rx, yr[1], xr[1]);
+  if (steps > 1) load_tiles(full_nk && lo + 2 * TW_ROWS <= hi, ry, rx, yr[1], xr[1]);
   load_rows(lo + 2 * TW_ROWS, ry, rx);
   auto step = [&](int s, int buf, uint4 (&yrs)[2], uint4 (&xrs)[2]) {
 #pragma unroll
@@ -342,7 +371,7 @@ __global__ __launch_bounds__(512) void moe_gemm_tn_wide_kernel(MoeTnParams p) {
     }
     __syncthreads();  // also: everyone is done reading the other buffer's previous contents
     if (s + 2 < steps) {
-      load_tiles(ry, rx, yrs, xrs);
+      load_tiles(full_nk && lo + (s + 3) * TW_ROWS <= hi, ry, rx, yrs, xrs);
       load_rows(lo + (s + 3) * TW_ROWS, ry, rx);
     }
     uint4 yf[8], xf[4];
