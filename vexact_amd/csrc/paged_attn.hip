@@ -884,6 +884,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   };
 
   auto block_compute = [&](int kb, int stage) {
+    __builtin_amdgcn_iglp_opt(1);  // scheduling hint: interleave the LDS fragment reads with the MFMAs (measured 3-4 %)
     const uint8_t* ks = pf_lds + stage * PFL_STAGE;
     const uint8_t* vs = ks + ATT_BLOCK * 256;
     // ---- S^T = K Q^T: the key fragments are shared by both query tiles; per accumulator the k-steps
