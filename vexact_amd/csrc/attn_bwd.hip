@@ -403,9 +403,14 @@ __global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwd
   const float c2 = p.scale * 1.44269504f;
   const float lse2 = p.lse[tq * p.Hq + h] * 1.44269504f;
   const float delta = p.delta[tq * p.Hq + h];
-  int wave_maxpos = pos;  // last key this wavefront's queries see
+  int wave_maxpos = pos, wave_minpos = pos;  // last key this wavefront's queries see; first row's limit (-1: a row is missing)
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) wave_maxpos = max(wave_maxpos, __shfl_xor(wave_maxpos, o, 64));
+  for (int o = 32; o > 0; o >>= 1) {
+    wave_maxpos = max(wave_maxpos, __shfl_xor(wave_maxpos, o, 64));
+    wave_minpos = min(wave_minpos, __shfl_xor(wave_minpos, o, 64));
+  }
+  wave_maxpos = __builtin_amdgcn_readfirstlane(wave_maxpos);
+  wave_minpos = __builtin_amdgcn_readfirstlane(wave_minpos);
   f32x4 acc[8];
 #pragma unroll
   for (int f = 0; f < 8; f++) acc[f] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -420,13 +425,14 @@ __global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwd
     bwl_issue_rows(vb_, p.svt, kb, kv_len - 1, lds0 + stage * BWL_STAGE + BWL_ARR, wave);
   };
   if (blk_maxpos >= 0) issue_block(0, 0);
-  for (int kb = 0, stage = 0; kb <= blk_maxpos; kb += 64, stage ^= 1) {
+  auto one_block = [&](int kb, const int stage) __attribute__((always_inline)) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // block kb is in LDS for everyone; everyone is done with the other stage
     if (kb + 64 <= blk_maxpos) issue_block(kb + 64, stage ^ 1);
-    if (kb > wave_maxpos) continue;  // nothing visible to this wavefront any more (it keeps loading and syncing)
+    if (kb > wave_maxpos) return;  // nothing visible to this wavefront any more (it keeps loading and syncing)
     const uint8_t* ks = bw_lds + stage * BWL_STAGE;
     const uint8_t* vs = ks + BWL_ARR;
+    const bool all_visible = kb + 63 <= wave_minpos;  // uniform: no key of the block is masked for any row
     float ds[4][4];
 #pragma unroll
     for (int tt = 0; tt < 4; tt++) {
@@ -436,17 +442,26 @@ __global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwd
         st = mfma16(bwl_frag(ks, tt, s), qf[s], st);
         dp = mfma16(bwl_frag(vs, tt, s), of[s], dp);
       }
+      if (all_visible) {
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int key = kb + 16 * tt + 4 * g + r;
-        const float pr = (key <= pos) ? __builtin_amdgcn_exp2f(st[r] * c2 - lse2) : 0.f;
-        ds[tt][r] = pr * (dp[r] - delta) * p.scale;
+        for (int r = 0; r < 4; r++)
+          ds[tt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[r], c2, -lse2)) * (dp[r] - delta) * p.scale;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int key = kb + 16 * tt + 4 * g + r;
+          const float pr = (key <= pos) ? __builtin_amdgcn_exp2f(__builtin_fmaf(st[r], c2, -lse2)) : 0.f;
+          ds[tt][r] = pr * (dp[r] - delta) * p.scale;
+        }
       }
     }
     uint4 pf[2];
     bwd_pack(ds, pf);
     bwl_tr_product(ks, pf, acc);
-  }
+  };
+  // (unrolling over the two stages would make the LDS offsets immediates but costs 13 registers, which
+  // takes the kernel over 128 and halves the wavefronts per SIMD)
+  for (int kb = 0, stage = 0; kb <= blk_maxpos; kb += 64, stage ^= 1) one_block(kb, stage);
   if (qok) bwl_store_tile(acc, p.dq + tq * p.sdqt + (int64_t)h * p.sdqh);
 }
 
@@ -510,16 +525,19 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
     }
   };
   if (nsteps > 0) issue_step(0, 0);
-  for (int step = 0, stage = 0; step < nsteps; step++, stage ^= 1) {
+  const bool tile_full = j0 + 15 < kv_len;  // uniform: every key of this wavefront's tile exists
+  auto one_step = [&](int step, const int stage) __attribute__((always_inline)) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // this step's rows are in LDS for everyone; everyone is done with the other stage
     if (step + 1 < nsteps) issue_step(step + 1, stage ^ 1);
     const int ib = ib0 + 64 * (step % nblk);
-    if (ib + 63 + shift < j0) continue;  // none of the block's queries sees any key of this wavefront's tile
+    if (ib + 63 + shift < j0) return;  // none of the block's queries sees any key of this wavefront's tile
     const uint8_t* qs = bw_lds + stage * BWK_STAGE;
     const uint8_t* os = qs + BWL_ARR;
     const float* lse_s = (const float*)(os + BWL_ARR);
     const float* del_s = lse_s + 64;
+    // uniform: all 64 queries exist and even the first of them sees the tile's last key
+    const bool all_visible = tile_full && ib + 63 < qlen && j0 + 15 <= shift + ib;
     float pr[4][4], ds[4][4];
 #pragma unroll
     for (int tt = 0; tt < 4; tt++) {
@@ -532,13 +550,22 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
       const float4 l4 = *(const float4*)(lse_s + 16 * tt + 4 * g);
       const float4 d4 = *(const float4*)(del_s + 16 * tt + 4 * g);
       const float lr[4] = {l4.x, l4.y, l4.z, l4.w}, dr[4] = {d4.x, d4.y, d4.z, d4.w};
+      if (all_visible) {
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int iq = ib + 16 * tt + 4 * g + r;  // this register's query (moving row)
-        const bool ok = iq < qlen && kok && j <= shift + iq;
-        const float e = ok ? __builtin_amdgcn_exp2f(st[r] * c2 - lr[r] * 1.44269504f) : 0.f;
-        pr[tt][r] = e;
-        ds[tt][r] = e * (dp[r] - dr[r]) * p.scale;
+        for (int r = 0; r < 4; r++) {
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(st[r], c2, -(lr[r] * 1.44269504f)));
+          pr[tt][r] = e;
+          ds[tt][r] = e * (dp[r] - dr[r]) * p.scale;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int iq = ib + 16 * tt + 4 * g + r;  // this register's query (moving row)
+          const bool ok = iq < qlen && kok && j <= shift + iq;
+          const float e = ok ? __builtin_amdgcn_exp2f(__builtin_fmaf(st[r], c2, -(lr[r] * 1.44269504f))) : 0.f;
+          pr[tt][r] = e;
+          ds[tt][r] = e * (dp[r] - dr[r]) * p.scale;
+        }
       }
     }
     uint4 pfp[2], pfs[2];
@@ -546,6 +573,10 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
     bwd_pack(ds, pfs);
     bwl_tr_product(os, pfp, dv);
     bwl_tr_product(qs, pfs, dk);
+  };
+  for (int step = 0; step < nsteps; step += 2) {
+    one_step(step, 0);
+    if (step + 1 < nsteps) one_step(step + 1, 1);
   }
   if (kok) {
     bwl_store_tile(dk, p.dk + tk * p.sdkt + (int64_t)kvh * p.sdkh);
