@@ -42,6 +42,8 @@ def parse():
     ap.add_argument("--max-prompt", type=int, default=2048)
     ap.add_argument("--drift-requests", type=int, default=8, help="requests re-run at batch 1 for the bit-drift check")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-packed-experts", action="store_true",
+                    help="decode reads the [E, N, K] expert tensors instead of their fragment-order copies")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--seed", type=int, default=5)
     ap.add_argument("--cpu-configs", action="store_true",
@@ -179,6 +181,25 @@ def main():
     del pb
     torch.cuda.empty_cache()
 
+    # ---- decode streams the expert weights from their fragment-order copies (made once per weight update)
+    if not args.no_packed_experts:
+        w.pack_experts()
+        torch.cuda.synchronize()
+
+    def moe_gate_up(li, lw, r):
+        if w.packed is not None:
+            pg = w.packed[li][0]
+            return ops.moe_gemm_packed(db.h, pg.rows(0, I), r, w2=pg.rows(I, 2 * I), row_src=r.sorted_token,
+                                       row_scale=db.topk_w, row_scale_idx=r.sorted_flat, out=db.hw)
+        gu = lw["gate_up"]
+        return ops.moe_gemm(db.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=db.topk_w,
+                            row_scale_idx=r.sorted_flat, out=db.hw)
+
+    def moe_down(li, lw, r):
+        if w.packed is not None:
+            return ops.moe_gemm_packed(db.hw, w.packed[li][1], r, out=db.eo)
+        return ops.moe_gemm(db.hw, lw["down"], r, out=db.eo)
+
     # ---- the decode step: 256 tokens, 256 sequences, captured in a HIP graph
     ctx = [int(n) + 1 for n in prompt_lens]
     reqs = [dict(num_computed_tokens=ctx[i], tokens_this_step=1, block_ids=blocks[i]) for i in range(B)]
@@ -247,10 +268,8 @@ def main():
             r = ops.moe_route(db.topk_idx, E, bm=db.bm, buffers=db.route_ints)
             if rep == 0:
                 experts_hit.append(int((r.splits > 0).sum()))
-            gu = lw["gate_up"]
-            timed("moe_gate_up", lambda: ops.moe_gemm(db.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token,
-                                                      row_scale=db.topk_w, row_scale_idx=r.sorted_flat, out=db.hw))
-            timed("moe_down", lambda: ops.moe_gemm(db.hw, lw["down"], r, out=db.eo))
+            timed("moe_gate_up", lambda: moe_gate_up(li, lw, r))
+            timed("moe_down", lambda: moe_down(li, lw, r))
             nxt = w.layers[li + 1]["in_norm"] if li + 1 < cfg.num_layers else w.final_norm
             ops.moe_gather(db.eo, r.scatter_index, residual=db.x, out=db.x)
             ops.rms_norm(db.x, nxt, cfg.rms_eps, hf_two_rounding=True, out=db.h)
@@ -267,10 +286,8 @@ def main():
     side.wait_stream(torch.cuda.current_stream())
 
     def gate_up_all_layers():
-        for lw_ in w.layers:
-            gu_ = lw_["gate_up"]
-            ops.moe_gemm(db.h, gu_[:, :I, :], r, w2=gu_[:, I:, :], row_src=r.sorted_token, row_scale=db.topk_w,
-                         row_scale_idx=r.sorted_flat, out=db.hw)
+        for li_, lw_ in enumerate(w.layers):
+            moe_gate_up(li_, lw_, r)
 
     with torch.cuda.stream(side):
         gate_up_all_layers()
@@ -312,7 +329,7 @@ def main():
             traffic = None
     kernels[dom]["in_graph_avg_us"] = round(avg_in_graph * 1e6, 1)
     achieved = kbytes[dom] / avg_in_graph / 1e9
-    roofline = {"bound": "hbm", "kernel": "gemm_stream_kernel<2, SWIGLU, grouped> (MoE gate/up)",
+    roofline = {"bound": "hbm", "kernel": "gemm_stream_kernel<2, SWIGLU, grouped%s> (MoE gate/up)" % (", packed" if w.packed is not None else ""),
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "timing": "HIP events around graph replays of 48 back-to-back launches (one per layer's weights)"}

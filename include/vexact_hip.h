@@ -204,6 +204,24 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
                 const int* row_src, const void* row_scale, const int* row_scale_idx, int epi, int64_t x_rows,
                 hipStream_t stream);
 
+/* Fragment-order ("packed") copy of [G][N][K] bf16 weights for the weight-streaming kernels, made once per
+ * weight update. No counterpart in the reference (its grouped GEMM, group_gemm/kernel/group_gemm.py:65-153,
+ * reads [E, N, K] as stored): the values and every product are the same, only the order in HBM differs, so
+ * that a wavefront reads one linear run per 16 weight rows instead of 16 pitched rows.
+ *   out[g][nb][c][lane][8] = W_g[16 nb + lane % 16][32 c + 8 (lane / 16) .. + 8], zero past N and K,
+ *   nb < ceil(N / 16), c < vx_packed_kchunks(K) (K rounded up to a multiple of 256, in 32-wide chunks):
+ *   G * ceil(N / 16) * vx_packed_kchunks(K) * 512 elements. */
+int vx_packed_kchunks(int64_t K);
+int vx_pack_weights(const void* w, int64_t ldw, int64_t w_gstride, int64_t G, int64_t N, int64_t K, void* out,
+                    hipStream_t stream);
+/* vx_moe_gemm on packed weights, bm in {16, 32, 64} (decode sizes). w (and w2 for epi 1) point at the packed
+ * image of the projection's first row, which must lie a multiple of 16 rows into the packed tensor;
+ * w_gstride = elements between consecutive experts there. Same bits as vx_moe_gemm. */
+int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2, int64_t w_gstride, void* c,
+                       int64_t ldc, int64_t N, int64_t K, const int* tile_group, const int* tile_row0,
+                       const int* tile_rows, int64_t max_tiles, int bm, const int* row_src, const void* row_scale,
+                       const int* row_scale_idx, int epi, hipStream_t stream);
+
 /* Grouped products of the fused-MoE backward (FusedMoeExpertFunction.backward, fused_moe.py:126-265), bf16
  * with fp32 accumulation, over the same tile table / expert offsets as the forward.
  *   vx_moe_gemm_nn: C[rows of expert e] = A[a_src[rows]] W_e (+ A2[rows] W2_e): the data gradient through a

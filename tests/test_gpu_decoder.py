@@ -216,3 +216,29 @@ def test_sampled_decode_is_batch_invariant_and_graph_safe():
     g.replay()
     torch.cuda.synchronize()
     assert torch.equal(bg.tokens.cpu()[:5], tok_e[order])
+
+
+def test_decode_on_packed_expert_weights_keeps_every_bit():
+    # the same decode step with the experts streamed from their fragment-order copies: eager and in a graph
+    cfg, w, dec, prompts, blocks = _setup(num_seqs=6, seed=9)
+    allseq = list(range(6))
+    tok, _, _, _ = _prefill(dec, cfg, prompts, blocks, allseq)
+    dmeta = _decode_meta(cfg, prompts, blocks, allseq)
+    b = dec.bucket(6, 6)
+    b.load(dmeta, tok.numpy())
+    dec.step(b, 1)
+    torch.cuda.synchronize()
+    lp0, tok0 = b.logprobs.cpu().clone(), b.tokens.cpu().clone()
+    w.pack_experts()
+    b.load(dmeta, tok.numpy())
+    dec.step(b, 1)
+    torch.cuda.synchronize()
+    assert_bitwise(b.logprobs.cpu(), lp0, "decode logprobs: packed vs [E, N, K] expert weights")
+    assert torch.equal(b.tokens.cpu(), tok0)
+    b.load(dmeta, tok.numpy())
+    graph = dec.capture(b, 1)
+    for _ in range(2):
+        b.logprobs.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bitwise(b.logprobs.cpu(), lp0, "graph replay on packed expert weights")

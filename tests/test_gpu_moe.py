@@ -360,3 +360,42 @@ def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
     u = matmul_ref(x[0, :5], gu[3, 128:].t())
     dense = matmul_ref((torch.nn.functional.silu(g.float()).to(torch.bfloat16).float() * u.float()).to(torch.bfloat16), dn[3].t())
     assert_bf16_close(one, dense, max_ulp=2, atol_frac=2e-3, what="single expert as a dense MLP")
+
+
+def _pack_restatement(w: torch.Tensor, kchunks: int) -> torch.Tensor:
+    """Fragment order by index arithmetic on the CPU: out[e][nb][c][lane][j] = W_e[16 nb + lane % 16][32 c + 8 (lane // 16) + j]."""
+    E, N, K = w.shape
+    nb = (N + 15) // 16
+    pad = torch.zeros(E, nb * 16, kchunks * 32, dtype=w.dtype)
+    pad[:, :N, :K] = w
+    v = pad.view(E, nb, 16, kchunks, 4, 8)  # [e, nb, r16, c, g, j]
+    return v.permute(0, 1, 3, 4, 2, 5).contiguous().view(-1)  # [e, nb, c, g, r16, j]
+
+
+@pytest.mark.parametrize("E,N,K", [(3, 64, 256), (2, 40, 100), (5, 48, 768), (1, 17, 8)])
+def test_pack_expert_weights_is_an_exact_permutation(E, N, K):
+    g = torch.Generator().manual_seed(31)
+    buf = torch.randn(E, N, K + 24, generator=g).to(torch.bfloat16)
+    w = buf[:, :, :K]  # pitched rows
+    pk = ops.pack_expert_weights(w.cuda())
+    assert pk.kchunks == (K + 255) // 256 * 8
+    assert_bitwise(pk.data.cpu(), _pack_restatement(w, pk.kchunks), "packed weights")
+
+
+@pytest.mark.parametrize("T,H,I,E,k", [(1, 512, 256, 32, 4), (70, 512, 256, 32, 4), (256, 2048, 768, 128, 8), (33, 200, 80, 6, 2)])
+def test_packed_expert_weights_give_the_same_bits(T, H, I, E, k):
+    # decode-sized steps on the fragment-order copy of the weights against the [E, N, K] tensors, at every
+    # streaming tile height; ragged K (200, 80) and N (80) exercise the zero fill of the packed image
+    x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=41)
+    xg, wg, sg, dg = x.cuda(), w.cuda(), sel.cuda(), down.cuda()
+    gu = torch.cat([gate, up], dim=1).cuda()  # [E, 2I, H], gate rows first
+    pgu, pdn = ops.pack_expert_weights(gu), ops.pack_expert_weights(dg)
+    for bm in (16, 32, 64):
+        r = ops.moe_route(sg, E, bm=bm)
+        hw = ops.moe_gemm(xg, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=wg, row_scale_idx=r.sorted_flat)
+        eo = ops.moe_gemm(hw, dg, r)
+        hw_p = ops.moe_gemm_packed(xg, pgu.rows(0, I), r, w2=pgu.rows(I, 2 * I), row_src=r.sorted_token, row_scale=wg,
+                                   row_scale_idx=r.sorted_flat)
+        eo_p = ops.moe_gemm_packed(hw, pdn, r)
+        assert_bitwise(hw_p, hw, f"gate/up + SwiGLU on packed weights, {bm}-row tiles")
+        assert_bitwise(eo_p, eo, f"down projection on packed weights, {bm}-row tiles")

@@ -57,7 +57,11 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u, float w) {
 // U  = k-steps of weight loads a wavefront keeps in flight (one group);
 // KD = divisor of the staged K chunk: KC = 32768 / (BM * KD) elements per LDS fill (64 KB / KD of
 //      LDS per block, so KD = 2 lets more blocks share a CU). 32 U must divide KC.
-template <int MT, int EPI, bool GROUPED, int U = 8, int KD = 1>
+// PACKED: the weights are in fragment order (pack_weights_kernel): the 1 KB that the 64 lanes of a
+// wavefront feed to one MFMA (16 weight rows x 32 k) is contiguous and in lane order, so a wavefront
+// streams one linear run of (K / 32) KB per 16-row block instead of 16 rows of pitch ldw. p.ldw is then
+// the number of 32-wide k-chunks stored per row block (K rounded up to a multiple of 32 U, zero filled).
+template <int MT, int EPI, bool GROUPED, int U = 8, int KD = 1, bool PACKED = false>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   constexpr int BM = 16 * MT;
   constexpr int KC = 32768 / (BM * KD);  // K elements staged per LDS fill
@@ -82,10 +86,17 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 64 + wave * 16;
   const int K = p.K;
-  const int nrow = min(n0 + r16, p.N - 1);
-  const bf16_t* wp = p.w + wbase + (int64_t)nrow * p.ldw + 8 * g;
+  const bf16_t* wp;
   const bf16_t* wp2 = nullptr;
-  if constexpr (EPI == EPI_SWIGLU) wp2 = p.w2 + wbase + (int64_t)nrow * p.ldw + 8 * g;
+  if constexpr (PACKED) {
+    const int64_t woff = wbase + (int64_t)min(n0 >> 4, ((p.N + 15) >> 4) - 1) * p.ldw * 512 + lane * 8;
+    wp = p.w + woff;
+    if constexpr (EPI == EPI_SWIGLU) wp2 = p.w2 + woff;
+  } else {
+    const int nrow = min(n0 + r16, p.N - 1);
+    wp = p.w + wbase + (int64_t)nrow * p.ldw + 8 * g;
+    if constexpr (EPI == EPI_SWIGLU) wp2 = p.w2 + wbase + (int64_t)nrow * p.ldw + 8 * g;
+  }
 
   f32x4 acc[MT], acc2[EPI == EPI_SWIGLU ? MT : 1];
 #pragma unroll
@@ -100,7 +111,21 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   // masking so the loads stay in flight across the MFMAs of the previous group; only a ragged last
   // group (K not a multiple of 32*U) pays for masks, and a group past K is all zeros.
   auto load_w = [&](int kstep0) {
-    if (kstep0 + 32 * U <= K) {
+    if constexpr (PACKED) {  // chunk c of the row block lies at 512 c elements; stored chunks past K are zero
+      if (kstep0 < K) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          wa[u] = ldg16_raw(wp + (int64_t)(kstep0 + 32 * u) * 16);
+          if constexpr (EPI == EPI_SWIGLU) wb[u] = ldg16_raw(wp2 + (int64_t)(kstep0 + 32 * u) * 16);
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          wa[u] = make_uint4(0, 0, 0, 0);
+          if constexpr (EPI == EPI_SWIGLU) wb[u] = make_uint4(0, 0, 0, 0);
+        }
+      }
+    } else if (kstep0 + 32 * U <= K) {
 #pragma unroll
       for (int u = 0; u < U; u++) {
         wa[u] = ldg16_raw(wp + kstep0 + 32 * u);

@@ -473,6 +473,31 @@ __global__ __launch_bounds__(256) void moe_gather_vec_kernel(const bf16_t* __res
 
 using namespace vx;
 
+// Fragment-order copy of [G][N][K] weights for the PACKED streaming kernel.
+__global__ __launch_bounds__(256) void pack_weights_kernel(const bf16_t* __restrict__ w, int64_t ldw, int64_t gstride,
+                                                           int N, int K, int kch, bf16_t* __restrict__ out,
+                                                           int64_t pieces) {
+  const int64_t pc = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (pc >= pieces) return;
+  const int lane = (int)(pc & 63);
+  const int64_t frag = pc >> 6;
+  const int c = (int)(frag % kch);
+  const int64_t nbg = frag / kch;
+  const int nblocks = (N + 15) >> 4;
+  const int nb = (int)(nbg % nblocks);
+  const int64_t grp = nbg / nblocks;
+  const int n = 16 * nb + (lane & 15), k0 = 32 * c + 8 * (lane >> 4);
+  bf16_t v[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) v[j] = (n < N && k0 + j < K) ? w[grp * gstride + (int64_t)n * ldw + k0 + j] : (bf16_t)0;
+  uint4 o;
+  o.x = (uint32_t)v[0] | ((uint32_t)v[1] << 16);
+  o.y = (uint32_t)v[2] | ((uint32_t)v[3] << 16);
+  o.z = (uint32_t)v[4] | ((uint32_t)v[5] << 16);
+  o.w = (uint32_t)v[6] | ((uint32_t)v[7] << 16);
+  *(uint4*)(out + pc * 8) = o;
+}
+
 extern "C" {
 
 int vx_router_topk(const void* logits, void* weights_out, void* idx_out, int64_t T, int E, int k,
@@ -631,6 +656,64 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
     default: return VX_ERR_ARG;
   }
 #undef VX_GG
+  return launch_status();
+}
+
+// ---- fragment-order ("packed") expert weights for the streaming kernel ----
+// out[g][nb][c][lane][8] = W_g[16 nb + lane % 16][32 c + 8 (lane / 16) .. + 8], zero past N and K; nb < ceil(N / 16),
+// c < kchunks. One thread per 16-byte piece.
+int vx_packed_kchunks(int64_t K) { return (int)((K + 255) / 256 * 8); }
+
+int vx_pack_weights(const void* w, int64_t ldw, int64_t w_gstride, int64_t G, int64_t N, int64_t K, void* out,
+                    hipStream_t stream) {
+  if (!w || !out || G <= 0 || N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff) return VX_ERR_ARG;
+  if (ldw < K || ((uintptr_t)out % 16) != 0) return VX_ERR_ARG;
+  const int kch = vx_packed_kchunks(K);
+  const int64_t pieces = G * ((N + 15) / 16) * kch * 64;
+  const int64_t blocks = (pieces + 255) / 256;
+  if (blocks > 0x7fffffff) return VX_ERR_UNSUPPORTED;
+  pack_weights_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)w, ldw, w_gstride, (int)N, (int)K, kch,
+                                                            (bf16_t*)out, pieces);
+  return launch_status();
+}
+
+// vx_moe_gemm on packed weights (streaming kernel only: bm in {16, 32, 64}). w / w2 point at the packed
+// image of the first row of the gate / up (or only) projection, which must be a multiple of 16 rows into
+// the packed tensor; w_gstride = elements between consecutive experts in the packed tensor.
+int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2, int64_t w_gstride, void* c,
+                       int64_t ldc, int64_t N, int64_t K, const int* tile_group, const int* tile_row0,
+                       const int* tile_rows, int64_t max_tiles, int bm, const int* row_src, const void* row_scale,
+                       const int* row_scale_idx, int epi, hipStream_t stream) {
+  if (!x || !w || !c || !tile_group || !tile_row0 || !tile_rows) return VX_ERR_ARG;
+  if (N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff || max_tiles < 0) return VX_ERR_ARG;
+  if (epi != EPI_PLAIN && epi != EPI_SWIGLU) return VX_ERR_ARG;
+  if (epi == EPI_SWIGLU && (!w2 || !row_scale)) return VX_ERR_ARG;
+  if (bm != 16 && bm != 32 && bm != 64) return VX_ERR_ARG;
+  if (((uintptr_t)x % 16) != 0 || ((uintptr_t)w % 16) != 0 || (ldx % 8) != 0 || (w_gstride % 8) != 0)
+    return VX_ERR_UNSUPPORTED;
+  if (epi == EPI_SWIGLU && ((uintptr_t)w2 % 16) != 0) return VX_ERR_UNSUPPORTED;
+  if (max_tiles == 0) return VX_OK;
+  if (max_tiles > 65535) return VX_ERR_UNSUPPORTED;
+  GemmParams p = {};
+  p.x = (const bf16_t*)x; p.ldx = ldx;
+  p.w = (const bf16_t*)w; p.w2 = (const bf16_t*)w2; p.ldw = vx_packed_kchunks(K); p.w_gstride = w_gstride;
+  p.c = (bf16_t*)c; p.ldc = ldc;
+  p.M = 0; p.N = (int)N; p.K = (int)K;
+  p.tile_group = tile_group; p.tile_row0 = tile_row0; p.tile_rows = tile_rows;
+  p.row_src = row_src;
+  p.row_scale = (const bf16_t*)row_scale; p.row_scale_idx = row_scale_idx;
+  const dim3 grid((unsigned)((N + 63) / 64), (unsigned)max_tiles);
+#define VX_GP(MT)                                                                                            \
+  do {                                                                                                       \
+    if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true, 8, 2, true><<<grid, 256, 0, stream>>>(p); \
+    else gemm_stream_kernel<MT, EPI_PLAIN, true, 8, 2, true><<<grid, 256, 0, stream>>>(p);                    \
+  } while (0)
+  switch (bm) {
+    case 16: VX_GP(1); break;
+    case 32: VX_GP(2); break;
+    default: VX_GP(4); break;
+  }
+#undef VX_GP
   return launch_status();
 }
 

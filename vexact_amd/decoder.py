@@ -104,6 +104,14 @@ class DecoderWeights:
                 )
             )
 
+        self.packed = None
+
+    def pack_experts(self) -> None:
+        """Add fragment-order copies of the expert weights (``ops.pack_expert_weights``): steps whose expert
+        tiles have at most 64 rows (decode) stream those; larger steps keep reading the ``[E, N, K]`` tensors.
+        Costs a second copy of the expert weights in HBM; call again after the weights change."""
+        self.packed = [(ops.pack_expert_weights(l["gate_up"]), ops.pack_expert_weights(l["down"])) for l in self.layers]
+
     def nbytes(self) -> int:
         n = self.embed.numel() + self.lm_head.numel() + self.final_norm.numel()
         for l in self.layers:
@@ -115,6 +123,7 @@ class DecoderWeights:
         c.cfg = self.cfg
         c.embed, c.lm_head, c.final_norm = self.embed.cpu(), self.lm_head.cpu(), self.final_norm.cpu()
         c.layers = [{k: v.cpu() for k, v in l.items()} for l in self.layers]
+        c.packed = None
         return c
 
 
@@ -345,10 +354,16 @@ class Qwen3MoeDecoder:
             if routing_log is not None:  # debugging / tests only (allocates; not for graph capture)
                 routing_log.append(b.topk_idx.clone())
             r = ops.moe_route(b.topk_idx, E, bm=b.bm, buffers=b.route_ints)
-            gu = lw["gate_up"]
-            ops.moe_gemm(b.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=b.topk_w,
-                         row_scale_idx=r.sorted_flat, out=b.hw)
-            ops.moe_gemm(b.hw, lw["down"], r, out=b.eo)
+            if w.packed is not None and r.bm <= 64:
+                pgu, pdn = w.packed[li]
+                ops.moe_gemm_packed(b.h, pgu.rows(0, I), r, w2=pgu.rows(I, 2 * I), row_src=r.sorted_token,
+                                    row_scale=b.topk_w, row_scale_idx=r.sorted_flat, out=b.hw)
+                ops.moe_gemm_packed(b.hw, pdn, r, out=b.eo)
+            else:
+                gu = lw["gate_up"]
+                ops.moe_gemm(b.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=b.topk_w,
+                             row_scale_idx=r.sorted_flat, out=b.hw)
+                ops.moe_gemm(b.hw, lw["down"], r, out=b.eo)
             nxt = w.layers[li + 1]["in_norm"] if li + 1 < cfg.num_layers else w.final_norm
             # x <- x + sum_slots(eo) ; h <- next norm(x)
             ops.moe_gather(b.eo, r.scatter_index, residual=b.x, out=b.x, norm_weight=nxt, norm_out=b.h,

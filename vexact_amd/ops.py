@@ -631,6 +631,65 @@ def moe_gemm(
     return c
 
 
+class PackedExpertWeights:
+    """Fragment-order copy of ``[E, N, K]`` expert weights (``vx_pack_weights``) for the weight-streaming
+    grouped GEMM at decode sizes. ``rows(a, b)`` names rows ``[a, b)`` of every expert (``a`` a multiple of 16)."""
+
+    __slots__ = ("data", "E", "N", "K", "kchunks", "row0", "rows_n")
+
+    def rows(self, a: int, b: int) -> "PackedExpertWeights":
+        assert a % 16 == 0 and 0 <= a < b <= self.rows_n
+        v = PackedExpertWeights()
+        v.data, v.E, v.N, v.K, v.kchunks = self.data, self.E, self.N, self.K, self.kchunks
+        v.row0, v.rows_n = self.row0 + a, b - a
+        return v
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr() + (self.row0 // 16) * self.kchunks * 512 * 2
+
+    @property
+    def gstride(self) -> int:
+        return ((self.N + 15) // 16) * self.kchunks * 512
+
+
+def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
+    """Pack ``w [E, N, K]`` (bf16, K contiguous, any row / expert pitch) into fragment order."""
+    _need_gpu("w", w)
+    assert w.dim() == 3 and w.dtype == torch.bfloat16 and w.stride(2) == 1
+    E, N, K = w.shape
+    lib = _lib.load()
+    pk = PackedExpertWeights()
+    pk.E, pk.N, pk.K, pk.kchunks, pk.row0, pk.rows_n = E, N, K, lib.vx_packed_kchunks(K), 0, N
+    pk.data = torch.empty(E * pk.gstride, dtype=torch.bfloat16, device=w.device)
+    _lib.check(lib.vx_pack_weights(w.data_ptr(), w.stride(1), w.stride(0), E, N, K, pk.data.data_ptr(), _stream()),
+               "vx_pack_weights")
+    return pk
+
+
+def moe_gemm_packed(
+    x: torch.Tensor, w: PackedExpertWeights, routing: MoeRouting, *, w2: Optional[PackedExpertWeights] = None,
+    row_src: Optional[torch.Tensor] = None, row_scale: Optional[torch.Tensor] = None,
+    row_scale_idx: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``moe_gemm`` on packed weights (tile tables of 16 / 32 / 64 rows); same bits."""
+    n_rows = routing.T * routing.k
+    assert x.dtype == torch.bfloat16 and x.stride(1) == 1 and routing.bm in (16, 32, 64)
+    if w2 is not None:
+        assert w2.data is w.data and w2.rows_n == w.rows_n and row_scale is not None
+    N = w.rows_n
+    c = out if out is not None else torch.empty((n_rows, N), dtype=torch.bfloat16, device=x.device)
+    _lib.check(
+        _lib.load().vx_moe_gemm_packed(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w2.data_ptr() if w2 is not None else None, w.gstride,
+            c.data_ptr(), c.stride(0), N, w.K, routing.tile_group.data_ptr(), routing.tile_row0.data_ptr(),
+            routing.tile_rows.data_ptr(), routing.max_tiles, routing.bm, _ptr(row_src), _ptr(row_scale),
+            _ptr(row_scale_idx), 1 if w2 is not None else 0, _stream(),
+        ),
+        "vx_moe_gemm_packed",
+    )
+    return c
+
+
 def moe_gemm_nn(
     a: torch.Tensor, w: torch.Tensor, routing: MoeRouting, *, a_src: Optional[torch.Tensor] = None,
     a2: Optional[torch.Tensor] = None, w2: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
