@@ -324,7 +324,7 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(dom)
+            traffic = json.load(open(tpath)).get(dom if w.packed is not None else dom + "_unpacked")
         except Exception:
             traffic = None
     kernels[dom]["in_graph_avg_us"] = round(avg_in_graph * 1e6, 1)

@@ -348,6 +348,18 @@ def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
         y1 = gpu(x[:, 7:8].cuda())
         one = gpu.experts(x[0, :5].cuda(), expert_idx=3)
     assert_bitwise(y1, y[:, 7:8], "token 7 alone vs in the batch")
+    # fragment-order copies for decode: same bits; dropped once a parameter is written in place
+    gpu.experts.pack_for_decode()
+    with torch.no_grad(), set_batch_invariant_mode(True):
+        yp = gpu(x.cuda())
+        assert gpu.experts._packed is not None
+        assert_bitwise(yp, y, "packed expert weights vs parameters")
+        gpu.experts.down_proj.mul_(2.0)
+        y2 = gpu(x.cuda())
+        assert gpu.experts._packed is None, "stale packed copies must be dropped"
+        gpu.experts.down_proj.mul_(0.5)
+        assert_bitwise(gpu(x.cuda()), y, "parameters restored")
+    assert not torch.equal(y2, y)
     cpu = blk.to("cpu")
     logits = matmul_ref(x[0], cpu.gate.weight.detach().t())
     w, idx = OM.router_ref(logits, 4)

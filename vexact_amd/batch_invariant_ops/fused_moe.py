@@ -91,10 +91,13 @@ def fused_moe_forward(
     fc1_2_weight: Optional[torch.Tensor],
     fc2_weight: torch.Tensor,
     fc1_1_2_weight: Optional[torch.Tensor] = None,
+    packed_weights: Optional[tuple] = None,
 ) -> torch.Tensor:
     """``hidden_states [T,H]``, ``routing_weights/selected_experts [T,k]``; expert weights either as
     ``fc1_1_weight`` (gate) + ``fc1_2_weight`` (up), each ``[E,I,H]``, or fused ``fc1_1_2_weight [E,2I,H]``
-    (gate rows first); ``fc2_weight [E,H,I]``. Returns ``[T,H]`` bf16."""
+    (gate rows first); ``fc2_weight [E,H,I]``. Returns ``[T,H]`` bf16. ``packed_weights`` (not in the
+    reference; inference only): fragment-order copies of the same weights, ``(ops.pack_expert_weights(
+    fc1_1_2_weight), ops.pack_expert_weights(fc2_weight))``, streamed instead at decode sizes."""
     routing_weights = routing_weights.bfloat16()
     hidden_states = hidden_states.bfloat16()
     gate_w, up_w = _split_weights(fc1_1_weight, fc1_2_weight, fc1_1_2_weight)
@@ -110,7 +113,7 @@ def fused_moe_forward(
     x = hidden_states.reshape(-1, shape[-1])
     out = ops.fused_moe(
         x, routing_weights.reshape(x.shape[0], -1), selected_experts.reshape(x.shape[0], -1), gate_w, up_w, down_w,
-        num_experts,
+        num_experts, packed=packed_weights,
     )
     return out.reshape(shape)
 

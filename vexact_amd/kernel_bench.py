@@ -104,6 +104,14 @@ def main() -> None:
                                               row_scale=w, row_scale_idx=r.sorted_flat, out=hw)),
                U * 2 * I * H * 2 + B * H * 2 + B * k * I * 2 + B * k * 6)
         report("moe down", timeit(lambda li: ops.moe_gemm(hw, dn[li], r, out=eo)), U * H * I * 2 + B * k * I * 2 + B * k * H * 2)
+        pgu = [ops.pack_expert_weights(t) for t in gu]  # fragment-order copies, as the decoder streams them
+        pdn = [ops.pack_expert_weights(t) for t in dn]
+        report(f"moe gate/up, packed weights",
+               timeit(lambda li: ops.moe_gemm_packed(x, pgu[li].rows(0, I), r, w2=pgu[li].rows(I, 2 * I), row_src=r.sorted_token,
+                                                     row_scale=w, row_scale_idx=r.sorted_flat, out=hw)),
+               U * 2 * I * H * 2 + B * H * 2 + B * k * I * 2 + B * k * 6)
+        report("moe down, packed weights", timeit(lambda li: ops.moe_gemm_packed(hw, pdn[li], r, out=eo)),
+               U * H * I * 2 + B * k * I * 2 + B * k * H * 2)
         report("moe route", timeit(lambda li: ops.moe_route(idx, E, bm=32)), B * k * 16)
         report("moe gather + residual", timeit(lambda li: ops.moe_gather(eo, r.scatter_index, residual=x, out=y)),
                B * k * H * 2 + 2 * B * H * 2)

@@ -36,6 +36,21 @@ class Qwen3MoeExperts(nn.Module):
         self.gate_up_proj = nn.Parameter(torch.empty(self.num_experts, 2 * self.intermediate_size, self.hidden_dim))
         self.down_proj = nn.Parameter(torch.empty(self.num_experts, self.hidden_dim, self.intermediate_size))
 
+        self._packed = None  # (packed gate_up, packed down, (data_ptr, version) of both parameters)
+
+    def _weights_key(self):
+        return (self.gate_up_proj.data_ptr(), self.gate_up_proj._version, self.down_proj.data_ptr(), self.down_proj._version)
+
+    def pack_for_decode(self) -> None:
+        """Keep fragment-order copies of both parameters for decode-sized steps (a second copy of the
+        expert weights in HBM). They are dropped, and the parameters read again, once a parameter has
+        been written in place (weight synchronisation) until this is called again."""
+        if self.intermediate_size % 16 != 0 or self.gate_up_proj.dtype != torch.bfloat16:
+            raise ValueError("packed expert weights need bf16 parameters and an intermediate size that is a multiple of 16")
+        with torch.no_grad():
+            self._packed = (ops.pack_expert_weights(self.gate_up_proj.detach()),
+                            ops.pack_expert_weights(self.down_proj.detach()), self._weights_key())
+
     def forward(self, hidden_states: torch.Tensor, expert_idx: Optional[int] = None,
                 routing_weights: Optional[torch.Tensor] = None, selected_experts: Optional[torch.Tensor] = None):
         if expert_idx is not None:  # one expert as a dense SwiGLU MLP
@@ -46,10 +61,16 @@ class Qwen3MoeExperts(nn.Module):
         assert routing_weights is not None and selected_experts is not None, (
             "routing_weights and selected_experts must be provided when expert_idx is None"
         )
+        packed = None
+        if self._packed is not None:
+            if self._packed[2] == self._weights_key():
+                packed = self._packed[:2]
+            else:
+                self._packed = None  # stale: the parameters were written since
         return fused_moe_forward(
             num_experts=self.num_experts, routing_weights=routing_weights, selected_experts=selected_experts,
             hidden_states=hidden_states, fc1_1_weight=None, fc1_2_weight=None, fc2_weight=self.down_proj,
-            fc1_1_2_weight=self.gate_up_proj,
+            fc1_1_2_weight=self.gate_up_proj, packed_weights=packed,
         )
 
 

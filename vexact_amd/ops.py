@@ -814,10 +814,13 @@ def fused_moe(
     num_experts: int,
     residual: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
+    packed: Optional[tuple] = None,
 ) -> torch.Tensor:
     """Router outputs -> expert SwiGLU MLPs -> slot-ordered combine, four launches:
     routing integers, gate/up grouped GEMM with gather-on-load and fused SiLU*up*weight,
-    down grouped GEMM, fp32 slot-order sum."""
+    down grouped GEMM, fp32 slot-order sum. ``packed`` = (``pack_expert_weights`` of the stacked
+    ``[E, 2I, H]`` gate/up weight, of ``down_w``): read instead of the tensors when the step's expert
+    tiles have at most 64 rows (same bits)."""
     T, H = hidden_states.shape
     k = selected_experts.shape[1]
     x = hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous()
@@ -825,8 +828,15 @@ def fused_moe(
     H_, I_ = gate_w.shape[-1], down_w.shape[-1]
     r = moe_route(selected_experts, num_experts,
                   bm=moe_tile_rows(selected_experts.shape[0], wide_ok=(H_ % 64 == 0 and I_ % 64 == 0)))
-    hw = moe_gemm(x, gate_w, r, w2=up_w, row_src=r.sorted_token, row_scale=rw, row_scale_idx=r.sorted_flat)
-    o = moe_gemm(hw, down_w, r)
+    if packed is not None and r.bm <= 64:
+        pgu, pdn = packed
+        assert pgu.rows_n == 2 * I_ and pgu.K == H_ and pdn.rows_n == down_w.shape[1] and pdn.K == I_
+        hw = moe_gemm_packed(x, pgu.rows(0, I_), r, w2=pgu.rows(I_, 2 * I_), row_src=r.sorted_token, row_scale=rw,
+                             row_scale_idx=r.sorted_flat)
+        o = moe_gemm_packed(hw, pdn, r)
+    else:
+        hw = moe_gemm(x, gate_w, r, w2=up_w, row_src=r.sorted_token, row_scale=rw, row_scale_idx=r.sorted_flat)
+        o = moe_gemm(hw, down_w, r)
     return moe_gather(o, r.scatter_index, residual=residual, out=out)
 
 
