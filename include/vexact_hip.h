@@ -252,6 +252,15 @@ int vx_moe_gather_norm(const void* x, const int* index, const void* residual, vo
                        int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
                        int64_t ldh, float eps, int mode, hipStream_t stream);
 
+/* vx_moe_gather_norm with a cache prefetch riding along: extra workgroups read `prefetch_bytes` (rounded down
+ * to 16) from `prefetch` (16-byte aligned, readable) and discard them while the combine runs and leaves HBM
+ * idle - e.g. the weights of the projection that follows, which it would otherwise read cold. Changes no
+ * result; ignored on layouts the vector kernel cannot take. No counterpart in the reference. */
+int vx_moe_gather_norm_prefetch(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                                int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
+                                int64_t ldh, float eps, int mode, const void* prefetch, int64_t prefetch_bytes,
+                                hipStream_t stream);
+
 /* ---- decoder-layer glue ---------------------------------------------------------------- */
 
 /* Per-head RMSNorm (mode 1 form) of q and k, bf16 rotary embedding from cos/sin tables

@@ -226,6 +226,16 @@ def test_gather_with_fused_norm_equals_separate_kernels():
             ops.moe_gather(x, idx, residual=res, out=y, norm_weight=w, norm_out=h, eps=1e-6, hf_two_rounding=two)
             assert_bitwise(y, y_ref, "fused gather output")
             assert_bitwise(h, h_ref, "fused norm output")
+            # a cache prefetch riding along (spare workgroups read and discard it) changes nothing; sizes that
+            # are not a multiple of 16 bytes and sizes beyond 1024 workgroups' first pass are fine
+            for n in (1, 8 * 1000 + 3, 3 * 1024 * 1024 + 5):
+                pf = torch.full((n,), 7, dtype=torch.bfloat16, device="cuda")
+                y2, h2 = torch.empty_like(y_ref), torch.empty_like(y_ref)
+                ops.moe_gather(x, idx, residual=res, out=y2, norm_weight=w, norm_out=h2, eps=1e-6, hf_two_rounding=two,
+                               prefetch=pf)
+                assert_bitwise(y2, y_ref, "gather output with a prefetch riding along")
+                assert_bitwise(h2, h_ref, "norm output with a prefetch riding along")
+                assert bool((pf == 7).all()), "prefetched memory must stay untouched"
         # in place over the residual
         r2 = res.clone()
         ops.moe_gather(x, idx, residual=r2, out=r2)

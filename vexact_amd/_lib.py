@@ -58,6 +58,7 @@ PROTOTYPES = {
     "vx_moe_scatter": (_I, [_P, _P, _P, _L, _I, _L, _L, _L, _P]),
     "vx_moe_gather": (_I, [_P, _P, _P, _P, _L, _I, _L, _L, _L, _L, _P]),
     "vx_moe_gather_norm": (_I, [_P, _P, _P, _P, _L, _I, _L, _L, _L, _L, _P, _P, _L, _F, _I, _P]),
+    "vx_moe_gather_norm_prefetch": (_I, [_P, _P, _P, _P, _L, _I, _L, _L, _L, _L, _P, _P, _L, _F, _I, _P, _L, _P]),
     "vx_qk_norm_rope_store": (
         _I,
         [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _F, _L, _I, _L, _L, _L, _P],

@@ -407,10 +407,24 @@ __global__ __launch_bounds__(256) void moe_gather_vec_kernel(const bf16_t* __res
                                                              const bf16_t* res, bf16_t* y, int k, int H,
                                                              int64_t ldx, int64_t ldr, int64_t ldy,
                                                              const bf16_t* __restrict__ nw, bf16_t* h,
-                                                             int64_t ldh, float eps, int mode) {
+                                                             int64_t ldh, float eps, int mode, int T,
+                                                             const uint4* __restrict__ pf, int64_t pf16) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const int tid = threadIdx.x;
+  if (t >= T) {
+    // Workgroups past the tokens read pf16 16-byte pieces and discard them: this kernel leaves most of
+    // the memory system idle, and the weights that the next kernel needs cold arrive in the caches
+    // meanwhile. The store below never happens; it keeps the loads alive.
+    uint32_t acc = 0;
+    const int64_t stride = (int64_t)(gridDim.x - T) * 256;
+    for (int64_t i = (t - T) * 256 + tid; i < pf16; i += stride) {
+      const uint4 v = pf[i];
+      acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9e3779b9u && pf16 < 0) y[0] = 0;
+    return;
+  }
   float o[MAXV][4];
   float ss = 0.f;
 #pragma unroll
@@ -742,10 +756,14 @@ int vx_moe_scatter(const void* x, void* out, const int* index, int64_t T, int k,
 
 // y = gather-sum (+ residual); when norm_weight and h are given, also h = RMSNorm(y) (mode as in
 // vx_rms_norm). The fused norm needs H % 4 == 0, H <= 8192 and 8-byte aligned rows.
-int vx_moe_gather_norm(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
-                       int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
-                       int64_t ldh, float eps, int mode, hipStream_t stream) {
+// prefetch / prefetch_bytes (optional, vector path only): memory that extra workgroups read and discard
+// while the combine runs, e.g. the weights of the projection that follows.
+int vx_moe_gather_norm_prefetch(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                                int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
+                                int64_t ldh, float eps, int mode, const void* prefetch, int64_t prefetch_bytes,
+                                hipStream_t stream) {
   if (!x || !y || !index || T < 0 || k <= 0 || H <= 0 || H > 0x7fffffff) return VX_ERR_ARG;
+  if (prefetch_bytes < 0 || (prefetch && ((uintptr_t)prefetch % 16) != 0)) return VX_ERR_ARG;
   if ((norm_weight == nullptr) != (h == nullptr)) return VX_ERR_ARG;
   if (mode != 0 && mode != 1) return VX_ERR_ARG;
   if (T == 0) return VX_OK;
@@ -759,16 +777,26 @@ int vx_moe_gather_norm(const void* x, const int* index, const void* residual, vo
                                                        (bf16_t*)y, k, (int)H, ldx, ldr, ldy);
     return launch_status();
   }
+  const int64_t pf16 = prefetch ? prefetch_bytes / 16 : 0;
+  const int64_t pfb = pf16 > 0 ? (pf16 + 1023) / 1024 : 0;  // four pieces per thread, at most 1024 workgroups
+  const unsigned grid = (unsigned)(T + (pfb > 1024 ? 1024 : pfb));
 #define VX_GV(MV)                                                                                     \
-  moe_gather_vec_kernel<MV><<<(unsigned)T, 256, 0, stream>>>(                                         \
+  moe_gather_vec_kernel<MV><<<grid, 256, 0, stream>>>(                                                \
       (const bf16_t*)x, index, (const bf16_t*)residual, (bf16_t*)y, k, (int)H, ldx, ldr, ldy,         \
-      (const bf16_t*)norm_weight, (bf16_t*)h, ldh, eps, mode)
+      (const bf16_t*)norm_weight, (bf16_t*)h, ldh, eps, mode, (int)T, (const uint4*)prefetch, pf16)
   if (H <= 1024) VX_GV(1);
   else if (H <= 2048) VX_GV(2);
   else if (H <= 4096) VX_GV(4);
   else VX_GV(8);
 #undef VX_GV
   return launch_status();
+}
+
+int vx_moe_gather_norm(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,
+                       int64_t H, int64_t ldx, int64_t ldr, int64_t ldy, const void* norm_weight, void* h,
+                       int64_t ldh, float eps, int mode, hipStream_t stream) {
+  return vx_moe_gather_norm_prefetch(x, index, residual, y, T, k, H, ldx, ldr, ldy, norm_weight, h, ldh, eps, mode,
+                                     nullptr, 0, stream);
 }
 
 int vx_moe_gather(const void* x, const int* index, const void* residual, void* y, int64_t T, int k,

@@ -323,6 +323,7 @@ class Qwen3MoeDecoder:
                             for _ in range(cfg.num_layers)]
         self.buffers: dict[tuple[int, int], StepBuffers] = {}
         self.graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
+        self.prefetch_next_qkv = True  # see forward(): a cache hint, never a result
 
     def bucket(self, num_tokens: int, num_seqs: int) -> StepBuffers:
         key = (num_tokens, num_seqs)
@@ -366,8 +367,10 @@ class Qwen3MoeDecoder:
                 ops.moe_gemm(b.hw, lw["down"], r, out=b.eo)
             nxt = w.layers[li + 1]["in_norm"] if li + 1 < cfg.num_layers else w.final_norm
             # x <- x + sum_slots(eo) ; h <- next norm(x)
+            # decode-sized steps read the next layer's qkv weights cold: spare workgroups of the combine fetch them
+            pf = w.layers[li + 1]["qkv"] if (self.prefetch_next_qkv and li + 1 < cfg.num_layers and b.num_tokens <= 512) else None
             ops.moe_gather(b.eo, r.scatter_index, residual=b.x, out=b.x, norm_weight=nxt, norm_out=b.h,
-                           eps=cfg.rms_eps, hf_two_rounding=True)
+                           eps=cfg.rms_eps, hf_two_rounding=True, prefetch=pf)
 
     def _router(self, b: StepBuffers) -> None:
         from . import _lib

@@ -780,9 +780,11 @@ def moe_scatter(x: torch.Tensor, index: torch.Tensor, out_dtype=None) -> torch.T
 
 def moe_gather(x: torch.Tensor, index: torch.Tensor, out_dtype=None, residual: Optional[torch.Tensor] = None,
                out: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None,
-               norm_out: Optional[torch.Tensor] = None, eps: float = 1e-6, hf_two_rounding: bool = True) -> torch.Tensor:
+               norm_out: Optional[torch.Tensor] = None, eps: float = 1e-6, hf_two_rounding: bool = True,
+               prefetch: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``y[t] = sum_i x[index[t, i]]`` (fp32, slot order) ``(+ residual)``; with ``norm_weight`` and
-    ``norm_out`` also writes ``norm_out = RMSNorm(y)`` in the same launch."""
+    ``norm_out`` also writes ``norm_out = RMSNorm(y)`` in the same launch. ``prefetch``: a contiguous tensor
+    (the next projection's weights) that spare workgroups read and discard meanwhile; changes no result."""
     assert x.is_cuda and index.is_cuda
     M, topk = index.shape
     assert x.shape[0] == M * topk
@@ -794,11 +796,16 @@ def moe_gather(x: torch.Tensor, index: torch.Tensor, out_dtype=None, residual: O
     xs = x if x.stride(1) == 1 else x.contiguous()
     y = out if out is not None else torch.empty(M, N, dtype=x.dtype, device=x.device)
     assert (norm_weight is None) == (norm_out is None)
+    pf_bytes = 0
+    if prefetch is not None:
+        assert prefetch.is_contiguous() and prefetch.device == x.device
+        pf_bytes = prefetch.numel() * prefetch.element_size()
     _lib.check(
-        _lib.load().vx_moe_gather_norm(
+        _lib.load().vx_moe_gather_norm_prefetch(
             xs.data_ptr(), idx.data_ptr(), _ptr(residual), y.data_ptr(), M, topk, N, xs.stride(0),
             residual.stride(0) if residual is not None else 0, y.stride(0), _ptr(norm_weight), _ptr(norm_out),
-            norm_out.stride(0) if norm_out is not None else 0, float(eps), 1 if hf_two_rounding else 0, _stream()),
+            norm_out.stride(0) if norm_out is not None else 0, float(eps), 1 if hf_two_rounding else 0,
+            _ptr(prefetch), pf_bytes, _stream()),
         "vx_moe_gather_norm",
     )
     return y
