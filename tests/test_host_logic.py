@@ -248,3 +248,15 @@ def test_qwen3_moe_patch_points():
         moe_block_forward(blk, torch.zeros(1, 2, 64))
     with pytest.raises(ValueError, match="silu"):
         Qwen3MoeExperts(types.SimpleNamespace(num_experts=2, hidden_size=8, moe_intermediate_size=8, hidden_act="gelu"))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # every pipeline stage runs on one MI355X here: asking for more must say so and exit, before any GPU work
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 2
+    assert "exactly one GPU" in res.stderr and res.stdout.strip() == ""
