@@ -21,10 +21,50 @@ def rotate_half(x):
     return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
 
 
+def rope_tables_ref(head_dim: int, rope_theta: float, max_positions: int):
+    """cos / sin ``[max_positions, D]`` in bf16 from ``rope_theta`` alone: ``inv_freq = theta^(-2i/D)``
+    (fp32), ``angle = position * inv_freq`` (one fp32 product), the ``D/2`` angles repeated over both
+    halves, cos / sin in fp32, then cast: HuggingFace's default rotary embedding for bf16 activations,
+    the un-overridden glue of the layer the reference patches
+    (vexact/models/qwen3_moe/modeling_qwen3_moe.py:119-145 runs inside that layer)."""
+    inv_freq = 1.0 / (rope_theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    angle = torch.arange(max_positions, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    emb = torch.cat((angle, angle), dim=-1)
+    return _bf(emb.cos()), _bf(emb.sin())
+
+
 def rope_ref(x, cos, sin):
     """``x * cos + rotate_half(x) * sin`` in bf16 tensor ops; ``x [T,H,D]``, ``cos/sin [T,D]``."""
     c, s = cos.unsqueeze(1), sin.unsqueeze(1)
     return _bf(_bf(x.float() * c.float()).float() + _bf(rotate_half(x).float() * s.float()).float())
+
+
+def embedding_ref(table, ids):
+    """Row gather ``table[ids]``."""
+    return table[torch.as_tensor(ids).long()]
+
+
+def qk_norm_rope_store_ref(qkv, q_norm_w, k_norm_w, cos_t, sin_t, positions, slot_mapping, k_cache, v_cache,
+                           num_heads: int, num_kv_heads: int, head_dim: int, eps: float = 1e-6):
+    """What sits between the q/k/v projection and attention in the patched layer: split the fused
+    projection ``[T, (Hq+2Hkv) D]``, per-head RMSNorm of q and k (HuggingFace's two-rounding form, each with
+    its OWN weight), rotary embedding at ``positions``, and the cache write of k and v at
+    ``slot_mapping`` (vexact/batch_invariant_ops/triton_invariant_attention.py:1047-1054 with
+    vexact/batch_invariant_ops/kv_cache_context.py:294-314). Caches are written in place (``None``: no
+    write); returns (q, k) after the rotary embedding."""
+    T = qkv.shape[0]
+    Hq, Hkv, D = num_heads, num_kv_heads, head_dim
+    q = qkv[:, : Hq * D].reshape(T, Hq, D)
+    k = qkv[:, Hq * D : (Hq + Hkv) * D].reshape(T, Hkv, D)
+    v = qkv[:, (Hq + Hkv) * D :].reshape(T, Hkv, D)
+    q = hf_rms_norm_ref(q, q_norm_w, eps)
+    k = hf_rms_norm_ref(k, k_norm_w, eps)
+    pos = torch.as_tensor(positions).long()
+    cos, sin = cos_t[pos], sin_t[pos]
+    q, k = rope_ref(q, cos, sin), rope_ref(k, cos, sin)
+    if k_cache is not None:
+        store_kvcache_ref(k, v.contiguous(), k_cache, v_cache, slot_mapping)
+    return q, k
 
 
 def layer_ref(cfg, lw, x, positions, meta, k_cache, v_cache, cos_t, sin_t, forced_idx=None, report=None):
@@ -38,14 +78,8 @@ def layer_ref(cfg, lw, x, positions, meta, k_cache, v_cache, cos_t, sin_t, force
     Hq, Hkv, D, I = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, cfg.moe_intermediate
     h = hf_rms_norm_ref(x, lw["in_norm"], cfg.rms_eps)
     qkv = matmul_ref(h, lw["qkv"].t())
-    q = qkv[:, : Hq * D].reshape(T, Hq, D)
-    k = qkv[:, Hq * D : (Hq + Hkv) * D].reshape(T, Hkv, D)
-    v = qkv[:, (Hq + Hkv) * D :].reshape(T, Hkv, D)
-    q = hf_rms_norm_ref(q, lw["q_norm"], cfg.rms_eps)
-    k = hf_rms_norm_ref(k, lw["k_norm"], cfg.rms_eps)
-    cos, sin = cos_t[positions], sin_t[positions]
-    q, k = rope_ref(q, cos, sin), rope_ref(k, cos, sin)
-    store_kvcache_ref(k, v.contiguous(), k_cache, v_cache, meta["slot_mapping"])
+    q, _ = qk_norm_rope_store_ref(qkv, lw["q_norm"], lw["k_norm"], cos_t, sin_t, positions, meta["slot_mapping"],
+                                  k_cache, v_cache, Hq, Hkv, D, cfg.rms_eps)
     outs = []
     qsl, lens, bt = meta["query_start_loc"], meta["context_lens"], meta["block_tables"]
     for s in range(len(lens)):
@@ -81,7 +115,7 @@ def decoder_step_ref(cfg, weights, input_ids, meta, key_cache, value_cache, cos_
                      report=None):
     """Full step: embedding, all layers, final norm, lm_head on each sequence's last token, greedy
     token and its fp32 logprob (vexact/inferencer/inferencer.py:391-449)."""
-    x = weights.embed[torch.as_tensor(input_ids).long()]
+    x = embedding_ref(weights.embed, input_ids)
     pos = torch.as_tensor(meta["positions"]).long()
     for li, lw in enumerate(weights.layers):
         forced = forced_routing[li] if forced_routing is not None else None

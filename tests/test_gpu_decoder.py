@@ -15,14 +15,13 @@ from vexact_amd.decoder import (  # noqa: E402
     DecoderWeights,
     Qwen3MoeDecoder,
     build_step_metadata,
-    rope_tables,
     tiny_config,
 )
 
 
 def _setup(num_seqs=5, seed=3, layers=2):
     cfg = tiny_config(num_layers=layers)
-    w = DecoderWeights(cfg, device="cuda", seed=seed, std=0.05)
+    w = DecoderWeights(cfg, device="cuda", seed=seed, std=0.05, norm_std=0.1)  # every norm weight differs from 1
     rng = np.random.default_rng(seed)
     prompt_lens = rng.integers(5, 300, size=num_seqs)
     prompts = [rng.integers(0, cfg.vocab_size, size=n) for n in prompt_lens]
@@ -71,7 +70,7 @@ def test_tiny_decoder_matches_cpu_oracle_and_is_batch_invariant():
 
     # CPU oracle on the same input bits, following the GPU's expert choice at near-ties
     wc = w.to_cpu()
-    cos, sin = rope_tables(cfg, "cpu")
+    cos, sin = OD.rope_tables_ref(cfg.head_dim, cfg.rope_theta, cfg.max_model_len)  # the oracle's own tables
     kc = [torch.zeros(t.shape, dtype=t.dtype) for t in dec.key_cache]
     vc = [torch.zeros(t.shape, dtype=t.dtype) for t in dec.value_cache]
     report = []

@@ -62,7 +62,9 @@ class DecoderWeights:
     expert gate/up projections as ``[E, 2I, H]`` (gate rows first), like the reference's
     ``Qwen3MoeExperts`` (vexact/models/qwen3_moe/modeling_qwen3_moe.py:42-67)."""
 
-    def __init__(self, cfg: DecoderConfig, device="cuda", seed: int = 5, std: float = 0.02, generator_device="cuda"):
+    def __init__(self, cfg: DecoderConfig, device="cuda", seed: int = 5, std: float = 0.02, generator_device="cuda",
+                 norm_std: float = 0.0):
+        """``norm_std``: spread of the RMSNorm weights around 1 (0 = exactly 1, a freshly initialised model)."""
         self.cfg = cfg
         g = torch.Generator(device=generator_device).manual_seed(seed)
         bf = torch.bfloat16
@@ -84,7 +86,13 @@ class DecoderWeights:
             return buf[..., : shape[-1]]
 
         H, D, E, I = cfg.hidden_size, cfg.head_dim, cfg.num_experts, cfg.moe_intermediate
-        ones = lambda n: torch.ones(n, dtype=bf, device=device)  # noqa: E731
+        def ones(n):
+            if norm_std == 0.0:
+                return torch.ones(n, dtype=bf, device=device)
+            t = torch.empty(n, dtype=torch.float32, device=generator_device)
+            t.normal_(1.0, norm_std, generator=g)
+            return t.to(bf).to(device)
+
         self.embed = rnd(cfg.vocab_size, H)
         self.lm_head = rnd(cfg.vocab_size, H)
         self.final_norm = ones(H)
