@@ -28,6 +28,16 @@ fused_moe_ref          k=1,w=1 => plain SwiGLU MLP; all tokens on one expert => 
                        fp64 brute force on tiny shapes; HF-eager form within bf16 tolerance
 prepare_gen_ctx_ref    hand-worked example; vectorised numpy twin
 BlockAllocatorRef      scan restatement of the reference allocator; hand-worked sequence
+rope_tables_ref        HuggingFace Qwen3MoeRotaryEmbedding bit for bit (three theta / head sizes, positions to
+                       40959); position 0 = identity, first pair turns by `position` radians
+rope_ref               HuggingFace apply_rotary_pos_emb bit for bit; pair lengths preserved
+qk_norm_rope_store_ref the HuggingFace attention module's own q_norm / k_norm (distinct non-unit weights) +
+                       apply_rotary_pos_emb bit for bit; cache rows by slot, slot -1 and unmapped rows untouched
+embedding_ref          torch indexing (library routine)
+layer_ref              HuggingFace Qwen3MoeDecoderLayer on the CPU (eager attention, eager experts, norm weights in
+                       [0.5, 1.5]): 0.8 % of the largest entry at worst (bound 2 %; swapped q/k norm weights: 4.3 %)
+decoder_step_ref       HuggingFace Qwen3MoeForCausalLM last-token logits, packed prefill through the paged cache and
+                       a decode step on top of it: logprob |d| <= 5e-2; a wrong rope_theta fails
 attention_backward_ref autograd through the fp32 eager attention; one visible key => dV = dO, dQ = dK = 0
 fused_moe_backward_ref autograd through an fp32 restatement of the expert MLPs
 sampler.philox4x32     Random123 known-answer vectors

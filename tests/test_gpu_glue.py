@@ -68,8 +68,8 @@ def test_qk_norm_rope_store_matches_oracle(D, Hq, Hkv, T, max_pos, theta, pos_dt
                            q, kc, vc, Hq, Hkv, D, 1e-6, k_out=k_out)
     torch.cuda.synchronize()
     q, k_out, kc, vc = q.cpu(), k_out.cpu(), kc.cpu().contiguous(), vc.cpu().contiguous()
-    # the kernel divides by sqrt where the oracle multiplies by rsqrt: at most one bf16 ulp on the normalised
-    # value, hence at most 2 on the sum of the two rotated products (measured below), never more
+    # the kernel divides by sqrt where the oracle multiplies by rsqrt: now and then one bf16 ulp on the normalised
+    # value, hence at most 2 on the sum of the two rotated products (measured: 1 or 2 elements of 10^6 differ)
     for name, got, want in (("q", q, q_ref), ("k", k_out, k_ref)):
         ulp = bf16_ulp_distance(got, want)
         absd = (got.float() - want.float()).abs()
@@ -77,7 +77,7 @@ def test_qk_norm_rope_store_matches_oracle(D, Hq, Hkv, T, max_pos, theta, pos_dt
         print(f"{name}: {float((ulp == 0).float().mean()):.4f} exact, {float((ulp <= 1).float().mean()):.4f} within 1 ulp, "
               f"worst {int(ulp.max())} ulp")
         assert bool(((ulp <= 2) | small).all()), f"{name}: beyond 2 bf16 ulp"
-        assert float((ulp == 0).float().mean()) >= 0.97, f"{name}: too few exact elements"
+        assert float((ulp == 0).float().mean()) >= 0.999, f"{name}: too few exact elements"
     # cache rows: the written K row is the kernel's own k output bit for bit, V is a plain copy, rows of slot -1
     # and rows no token maps to keep the marker
     flat_k, flat_v = kc.view(-1, Hkv, D), vc.view(-1, Hkv, D)
