@@ -67,6 +67,19 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
                 int64_t rows, int64_t n, int64_t x_stride, void* workspace, int64_t workspace_bytes,
                 hipStream_t stream);
 
+/* vx_logprobs for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): no workspace argument, no counterpart in the reference. The chunk partials live in a
+ * 1 MiB array inside the library's device image (VX_LOGPROBS_STATIC_BYTES; every GPU the library runs on holds
+ * it until the process ends), so rows * ceil(n / 4096) * 16 bytes must not exceed that: 256 rows of a
+ * 151936-entry vocabulary need 152 KiB. Larger problems return VX_ERR_WORKSPACE before anything is launched.
+ * Calls no hipMalloc / hipFree or other allocating routine; the first call on a device looks the array's address
+ * up once (make that call outside a capture). Same kernels and same bits as vx_logprobs. All calls on one GPU
+ * share the array: calls that overlap on one GPU (different streams, different threads) race; calls on one
+ * stream are ordered and safe. Nothing in the array has to be cleared between calls. */
+#define VX_LOGPROBS_STATIC_BYTES (1 << 20)
+int vx_logprobs_static(const void* logits, const int64_t* labels, float* out, int64_t* tokens_out, int dtype,
+                       int64_t rows, int64_t n, int64_t x_stride, hipStream_t stream);
+
 /* ---- dense GEMM ----------------------------------------------------------------------- */
 
 /* C[M,N] = X[M,K] * W[N,K]^T (+ bias[N]), bf16 in/out, fp32 accumulate, K ascending, no split-K.

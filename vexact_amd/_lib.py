@@ -22,6 +22,7 @@ PROTOTYPES = {
     "vx_log_softmax_workspace_bytes": (_L, [_L, _L]),
     "vx_log_softmax": (_I, [_P, _P, _I, _L, _L, _L, _L, _P, _L, _P]),
     "vx_logprobs": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _P, _L, _P]),
+    "vx_logprobs_static": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _P]),
     "vx_gemm_bf16_nt": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _P]),
     "vx_gemm_bf16_nt_variant": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _I, _P]),
     "vx_gemm_swiglu_bf16_nt": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _I, _P]),

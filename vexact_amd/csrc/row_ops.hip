@@ -7,6 +7,7 @@
 // wave-order pass finish the sum. The schedule never looks at the number of rows.
 #include "common.h"
 #include <math.h>
+#include <atomic>
 
 namespace vx {
 
@@ -329,6 +330,29 @@ __global__ __launch_bounds__(64) void logprob_final_kernel(
 
 using namespace vx;
 
+// ---------------------------------------------------------------------------------------
+// Chunk partials of vx_logprobs_static live in this array instead of a caller's workspace. The
+// name `scratch` is a host-side stand-in for the symbol: host code uses the per-device address
+// that hipGetSymbolAddress returns (every GPU holds its own copy at its own address).
+// ---------------------------------------------------------------------------------------
+constexpr int64_t kStaticScratchBytes = 1 << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return VX_ERR_LAUNCH;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return VX_ERR_LAUNCH;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing first calls store the same address
+  }
+  *out = p;
+  return VX_OK;
+}
+
 extern "C" {
 
 int vx_mean_dim(const void* in, void* out, int dtype, int64_t M, int64_t N, int64_t K, int64_t s0,
@@ -493,6 +517,19 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
     default: return VX_ERR_UNSUPPORTED;
   }
   return launch_status();
+}
+
+int vx_logprobs_static(const void* logits, const int64_t* labels, float* out, int64_t* tokens_out,
+                       int dtype, int64_t rows, int64_t n, int64_t x_stride, hipStream_t stream) {
+  if (rows < 0 || n <= 0) return VX_ERR_ARG;
+  // the size limit is checked before anything touches the device
+  if (vx_log_softmax_workspace_bytes(rows, n) > kStaticScratchBytes) return VX_ERR_WORKSPACE;
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != VX_OK) return rc;
+  // every partial the final kernel reads is written by the partial kernel of this call first, so
+  // nothing in the array has to start at zero
+  return vx_logprobs(logits, labels, out, tokens_out, dtype, rows, n, x_stride, ws, kStaticScratchBytes, stream);
 }
 
 }  // extern "C"
