@@ -9,9 +9,12 @@ step (256 tokens, 256 sequences, greedy token + fp32 logprob) is captured in a H
 replayed: warm-up W times, then exactly K timed replays.
 
 Prints one JSON line: whole-job tok/s, the roofline of the dominant kernel (MoE gate/up grouped
-GEMM, HBM bound) measured with HIP events in an eager pass, per-kernel GB/s of the other
-memory-bound kernels, the logprob bit drift between batch 256 and batch 1, and the CPU oracle timed
-on the host cores for a bounded sample (one decoder layer + lm_head at batch 256, scaled to 48 layers).
+GEMM, HBM bound) measured with HIP events, per-kernel GB/s of the other memory-bound kernels, the
+logprob bit drift between batch 256 and batch 1 for every request, an advancing decode loop (per-step host
+metadata + one host-to-device copy + graph replay + sampled tokens fed back) beside the replay figure, the
+reference's other configurations (op chain, decode attention, chunked prefill, fused MoE) and the prefill
+q/k/v GEMM against their HBM / MFMA rooflines, and the CPU oracle timed on the host cores for a bounded
+sample (one decoder layer + lm_head at batch 256, scaled to 48 layers).
 """
 
 from __future__ import annotations
@@ -40,7 +43,10 @@ def parse():
     ap.add_argument("--layers", type=int, default=48, help="fewer layers = a smoke run, flagged as such in the output")
     ap.add_argument("--min-prompt", type=int, default=256)
     ap.add_argument("--max-prompt", type=int, default=2048)
-    ap.add_argument("--drift-requests", type=int, default=8, help="requests re-run at batch 1 for the bit-drift check")
+    ap.add_argument("--drift-requests", type=int, default=256, help="requests re-run at batch 1 for the bit-drift check")
+    ap.add_argument("--loop-steps", type=int, default=20,
+                    help="steps of the advancing decode loop (host metadata + copy + replay + token feedback); 0 = skip")
+    ap.add_argument("--no-configs", action="store_true", help="skip the reference's other configurations (C1-C4, prefill GEMM)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-packed-experts", action="store_true",
                     help="decode reads the [E, N, K] expert tensors instead of their fragment-order copies")
@@ -142,7 +148,8 @@ def main():
     rng = np.random.default_rng(args.seed)
     prompt_lens = rng.integers(args.min_prompt, args.max_prompt + 1, size=B)
     prompts = [rng.integers(0, cfg.vocab_size, size=int(n)) for n in prompt_lens]
-    pages = [(int(n) + 1 + cfg.page_size - 1) // cfg.page_size for n in prompt_lens]
+    grow = 1 + max(0, args.loop_steps)  # room for the decode step and the advancing loop
+    pages = [(int(n) + grow + cfg.page_size - 1) // cfg.page_size for n in prompt_lens]
     pool = sum(pages) + 64
     perm = rng.permutation(pool)
     blocks, o = [], 0
@@ -221,6 +228,7 @@ def main():
     tok_graph = db.tokens.cpu().clone()
 
     # ---- logprob bit drift: the same requests at batch 1 (eager)
+    t0 = time.time()
     drift_bits, checked = 0, 0
     b1 = dec.bucket(1, 1)
     for i in range(min(args.drift_requests, B)):
@@ -233,6 +241,35 @@ def main():
         bb = lp_graph[r : r + 1].view(torch.int32)
         drift_bits += bin(int(a[0]) ^ int(bb[0])).count("1") + (0 if int(b1.tokens[0]) == int(tok_graph[r]) else 64)
         checked += 1
+    print(f"[bench] drift check of {checked} requests at batch 1: {time.time() - t0:.1f}s, {drift_bits} bits", file=sys.stderr, flush=True)
+
+    # ---- an advancing decode loop: what a serving step pays around the graph (inferencer.py:124-191, 193-349):
+    # native step metadata into the pinned staging buffer, ONE host-to-device copy, graph replay, sampled
+    # tokens back to the host (the scheduler appends them to the requests) and in as the next input ids,
+    # every context one token longer
+    loop = None
+    if args.loop_steps > 0:
+        lreqs = [dict(num_computed_tokens=ctx[i], tokens_this_step=1, block_ids=np.asarray(blocks[i], np.int32)) for i in range(B)]
+        toks = first_tokens.copy()
+        host_s = 0.0
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.loop_steps):
+            h0 = time.perf_counter()
+            db.load_requests(lreqs, toks, cfg.page_size)
+            host_s += time.perf_counter() - h0
+            graph.replay()
+            toks = db.tokens.cpu().numpy()  # waits for the step
+            h0 = time.perf_counter()
+            for r_ in lreqs:
+                r_["num_computed_tokens"] += 1
+            host_s += time.perf_counter() - h0
+        dt_loop = time.perf_counter() - t0
+        loop = {"decode_loop_tok_s": round(B * args.loop_steps / dt_loop, 1), "loop_steps": args.loop_steps,
+                "loop_ms_per_step": round(dt_loop / args.loop_steps * 1e3, 3),
+                "host_ms_per_step": round(host_s / args.loop_steps * 1e3, 3),
+                "what": "per step: vx_host_step_metadata into pinned staging + one H2D copy, graph replay, tokens D2H and "
+                        "fed back as the next input ids, contexts growing by one"}
 
     # ---- per-kernel timing with HIP events on the launch stream (eager pass over all layers)
     E, k, I, H = cfg.num_experts, cfg.top_k, cfg.moe_intermediate, cfg.hidden_size
@@ -359,9 +396,28 @@ def main():
         "kernels": kernels,
     }
 
+    if loop is not None:
+        out.update(loop)
+    if not args.no_configs:
+        out["configs"], out["roofline_mfma"] = other_configs()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, args.cpu_seconds)
     print(json.dumps(out), flush=True)
+
+
+def other_configs():
+    """The reference's other benchmark configurations at their own shapes, graph-replayed and timed with HIP
+    events (kernel_bench.py): C1 op chain at M = 1 / 7 / 64, C2 decode attention, C3 chunked prefill attention,
+    C4 fused MoE block at T = 1 / 64 / 256 / 4096, and the q/k/v projection of an 8192-token prefill chunk.
+    Each line carries its algorithmic bytes or flops and the fraction of the HBM / bf16 MFMA peak."""
+    import argparse as _ap
+
+    import kernel_bench
+
+    res = kernel_bench.run(_ap.Namespace(what=["configs", "mfma"], batch=256, layers=2, reps=3, kv_layout="head", page=16,
+                                         nograph=False), quiet=True)
+    mfma = [r for r in res if r["bound"] == "mfma"]
+    return res, mfma
 
 
 def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
@@ -371,13 +427,20 @@ def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
 
     from oracle import decoder as OD
     from oracle.row_ops import hf_rms_norm_ref, logprobs_ref, matmul_ref
-    from vexact_amd.decoder import rope_tables
-
+    # threads: the harness gives a one-GPU job 16 host cores (OMP_NUM_THREADS), whatever os.cpu_count() shows
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
     torch.set_num_threads(cores)
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     lw = {k_: v.cpu() for k_, v in w.layers[0].items()}
     kc, vc = dec.key_cache[0].cpu().contiguous(), dec.value_cache[0].cpu().contiguous()
-    cos, sin = rope_tables(cfg, "cpu")
+    cos, sin = OD.rope_tables_ref(cfg.head_dim, cfg.rope_theta, cfg.max_model_len)
     x = w.embed[torch.as_tensor(first_tokens).to(w.embed.device)].cpu()
     pos = torch.as_tensor(dmeta["positions"]).long()
     lm_head, fnorm = w.lm_head.cpu(), w.final_norm.cpu()
@@ -397,7 +460,8 @@ def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
         if time.perf_counter() - t_start > budget_s or n >= 5:
             break
     step = cfg.num_layers * t_layer / n + t_head / n
-    return {"value": round(B / step, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+    return {"value": round(B / step, 3), "unit": "tok/s", "cores": cores, "kind": "port", "cpu_model": model,
+            "host_cpus": os.cpu_count(),
             "sample": f"1 of {cfg.num_layers} decoder layers + lm_head at batch {B}, {n} repeats "
                       f"({t_layer / n:.2f}s per layer, {t_head / n:.2f}s head), scaled to {cfg.num_layers} layers"}
 

@@ -7,7 +7,7 @@ out, and the replay is timed with events. Prints time, algorithmic bytes (or flo
 fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
 to run under ``rocprofv3 --pmc``.
 
-    python -m vexact_amd.kernel_bench --what moe,attn,gemm,small,prefill,dense,train,sampler,copy
+    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,copy
 """
 
 from __future__ import annotations
@@ -19,14 +19,14 @@ import sys
 import numpy as np
 import torch
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from vexact_amd import _lib, ops  # noqa: E402
 
 HBM_PEAK = 8.0e12
 MFMA_PEAK = 2.5e15
 
 
-def main() -> None:
+def parse(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--what", default="moe,attn,gemm,small")
     ap.add_argument("--batch", type=int, default=256)
@@ -36,8 +36,14 @@ def main() -> None:
                     help="physical KV cache layout: [blocks, Hkv, page, D] (what the decoder allocates) or [blocks, page, Hkv, D]")
     ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
     ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
-    a = ap.parse_args()
+    return ap.parse_args(argv)
+
+
+def run(a, quiet: bool = False) -> list:
+    """Run the sections named in ``a.what``; returns one dict per reported line (name, us, bytes or flops,
+    achieved rate, fraction of the MI355X peak)."""
     dev = "cuda"
+    results = []
     B, NL = a.batch, a.layers
     H, I, E, k = 2048, 768, 128, 8
     g = torch.Generator(device=dev).manual_seed(0)
@@ -70,14 +76,19 @@ def main() -> None:
         return float(np.mean(ts))
 
     def report(name, t, nbytes=None, flops=None):
+        say = (lambda *x, **k: None) if quiet else print
         if t is None:
-            print(f"{name:34s} launched", flush=True)
+            say(f"{name:34s} launched", flush=True)
         elif flops is not None:
-            print(f"{name:34s} {t * 1e6:9.1f} us  {flops / t / 1e12:8.1f} TFLOP/s  ({flops / t / MFMA_PEAK * 100:5.1f}% of 2.5 PFLOP/s)", flush=True)
+            results.append({"name": name, "us": round(t * 1e6, 1), "flops": int(flops), "bound": "mfma",
+                            "TFLOPs": round(flops / t / 1e12, 1), "frac": round(flops / t / MFMA_PEAK, 4)})
+            say(f"{name:34s} {t * 1e6:9.1f} us  {flops / t / 1e12:8.1f} TFLOP/s  ({flops / t / MFMA_PEAK * 100:5.1f}% of 2.5 PFLOP/s)", flush=True)
         else:
-            print(f"{name:34s} {t * 1e6:9.1f} us  {nbytes / t / 1e9:8.1f} GB/s  ({nbytes / t / HBM_PEAK * 100:5.1f}% of 8 TB/s)  {nbytes / 1e6:.1f} MB", flush=True)
+            results.append({"name": name, "us": round(t * 1e6, 1), "bytes": int(nbytes), "bound": "hbm",
+                            "GBps": round(nbytes / t / 1e9, 1), "frac": round(nbytes / t / HBM_PEAK, 4)})
+            say(f"{name:34s} {t * 1e6:9.1f} us  {nbytes / t / 1e9:8.1f} GB/s  ({nbytes / t / HBM_PEAK * 100:5.1f}% of 8 TB/s)  {nbytes / 1e6:.1f} MB", flush=True)
 
-    what = a.what.split(",")
+    what = a.what.split(",") if isinstance(a.what, str) else list(a.what)
     if "sampler" in what:
         V = 151936
         lg = (torch.randn(B, V, generator=g, device=dev) * 2.5).to(torch.bfloat16)
@@ -259,8 +270,15 @@ def main() -> None:
         report(f"prefill attention {S} x {Lp} tokens",
                timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, bt, D**-0.5, Lp, out=out), n_layers=2),
                flops=4 * S * Hq * D * Lp * (Lp + 1) // 2)
-    if "prefill" in what:
-        # chunked prefill: 16 sequences, a 512-token chunk on a cached prefix of 0..8192 tokens, Hq=32, Hkv=8
+    if "mfma" in what:
+        # the q/k/v projection of an 8192-token prefill chunk at the model's own shape
+        M, N, K = 8192, 5120, 2048
+        w_, xx = rnd(N, K), rnd(M, K, std=1.0)
+        c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        report(f"prefill gemm qkv M={M} N={N} K={K}", timeit(lambda li: ops.gemm_nt(xx, w_, out=c), n_layers=2), flops=2 * M * N * K)
+        del w_, xx, c
+    if "prefill" in what or "configs" in what:
+        # C3, chunked prefill: 16 sequences, a 512-token chunk on a cached prefix of 0..8192 tokens, Hq=32, Hkv=8
         Hq, Hkv, D, page, S, C = 32, 8, 128, 16, 16, 512
         rng = np.random.default_rng(3)
         prefix = rng.integers(0, 8193, size=S)
@@ -281,7 +299,7 @@ def main() -> None:
         btd = torch.tensor(bt, device=dev)
         out = torch.empty(S * C, Hq, D, dtype=torch.bfloat16, device=dev)
         fl = 4 * Hq * D * int(sum(C * int(pf) + C * (C + 1) // 2 for pf in prefix))
-        report(f"chunked prefill attention 16 x 512 on prefixes (sum L={int(Ls.sum())})",
+        report(f"C3 chunked prefill attention 16 x 512 on prefixes (sum L={int(Ls.sum())})",
                timeit(lambda li: ops.paged_attention(q, kc, vc, cu, used, btd, D**-0.5, C, out=out), n_layers=2), flops=fl)
     if "small" in what:
         one = torch.zeros(64, dtype=torch.int32, device=dev)
@@ -324,6 +342,14 @@ def main() -> None:
             report(f"C1 log_softmax fp32 M={M}", timeit(lambda li: ops.log_softmax(lf), n_layers=2), 2 * M * V * 4)
             report(f"C1 rms_norm M={M}", timeit(lambda li: ops.rms_norm(x, wn, 1e-6, hf_two_rounding=True, out=hn), n_layers=2),
                    2 * M * H * 2 + 2 * H)
+
+            def chain(li):
+                ops.rms_norm(x, wn, 1e-6, hf_two_rounding=True, out=hn)
+                ops.gemm_nt(hn, wl, out=lg)
+                ops.log_softmax(lg.float())
+
+            report(f"C1 chain norm -> lm_head -> fp32 log_softmax M={M}", timeit(chain, n_layers=2),
+                   2 * (V * H + M * H + M * V) + 2 * M * V * 4 + 2 * M * H * 2 + 2 * H)
         del wl
         # C2: decode attention, 64 sequences, context 128..4096, Hq=16, Hkv=8, D=128, page 16
         Hq, Hkv, D, page, S = 16, 8, 128, 16, 64
@@ -361,12 +387,17 @@ def main() -> None:
             t = timeit(lambda li: ops.fused_moe(x, w, idx, gu[:, :I, :], gu[:, I:, :], dn, E, out=y), n_layers=2)
             report(f"C4 fused MoE T={T} ({U} experts)", t, U * 3 * H * I * 2 + 2 * T * H * 2 + T * k * 6)
             if T == 4096 and t is not None:
-                print(f"{'':34s} = {T * k * 6 * H * I / t / 1e12:.1f} TFLOP/s", flush=True)
+                report(f"C4 fused MoE T={T}, as flops", t, flops=T * k * 6 * H * I)
     if "copy" in what:
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
         report("copy 1 GiB", timeit(lambda li: dst.copy_(src), n_layers=2), 2 << 30)
+    return results
+
+
+def main() -> None:
+    run(parse())
 
 
 if __name__ == "__main__":
