@@ -120,35 +120,24 @@ def cpu_configs(seed):
     print(json.dumps({"cpu_configs": res}), flush=True)
 
 
-def main():
-    args = parse()
-    if args.cpu_configs:
-        cpu_configs(args.seed)
-        return
-    if args.gpus != 1:
-        print("bench.py: this build runs on exactly one GPU (all pipeline stages collapsed onto one MI355X); "
-              "--gpus must be 1", file=sys.stderr)
-        sys.exit(2)
+def build_workload(layers=48, batch=256, seed=5, min_prompt=256, max_prompt=2048, grow=1, packed=True, log=True):
+    """The headline workload: random-init weights, ``batch`` prompts of random ids prefilled with the library's own
+    kernels into a paged cache (page 16, block tables from a random permutation of the pool, room for ``grow``
+    more tokens per sequence), and the metadata of the decode step that follows."""
+    import types
+
     import torch
 
-    from vexact_amd import _build, _lib, ops
-    from vexact_amd.decoder import (DecoderWeights, Qwen3MoeDecoder, build_step_metadata, decode_bytes_per_step,
-                                    qwen3_30b_a3b)
+    from vexact_amd.decoder import DecoderWeights, Qwen3MoeDecoder, build_step_metadata, qwen3_30b_a3b
 
-    if not os.path.exists(_build.LIB_PATH):
-        _build.build()
-    _lib.load()
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda"
-    torch.cuda.set_device(0)
-
+    say = (lambda m: print(m, file=sys.stderr, flush=True)) if log else (lambda m: None)
     cfg = qwen3_30b_a3b()
-    cfg.num_layers = args.layers
-    B = args.batch
-    rng = np.random.default_rng(args.seed)
-    prompt_lens = rng.integers(args.min_prompt, args.max_prompt + 1, size=B)
+    cfg.num_layers = layers
+    B = batch
+    rng = np.random.default_rng(seed)
+    prompt_lens = rng.integers(min_prompt, max_prompt + 1, size=B)
     prompts = [rng.integers(0, cfg.vocab_size, size=int(n)) for n in prompt_lens]
-    grow = 1 + max(0, args.loop_steps)  # room for the decode step and the advancing loop
     pages = [(int(n) + grow + cfg.page_size - 1) // cfg.page_size for n in prompt_lens]
     pool = sum(pages) + 64
     perm = rng.permutation(pool)
@@ -159,12 +148,11 @@ def main():
     max_blocks = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
 
     t0 = time.time()
-    w = DecoderWeights(cfg, device=dev, seed=args.seed)
+    w = DecoderWeights(cfg, device=dev, seed=seed)
     dec = Qwen3MoeDecoder(cfg, w, num_cache_blocks=pool, device=dev)
     torch.cuda.synchronize()
-    print(f"[bench] weights {w.nbytes() / 1e9:.1f} GB, KV pool {pool} pages "
-          f"({2 * cfg.num_layers * dec.key_cache[0].numel() * 2 / 1e9:.1f} GB), init {time.time() - t0:.1f}s",
-          file=sys.stderr, flush=True)
+    say(f"[bench] weights {w.nbytes() / 1e9:.1f} GB, KV pool {pool} pages "
+        f"({2 * cfg.num_layers * dec.key_cache[0].numel() * 2 / 1e9:.1f} GB), init {time.time() - t0:.1f}s")
 
     # ---- prefill with the library's own kernels, several sequences per pass
     t0 = time.time()
@@ -183,15 +171,71 @@ def main():
         dec.step(pb, max_q)
         first_tokens[grp] = pb.tokens[: len(grp)].cpu().numpy()
     torch.cuda.synchronize()
-    print(f"[bench] prefill of {int(prompt_lens.sum())} tokens: {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+    say(f"[bench] prefill of {int(prompt_lens.sum())} tokens: {time.time() - t0:.1f}s")
     del dec.buffers[(PT, PB)]
     del pb
     torch.cuda.empty_cache()
 
     # ---- decode streams the expert weights from their fragment-order copies (made once per weight update)
-    if not args.no_packed_experts:
+    if packed:
         w.pack_experts()
         torch.cuda.synchronize()
+
+    ctx = [int(n) + 1 for n in prompt_lens]
+    reqs = [dict(num_computed_tokens=ctx[i], tokens_this_step=1, block_ids=blocks[i]) for i in range(B)]
+    dmeta = build_step_metadata(reqs, cfg.page_size, max_blocks)
+    return types.SimpleNamespace(cfg=cfg, w=w, dec=dec, B=B, prompts=prompts, prompt_lens=prompt_lens, blocks=blocks,
+                                 ctx=ctx, reqs=reqs, dmeta=dmeta, first_tokens=first_tokens, max_blocks=max_blocks, pool=pool)
+
+
+def drift_check(wl, lp_batch, tok_batch, n):
+    """Re-run ``n`` of the workload's requests alone (batch 1, eager) and count the bits in which the logprob
+    differs from the batched step's (64 more for a different token). Returns (bits, requests checked)."""
+    import torch
+
+    from vexact_amd.decoder import build_step_metadata
+
+    bits, checked = 0, 0
+    b1 = wl.dec.bucket(1, 1)
+    for i in range(min(n, wl.B)):
+        r = (i * 37) % wl.B
+        m1 = build_step_metadata([wl.reqs[r]], wl.cfg.page_size, wl.max_blocks)
+        b1.load(m1, wl.first_tokens[r : r + 1])
+        wl.dec.step(b1, 1)
+        torch.cuda.synchronize()
+        a = b1.logprobs.cpu().view(torch.int32)
+        bb = lp_batch[r : r + 1].view(torch.int32)
+        bits += bin((int(a[0]) ^ int(bb[0])) & 0xFFFFFFFF).count("1") + (0 if int(b1.tokens[0]) == int(tok_batch[r]) else 64)
+        checked += 1
+    return bits, checked
+
+
+def main():
+    args = parse()
+    if args.cpu_configs:
+        cpu_configs(args.seed)
+        return
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (all pipeline stages collapsed onto one MI355X); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from vexact_amd import _build, _lib, ops
+    from vexact_amd.decoder import decode_bytes_per_step
+
+    if not os.path.exists(_build.LIB_PATH):
+        _build.build()
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda"
+    torch.cuda.set_device(0)
+
+    wl = build_workload(args.layers, args.batch, args.seed, args.min_prompt, args.max_prompt,
+                        grow=1 + max(0, args.loop_steps), packed=not args.no_packed_experts)
+    cfg, w, dec, B = wl.cfg, wl.w, wl.dec, wl.B
+    blocks, ctx, reqs, dmeta, first_tokens, max_blocks = wl.blocks, wl.ctx, wl.reqs, wl.dmeta, wl.first_tokens, wl.max_blocks
+    E, k, I, H = cfg.num_experts, cfg.top_k, cfg.moe_intermediate, cfg.hidden_size
 
     def moe_gate_up(li, lw, r):
         if w.packed is not None:
@@ -208,9 +252,6 @@ def main():
         return ops.moe_gemm(db.hw, lw["down"], r, out=db.eo)
 
     # ---- the decode step: 256 tokens, 256 sequences, captured in a HIP graph
-    ctx = [int(n) + 1 for n in prompt_lens]
-    reqs = [dict(num_computed_tokens=ctx[i], tokens_this_step=1, block_ids=blocks[i]) for i in range(B)]
-    dmeta = build_step_metadata(reqs, cfg.page_size, max_blocks)
     db = dec.bucket(B, B)
     db.load(dmeta, first_tokens)
     graph = dec.capture(db, 1)
@@ -229,18 +270,7 @@ def main():
 
     # ---- logprob bit drift: the same requests at batch 1 (eager)
     t0 = time.time()
-    drift_bits, checked = 0, 0
-    b1 = dec.bucket(1, 1)
-    for i in range(min(args.drift_requests, B)):
-        r = (i * 37) % B
-        m1 = build_step_metadata([reqs[r]], cfg.page_size, max_blocks)
-        b1.load(m1, first_tokens[r : r + 1])
-        dec.step(b1, 1)
-        torch.cuda.synchronize()
-        a = b1.logprobs.cpu().view(torch.int32)
-        bb = lp_graph[r : r + 1].view(torch.int32)
-        drift_bits += bin(int(a[0]) ^ int(bb[0])).count("1") + (0 if int(b1.tokens[0]) == int(tok_graph[r]) else 64)
-        checked += 1
+    drift_bits, checked = drift_check(wl, lp_graph, tok_graph, args.drift_requests)
     print(f"[bench] drift check of {checked} requests at batch 1: {time.time() - t0:.1f}s, {drift_bits} bits", file=sys.stderr, flush=True)
 
     # ---- an advancing decode loop: what a serving step pays around the graph (inferencer.py:124-191, 193-349):
@@ -272,7 +302,6 @@ def main():
                         "fed back as the next input ids, contexts growing by one"}
 
     # ---- per-kernel timing with HIP events on the launch stream (eager pass over all layers)
-    E, k, I, H = cfg.num_experts, cfg.top_k, cfg.moe_intermediate, cfg.hidden_size
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
     names = ("moe_gate_up", "moe_down", "attn_decode", "qkv_gemm", "o_gemm")
     times = {n: [] for n in names}

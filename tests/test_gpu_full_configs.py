@@ -13,7 +13,8 @@ import torch
 
 from oracle import attention as OA
 from oracle import moe as OM
-from tests.util import assert_bf16_close, assert_bitwise
+from oracle import row_ops as OR
+from tests.util import assert_bf16_close, assert_bitwise, ulp_histogram
 
 pytestmark = pytest.mark.gpu
 
@@ -32,6 +33,77 @@ def _bf16_normal(shape, seed):
     t = torch.empty(shape, dtype=torch.bfloat16, device="cuda")
     t.normal_(0.0, 1.0, generator=g)
     return t
+
+
+def test_config1_op_chain_full_size():
+    # Qwen3-1.7B op chain at hidden 2048, vocabulary 151936: RMSNorm -> lm_head -> .float() -> log_softmax on the
+    # first M rows of ONE 64-row draw, M = 1 / 7 / 64; both RMSNorm forms: HuggingFace's module arithmetic under the
+    # aten overrides (its mean goes through mean_dim, two roundings) and batch_invariant_rms_norm (one rounding)
+    from vexact_amd.batch_invariant_ops import batch_invariant_rms_norm, set_batch_invariant_mode
+
+    H, V = 2048, 151936
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(64, H, generator=g).to(torch.bfloat16)
+    wn = (1 + 0.02 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    W_t = _bf16_normal((V, H), 11) * 0.02  # contiguous [V, H]; the chain multiplies by W_t.t()
+    xd, wnd = x.cuda(), wn.cuda()
+
+    def hf_norm(t):  # the module's forward, op by op
+        t32 = t.to(torch.float32)
+        var = t32.pow(2).mean(-1, keepdim=True)
+        return wnd * (t32 * torch.rsqrt(var + 1e-6)).to(t.dtype)
+
+    def chain(t, form):
+        h = hf_norm(t) if form == "hf" else batch_invariant_rms_norm(t, wnd, 1e-6)
+        logits = torch.mm(h, W_t.t())
+        return h, logits, torch.log_softmax(logits.float(), dim=-1)
+
+    W_cpu = W_t.cpu()
+    for form in ("hf", "one-rounding"):
+        with set_batch_invariant_mode(True):
+            outs = {M: chain(xd[:M], form) for M in (1, 7, 64)}
+        full = outs[64]
+        for M in (1, 7):
+            for name, a, b in zip(("norm", "logits", "log_softmax"), outs[M], full):
+                assert_bitwise(a, b[:M], f"{form}: {name} rows at M={M} vs the same rows at M=64")
+        # against the CPU oracle on the same bits
+        h_ref = OR.hf_rms_norm_ref(x, wn) if form == "hf" else OR.rms_norm_ref(x, wn)
+        ulp_histogram(full[0], h_ref, f"C1 {form} RMSNorm vs oracle")
+        assert_bf16_close(full[0], h_ref, max_ulp=1, atol_frac=0.0, what=f"{form} RMSNorm")
+        logits_ref = OR.matmul_ref(full[0].cpu(), W_cpu.t())  # the GEMM on the kernel's own normalised rows
+        hist = ulp_histogram(full[1], logits_ref, f"C1 {form} logits [64, 151936] vs oracle")
+        # <= 2 bf16 ulp; the few elements beyond sit where the 2048-term sum cancels to a small number
+        assert hist[">2"] <= 1e-4
+        assert_bf16_close(full[1], logits_ref, max_ulp=2, atol_frac=1e-3, what=f"{form} logits")
+        lp_ref = OR.log_softmax_ref(full[1].cpu().float())
+        assert float((full[2].cpu() - lp_ref).abs().max()) <= 2e-5, "log_softmax of the kernel's logits vs oracle"
+        lp_chain = OR.log_softmax_ref(OR.matmul_ref(h_ref, W_cpu.t()).float())
+        assert float((full[2].cpu() - lp_chain).abs().max()) <= 2e-2, "whole chain logprob vs oracle"
+
+
+def test_config5_full_model_batch_256_equals_batch_1():
+    # the whole 48-layer Qwen3-30B-A3B-shaped decoder: one graph-captured decode step at batch 256 against every
+    # request alone at batch 1 (eager): 0 differing logprob bits, same greedy token
+    import bench
+
+    wl = bench.build_workload(layers=48, batch=256, seed=5, log=False)
+    db = wl.dec.bucket(wl.B, wl.B)
+    db.load(wl.dmeta, wl.first_tokens)
+    graph = wl.dec.capture(db, 1)
+    for rep in range(2):
+        db.logprobs.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        lp, tok = db.logprobs.cpu().clone(), db.tokens.cpu().clone()
+        if rep == 0:
+            lp0, tok0 = lp, tok
+        else:
+            assert_bitwise(lp, lp0, "second replay of the decode graph")
+    assert bool(torch.isfinite(lp0).all()) and bool((lp0 < 0).all())
+    bits, checked = bench.drift_check(wl, lp0, tok0, 256)
+    assert checked == 256 and bits == 0, f"{bits} differing bits over {checked} requests"
+    del wl, db, graph
+    torch.cuda.empty_cache()
 
 
 def test_config2_paged_decode_full_size():
@@ -64,6 +136,7 @@ def test_config2_paged_decode_full_size():
     # tolerance of the reference's own paged-vs-eager test (test_triton_attention_varlen.py:390-415): the eager
     # oracle rounds normalised probabilities, the kernel un-normalised ones, over up to 4096 keys
     torch.testing.assert_close(out[sub].cpu().float(), ref.float(), atol=3e-3, rtol=3e-3)
+    ulp_histogram(out[sub], ref, "C2 decode attention rows vs eager oracle")
 
 
 def test_config3_chunked_prefill_full_size():
@@ -99,6 +172,7 @@ def test_config3_chunked_prefill_full_size():
     assert_bitwise(dec, out[last.cuda()], "last row of each chunk vs decode")
     # oracle on a few rows: row i of a chunk is the last row of attention over the first prefix + i + 1 keys
     kc, vc, qc = k_cache.cpu(), v_cache.cpu(), q.cpu()
+    got_rows, ref_rows = [], []
     for s in (0, 1, 5):
         ks = OA.gather_paged(kc, table[s], kv_lens[s])
         vs = OA.gather_paged(vc, table[s], kv_lens[s])
@@ -107,6 +181,9 @@ def test_config3_chunked_prefill_full_size():
             ref = OA.eager_attention(qc[s * C + i : s * C + i + 1], ks[:n], vs[:n], D**-0.5)
             torch.testing.assert_close(out[s * C + i : s * C + i + 1].cpu().float(), ref.float(), atol=3e-3, rtol=3e-3,
                                        msg=lambda m: f"sequence {s} chunk row {i} vs eager oracle: {m}")
+            got_rows.append(out[s * C + i : s * C + i + 1].cpu())
+            ref_rows.append(ref)
+    ulp_histogram(torch.cat(got_rows), torch.cat(ref_rows), "C3 chunked prefill rows vs eager oracle")
 
 
 def test_config4_fused_moe_full_size():
@@ -138,4 +215,5 @@ def test_config4_fused_moe_full_size():
     rows = torch.tensor([0, 63, 255, 1000, 4095])
     gu = gate_up.cpu()
     ref = OM.fused_moe_ref(x.cpu()[rows], w.cpu()[rows], idx.cpu()[rows], gu[:, :I], gu[:, I:], down.cpu())
+    ulp_histogram(full[rows.cuda()], ref, "C4 fused MoE rows vs fused-order oracle")
     assert_bf16_close(full[rows.cuda()], ref, max_ulp=2, atol_frac=2e-3, what="config-4 rows vs fused-order oracle")

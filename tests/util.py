@@ -46,3 +46,15 @@ def assert_bf16_close(a, b, max_ulp=2, atol_frac=1e-4, what=""):
         f"{what}: {int(bad.sum())} of {a.numel()} elements beyond {max_ulp} ulp "
         f"(worst {int(ulp.max())} ulp, |d|max {float(absd.max()):.3e}, atol {atol:.3e})"
     )
+
+
+def ulp_histogram(a: torch.Tensor, b: torch.Tensor, what: str = "") -> dict:
+    """Share of elements at 0 / 1 / 2 / more bf16 ulps from the reference, with no absolute floor; printed so
+    that the tolerance a test meets is a measured one."""
+    ulp = bf16_ulp_distance(a, b)
+    n = max(1, ulp.numel())
+    h = {"0": float((ulp == 0).sum()) / n, "1": float((ulp == 1).sum()) / n, "2": float((ulp == 2).sum()) / n,
+         ">2": float((ulp > 2).sum()) / n, "worst": int(ulp.max()) if ulp.numel() else 0}
+    print(f"[ulp] {what}: 0 ulp {h['0']:.4%}, 1 ulp {h['1']:.4%}, 2 ulp {h['2']:.4%}, >2 ulp {h['>2']:.4%} "
+          f"(worst {h['worst']}) of {ulp.numel()} elements", flush=True)
+    return h
