@@ -41,6 +41,13 @@ def test_host_only_helpers():
     assert lib.vx_paged_attn_decode_workspace_bytes(64, 16, 4, 128, 4096) == 64 * 4 * 16 * 9 * 1024
     assert lib.vx_paged_attn_decode_workspace_bytes(1, 1, 1, 128, 1) == 9 * 1024
     assert lib.vx_paged_attn_decode_workspace_bytes(2, 64, 2, 256, 257) == 2 * 2 * 2 * (2 * 2 * 8 + 2) * 1024
+    # what a launch really uses: nothing when the fused decode form is taken (mode 4, or mode 0 from 512 (sequence, kv head) pairs)
+    assert lib.vx_paged_attn_decode_workspace_needed(256, 32, 4, 128, 4096, 0) == 0
+    assert lib.vx_paged_attn_decode_workspace_needed(64, 16, 8, 128, 4096, 0) == 0
+    assert lib.vx_paged_attn_decode_workspace_needed(8, 32, 4, 128, 4096, 0) == lib.vx_paged_attn_decode_workspace_bytes(8, 32, 4, 128, 4096)
+    assert lib.vx_paged_attn_decode_workspace_needed(256, 32, 4, 128, 4096, 3) == lib.vx_paged_attn_decode_workspace_bytes(256, 32, 4, 128, 4096)
+    assert lib.vx_paged_attn_decode_workspace_needed(8, 32, 4, 128, 4096, 4) == 0
+    assert lib.vx_paged_attn_decode_workspace_needed(8, 32, 4, 128, 4096, 1) == 0  # not a decode mode
     # 16 bytes per (row, 4096-column chunk)
     assert lib.vx_log_softmax_workspace_bytes(7, 151936) == 7 * 38 * 16
     assert lib.vx_moe_max_tiles(2048, 128, 32) == 128 + 64

@@ -200,6 +200,85 @@ def test_attention_wrapper_shape_and_cache_write():
     assert_bitwise(kc, full_k, "wrapper wrote the new keys")
 
 
+def test_attention_wrapper_gives_the_same_bits_for_any_memory_layout():
+    # HuggingFace hands [1, heads, tokens, dim] tensors that are views of [1, tokens, heads, dim] memory; the wrapper
+    # reads them through strides. A tensor that really is head-major in memory must give the same bits, in the
+    # paged, the packed-context and the no-context branch.
+    qh, kh, d, page = 8, 2, 128, 16
+    lens = [37, 5, 64]
+    q, k, v = _seqs(lens, qh, d, 40), _seqs(lens, kh, d, 41), _seqs(lens, kh, d, 42)
+    T = sum(lens)
+    cu = _cu(lens).cuda()
+    module = torch.nn.Module()
+    module.layer_idx = 0
+    module.is_causal = True
+
+    def views(layout):
+        outs = []
+        for t in (torch.cat(q), torch.cat(k), torch.cat(v)):
+            x = t.cuda()                                        # [T, H, D] in memory
+            if layout == "token-major":
+                outs.append(x.transpose(0, 1).unsqueeze(0))     # [1, H, T, D] view of it
+            else:
+                outs.append(x.transpose(0, 1).contiguous().unsqueeze(0))  # [1, H, T, D] in memory
+        return outs
+
+    results = {}
+    for layout in ("token-major", "head-major"):
+        qq, kk, vv = views(layout)
+        # paged: empty cache, every token of the step is written, then attended
+        k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, page)
+        kc, vc = torch.zeros_like(k_cache).cuda(), torch.zeros_like(v_cache).cuda()
+        slots = [int(table[s, pos // page]) * page + pos % page for s, n in enumerate(lens) for pos in range(n)]
+        set_kv_cache_context(is_paged_attn=True, key_cache={0: kc}, value_cache={0: vc}, block_tables=table.cuda(),
+                             context_lens=torch.tensor(lens, dtype=torch.int32).cuda(),
+                             slot_mapping=torch.tensor(slots, dtype=torch.int32).cuda(), query_start_loc=cu, max_seqlen_q=max(lens))
+        try:
+            paged, _ = flash_attention_forward(module, qq, kk, vv, None, scaling=d**-0.5)
+        finally:
+            clear_kv_cache_context()
+        assert_bitwise(kc, k_cache, f"{layout}: keys written by the wrapper")
+        # packed context
+        set_kv_cache_context(is_paged_attn=False, context_lens=torch.tensor(lens, dtype=torch.int32).cuda(),
+                             query_start_loc=cu, max_seqlen_q=max(lens))
+        try:
+            packed, _ = flash_attention_forward(module, qq, kk, vv, None, scaling=d**-0.5)
+        finally:
+            clear_kv_cache_context()
+        # no context: boundaries in the call
+        plain, _ = flash_attention_forward(module, qq, kk, vv, None, scaling=d**-0.5, cu_seq_lens_q=cu, cu_seq_lens_k=cu,
+                                           max_length_q=max(lens), max_length_k=max(lens))
+        assert paged.shape == (T, qh, d) and packed.shape == (T, qh, d) and plain.shape == (1, T, qh, d)
+        assert_bitwise(packed, paged, f"{layout}: packed context vs paged")
+        assert_bitwise(plain[0], paged, f"{layout}: no context vs paged")
+        results[layout] = paged
+    assert_bitwise(results["head-major"], results["token-major"], "head-major vs token-major inputs")
+    ref = torch.cat([OA.eager_attention(a, b, c, d**-0.5) for a, b, c in zip(q, k, v)], dim=0)
+    assert_bf16_close(results["token-major"], ref, max_ulp=2, atol_frac=2e-3, what="wrapper vs eager oracle")
+
+
+def test_rows_of_a_sequence_without_any_key_are_left_alone():
+    # a sequence that has a query token but seqused_k = 0 (never built by the model runner): its output row is not
+    # written by any kernel form, and the other sequences are not disturbed
+    from vexact_amd import ops
+
+    qh, kh, d, page = 4, 2, 128, 16
+    kv_lens = [40, 0, 300]
+    k, v = _seqs([40, 1, 300], kh, d, 51), _seqs([40, 1, 300], kh, d, 52)
+    q = _seqs([1, 1, 1], qh, d, 50)
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, page)
+    used = torch.tensor(kv_lens, dtype=torch.int32).cuda()
+    cu = _cu([1, 1, 1]).cuda()
+    ref = [OA.eager_attention(q[s], k[s], v[s], d**-0.5) for s in (0, 2)]
+    for max_q, kernel in ((1, "split"), (1, "fused"), (2, "auto")):
+        out = torch.full((3, qh, d), 9.0, dtype=torch.bfloat16, device="cuda")
+        ops.paged_attention(torch.cat(q).cuda(), k_cache.cuda(), v_cache.cuda(), cu, used, table.cuda(), d**-0.5, max_q,
+                            out=out, decode_kernel=kernel)
+        assert bool((out[1] == 9.0).all()), f"{kernel}: the row without keys was written"
+        for row, want in ((0, ref[0]), (2, ref[1])):  # the neighbours are undisturbed (precision is tested elsewhere)
+            assert float((out[row: row + 1].cpu().float() - want.float()).abs().max()) <= 1e-2, f"{kernel}: sequence {row}"
+
+
 def test_argument_errors():
     q, k, v = _seqs([2], 4, 32, 23), _seqs([2], 2, 32, 24), _seqs([2], 2, 32, 25)
     qg, kg, vg = q[0].cuda(), k[0].cuda(), v[0].cuda()

@@ -7,6 +7,8 @@ routing bit-exact, and the step-by-step path through the public helpers against 
 """
 
 import numpy as np
+import types
+
 import pytest
 import torch
 
@@ -340,13 +342,18 @@ def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
 
     from oracle.row_ops import matmul_ref
     from vexact_amd.batch_invariant_ops import set_batch_invariant_mode
-    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches
+    from vexact_amd.models.qwen3_moe import (apply_qwen3_moe_patches, invalidate_packed_experts, moe_block_forward,
+                                             remove_qwen3_moe_patches)
 
-    apply_qwen3_moe_patches()
     cfg = Qwen3MoeConfig(hidden_size=256, moe_intermediate_size=128, num_experts=16, num_experts_per_tok=4, norm_topk_prob=True,
                          num_hidden_layers=1, vocab_size=100, intermediate_size=64, num_attention_heads=2, num_key_value_heads=1)
     torch.manual_seed(3)
-    blk = Qwen3MoeSparseMoeBlock(cfg).to(torch.bfloat16)
+    apply_qwen3_moe_patches()
+    try:
+        blk = Qwen3MoeSparseMoeBlock(cfg).to(torch.bfloat16)
+    finally:
+        remove_qwen3_moe_patches()  # the instance keeps the fused experts; its forward is called explicitly below
+    blk.forward = types.MethodType(moe_block_forward, blk)
     with torch.no_grad():
         blk.gate.weight.normal_(0, 0.5)
         blk.experts.gate_up_proj.normal_(0, 0.06)
@@ -369,7 +376,25 @@ def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
         assert gpu.experts._packed is None, "stale packed copies must be dropped"
         gpu.experts.down_proj.mul_(0.5)
         assert_bitwise(gpu(x.cuda()), y, "parameters restored")
-    assert not torch.equal(y2, y)
+        # a write through .data (what a weight synchronisation does) leaves no trace on the parameter: the
+        # contract is an explicit invalidation, after which the forward reads the new parameters
+        gpu.experts.pack_for_decode()
+        saved = gpu.experts.gate_up_proj.detach().clone()
+        gpu.experts.gate_up_proj.data.copy_(saved * 0.5)
+        assert invalidate_packed_experts(gpu) == 1 and gpu.experts._packed is None
+        y3 = gpu(x.cuda())
+        gpu.experts.pack_for_decode()
+        assert_bitwise(gpu(x.cuda()), y3, "after a .data write + invalidate: packed again vs parameters")
+        # load_state_dict and .to() are noticed by the module itself
+        sd = {k_: v_.clone() for k_, v_ in gpu.state_dict().items()}
+        sd["experts.gate_up_proj"] = saved
+        gpu.load_state_dict(sd)
+        assert gpu.experts._packed is None, "load_state_dict must drop the packed copies"
+        assert_bitwise(gpu(x.cuda()), y, "weights loaded back")
+        gpu.experts.pack_for_decode()
+        gpu = gpu.to("cuda")
+        assert gpu.experts._packed is None, ".to() must drop the packed copies"
+    assert not torch.equal(y2, y) and not torch.equal(y3, y)
     cpu = blk.to("cpu")
     logits = matmul_ref(x[0], cpu.gate.weight.detach().t())
     w, idx = OM.router_ref(logits, 4)

@@ -232,13 +232,20 @@ def test_qwen3_moe_patch_points():
     # container with the reference's parameter names and layout, a plain linear router
     from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeConfig, Qwen3MoeSparseMoeBlock
 
-    from vexact_amd.models.qwen3_moe import Qwen3MoeExperts, apply_qwen3_moe_patches, moe_block_forward
+    from vexact_amd.models.qwen3_moe import (Qwen3MoeExperts, apply_qwen3_moe_patches, moe_block_forward,
+                                             remove_qwen3_moe_patches)
 
+    original = (Qwen3MoeSparseMoeBlock.__init__, Qwen3MoeSparseMoeBlock.forward)
     apply_qwen3_moe_patches()
     apply_qwen3_moe_patches()
     cfg = Qwen3MoeConfig(hidden_size=64, moe_intermediate_size=32, num_experts=8, num_experts_per_tok=2, norm_topk_prob=True,
                          num_hidden_layers=1, vocab_size=100, intermediate_size=64, num_attention_heads=2, num_key_value_heads=1)
-    blk = Qwen3MoeSparseMoeBlock(cfg)
+    try:
+        blk = Qwen3MoeSparseMoeBlock(cfg)
+    finally:
+        remove_qwen3_moe_patches()
+        remove_qwen3_moe_patches()
+    assert (Qwen3MoeSparseMoeBlock.__init__, Qwen3MoeSparseMoeBlock.forward) == original, "the original block is back"
     assert isinstance(blk.experts, Qwen3MoeExperts) and isinstance(blk.gate, torch.nn.Linear) and blk.gate.bias is None
     assert dict(blk.named_parameters()).keys() == {"gate.weight", "experts.gate_up_proj", "experts.down_proj"}
     assert blk.experts.gate_up_proj.shape == (8, 64, 64) and blk.experts.down_proj.shape == (8, 64, 32)

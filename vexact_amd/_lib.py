@@ -31,6 +31,7 @@ PROTOTYPES = {
     "vx_store_kvcache": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _P]),
     "vx_attn_chunk_size": (_I, []),
     "vx_paged_attn_decode_workspace_bytes": (_L, [_L, _L, _L, _L, _L]),
+    "vx_paged_attn_decode_workspace_needed": (_L, [_L, _L, _L, _L, _L, _I]),
     "vx_attention": (
         _I,
         [_P] * 8 + [_L, _L, _I, _I, _I, _I] + [_L] * 12 + [_I, _F, _I, _I, _I, _P, _L, _P],

@@ -143,27 +143,29 @@ class KVCacheManager:
             self._lib.vx_kv_allocator_free(self._h, (ctypes.c_int32 * len(ids))(*ids), len(ids))
 
 
+def _kv_head_dims(hf_config) -> tuple[int, int]:
+    """(key head size, value head size): models with separate sizes (multi-head latent attention) name them
+    ``qk_head_dim`` / ``v_head_dim``; the others have one ``head_dim`` or ``hidden_size / heads``."""
+    base = getattr(hf_config, "head_dim", None) or hf_config.hidden_size // hf_config.num_attention_heads
+    dk = getattr(hf_config, "qk_head_dim", base)
+    return dk, getattr(hf_config, "v_head_dim", dk)
+
+
 class KVCacheStore:
-    """Owns per-layer ``[num_blocks, page_size, Hkv, D]`` key/value tensors (zero initialised)."""
+    """Paged key / value memory of a model: ``key_cache[layer]`` and ``value_cache[layer]`` are
+    ``[max_cache_blocks, page_size, Hkv, D]`` tensors, zero initialised (reference: kv_cache_context.py:220-253).
+    All layers of a kind live in ONE allocation (a ``[layers, blocks, page, Hkv, D]`` slab): two large
+    allocations for the whole pool instead of two per layer, and the per-layer tensors are views of it."""
 
     def __init__(self, hf_config, cache_config, device: torch.device):
-        self.hf_config = hf_config
-        self.cache_config = cache_config
-        self.device = device
-        self.page_size = cache_config.page_size
-        self.max_blocks = cache_config.max_cache_blocks
-        num_kv_heads = hf_config.num_key_value_heads
-        default_head_dim = getattr(hf_config, "head_dim", hf_config.hidden_size // hf_config.num_attention_heads)
-        k_head_dim = getattr(hf_config, "qk_head_dim", default_head_dim)
-        v_head_dim = getattr(hf_config, "v_head_dim", k_head_dim)
-        k_shape = (cache_config.max_cache_blocks, cache_config.page_size, num_kv_heads, k_head_dim)
-        v_shape = (cache_config.max_cache_blocks, cache_config.page_size, num_kv_heads, v_head_dim)
+        self.hf_config, self.cache_config, self.device = hf_config, cache_config, device
+        self.page_size, self.max_blocks = cache_config.page_size, cache_config.max_cache_blocks
         dtype = getattr(hf_config, "torch_dtype", None) or torch.bfloat16
-        self.key_cache: dict[int, torch.Tensor] = {}
-        self.value_cache: dict[int, torch.Tensor] = {}
-        for layer_idx in range(hf_config.num_hidden_layers):
-            self.key_cache[layer_idx] = torch.zeros(k_shape, device=device, dtype=dtype)
-            self.value_cache[layer_idx] = torch.zeros(v_shape, device=device, dtype=dtype)
+        layers, heads = hf_config.num_hidden_layers, hf_config.num_key_value_heads
+        slabs = [torch.zeros((layers, self.max_blocks, self.page_size, heads, d), device=device, dtype=dtype)
+                 for d in _kv_head_dims(hf_config)]
+        self.key_cache: dict[int, torch.Tensor] = dict(enumerate(slabs[0].unbind(0)))
+        self.value_cache: dict[int, torch.Tensor] = dict(enumerate(slabs[1].unbind(0)))
 
 
 def store_kvcache(

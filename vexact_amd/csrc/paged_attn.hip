@@ -1021,18 +1021,30 @@ __global__ __launch_bounds__(256) void store_kv_kernel(const uint8_t* __restrict
       *(uint4*)(vc + (int64_t)slot * v_row_bytes + b) = *(const uint4*)(vsrc + t * vs_stride + b);
 }
 
+// Which decode form a launch takes: chunks folded inside one workgroup per (sequence, kv head) when that
+// fills the machine (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3); only the
+// latter uses the workspace. A function of the shapes alone. Returns 1 = fused, 0 = split, < 0 = error.
+static int decode_form(int mode, int64_t num_seqs, int Hq, int Hkv, int Dv) {
+  const int G = Hq / Hkv;
+  if (G > 32) return VX_ERR_UNSUPPORTED;
+  const int QT = G <= 16 ? 1 : 2, NW = G <= 16 ? 8 : 4;
+  const int64_t lds = ((int64_t)NW * (QT * ((Dv + 127) / 128) * 8 + QT) * 64 + 16 * QT * (Dv / 4)) * 16 + 16 * QT * (Dv / 4) * 8;
+  const bool fits = lds <= 160 * 1024;
+  if (mode == 4 && !fits) return VX_ERR_UNSUPPORTED;
+  return (mode == 4 || (mode == 0 && fits && num_seqs * Hkv >= 512)) ? 1 : 0;
+}
+
 template <int DK, int DV>
 static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hipStream_t stream) {
   const bool fast = p.page_shift >= 4;  // page size a power of two >= 16
   if (mode == 0 || mode == 3 || mode == 4) {
-    // decode: chunks folded inside one workgroup per (sequence, kv head) when that fills the machine
-    // (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3). Same bits.
     const int G = p.Hq / p.Hkv;
     constexpr int NW1 = 8, NW1S = 4, NW2 = 4;  // wavefronts per block for one (many / very many workgroups) / two q-tiles
-    if (G > 32) return VX_ERR_UNSUPPORTED;
-    const bool fits = (G <= 16 ? fused_lds_bytes<DV, 1, NW1>() : fused_lds_bytes<DV, 2, NW2>()) <= 160 * 1024;
-    if (mode == 4 && !fits) return VX_ERR_UNSUPPORTED;
-    const bool fused = mode == 4 || (mode == 0 && fits && (int64_t)p.num_seqs * p.Hkv >= 512);
+    static_assert(fused_lds_bytes<DV, 1, NW1>() == ((int64_t)NW1 * (((DV + 127) / 128) * 8 + 1) * 64 + 16 * (DV / 4)) * 16 + 16 * (DV / 4) * 8,
+                  "decode_form() restates fused_lds_bytes");
+    const int form = decode_form(mode, p.num_seqs, p.Hq, p.Hkv, DV);
+    if (form < 0) return form;
+    const bool fused = form == 1;
     if (fused) {
       const dim3 grid(p.Hkv, p.num_seqs);
 #define VX_FUSED(KERNEL, QTV, KINDV, NW)                                                             \
@@ -1147,12 +1159,21 @@ static inline int64_t part_image_floats(int64_t Hq, int64_t Hkv, int64_t Dv) {
   return (qt * ndv * 8 + qt) * 256;
 }
 
-// bytes of workspace the decode path needs
+// bytes of workspace that is enough for any decode mode (the split form's chunk images)
 int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Hkv, int64_t Dv,
                                              int64_t max_kv_len) {
   if (num_seqs <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Dv <= 0 || max_kv_len <= 0) return 0;
   const int64_t nch = (max_kv_len + ATT_CHUNK - 1) / ATT_CHUNK;
   return num_seqs * Hkv * nch * part_image_floats(Hq, Hkv, Dv) * 4;
+}
+
+// bytes the launch with this mode will really use: 0 when it takes the fused form
+int64_t vx_paged_attn_decode_workspace_needed(int64_t num_seqs, int64_t Hq, int64_t Hkv, int64_t Dv,
+                                              int64_t max_kv_len, int mode) {
+  if (mode != 0 && mode != 3 && mode != 4) return 0;
+  if (num_seqs <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Dv <= 0 || max_kv_len <= 0) return 0;
+  if (decode_form(mode, num_seqs, (int)Hq, (int)Hkv, (int)Dv) == 1) return 0;
+  return vx_paged_attn_decode_workspace_bytes(num_seqs, Hq, Hkv, Dv, max_kv_len);
 }
 
 // mode: 0 = paged decode (every sequence has <= 1 query token; needs workspace); 3 / 4 = the same,
@@ -1223,10 +1244,12 @@ int vx_attention_ex(const void* q, const void* k, const void* v, void* out, floa
     const int64_t nch = (max_kv + ATT_CHUNK - 1) / ATT_CHUNK;
     if (nch > 0x7fffffff) return VX_ERR_ARG;
     p.img_floats = part_image_floats(Hq, Hkv, Dv);
-    const int64_t need = num_seqs * Hkv * nch * p.img_floats * 4;
-    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return VX_ERR_WORKSPACE;
     p.max_chunks = (int)nch;
-    p.part = (float*)workspace;
+    if (decode_form(mode, num_seqs, Hq, Hkv, Dv) != 1) {  // the fused form keeps its chunk states in LDS
+      const int64_t need = num_seqs * Hkv * nch * p.img_floats * 4;
+      if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return VX_ERR_WORKSPACE;
+      p.part = (float*)workspace;
+    }
   }
   const int tq = (int)total_q;
   if (Dk == 128 && Dv == 128) return launch_attn<128, 128>(p, mode, max_seqlen_q, tq, stream);

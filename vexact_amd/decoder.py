@@ -264,10 +264,10 @@ class StepBuffers:
         lib = _lib.load()
         self.max_tiles = lib.vx_moe_max_tiles(T * k, cfg.num_experts, self.bm)
         self.route_ints = z(2 * cfg.num_experts + 1 + 3 * T * k + 3 * self.max_tiles, dtype=i32)
-        self.attn_ws = torch.empty(
-            max(16, lib.vx_paged_attn_decode_workspace_bytes(B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
-                                                            self.max_blocks * cfg.page_size)),
-            dtype=torch.uint8, device=device)
+        # chunk states of the split decode form (nothing when this bucket's decode takes the fused form)
+        self.attn_ws_bytes = lib.vx_paged_attn_decode_workspace_needed(B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
+                                                                      self.max_blocks * cfg.page_size, 0)
+        self.attn_ws = None  # handed out by the decoder: one workspace shared by all buckets
         # sampling: one row per sequence
         self.last_h = z(B, H, dtype=bf)
         self.logits = z(B, cfg.vocab_size, dtype=bf)
@@ -332,11 +332,19 @@ class Qwen3MoeDecoder:
         self.buffers: dict[tuple[int, int], StepBuffers] = {}
         self.graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
         self.prefetch_next_qkv = True  # see forward(): a cache hint, never a result
+        self._attn_ws: Optional[torch.Tensor] = None
 
     def bucket(self, num_tokens: int, num_seqs: int) -> StepBuffers:
         key = (num_tokens, num_seqs)
         if key not in self.buffers:
-            self.buffers[key] = StepBuffers(self.cfg, num_tokens, num_seqs, self.device)
+            b = self.buffers[key] = StepBuffers(self.cfg, num_tokens, num_seqs, self.device)
+            # Steps run one at a time on one stream, so buckets share one decode-attention workspace. A bucket
+            # that needs more than the shared one holds gets a new, larger one, which later buckets share;
+            # earlier buckets (and graphs captured on them) keep the tensor they were given.
+            if b.attn_ws_bytes > 0:
+                if self._attn_ws is None or self._attn_ws.numel() < b.attn_ws_bytes:
+                    self._attn_ws = torch.empty(b.attn_ws_bytes, dtype=torch.uint8, device=self.device)
+                b.attn_ws = self._attn_ws
         return self.buffers[key]
 
     # ---- one forward pass over a bucket's static buffers (capture-safe: no sync, no host reads)

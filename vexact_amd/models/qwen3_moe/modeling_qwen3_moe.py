@@ -20,7 +20,7 @@ import torch.nn as nn
 from ... import ops
 from ...batch_invariant_ops.fused_moe import fused_moe_forward
 
-_PATCHED = False
+_ORIGINAL = None  # (Qwen3MoeSparseMoeBlock.__init__, .forward) while the patches are applied
 
 
 class Qwen3MoeExperts(nn.Module):
@@ -37,19 +37,35 @@ class Qwen3MoeExperts(nn.Module):
         self.down_proj = nn.Parameter(torch.empty(self.num_experts, self.hidden_dim, self.intermediate_size))
 
         self._packed = None  # (packed gate_up, packed down, (data_ptr, version) of both parameters)
+        # every path of this module that replaces or rewrites the parameters drops the copies
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module.invalidate_packed())
 
     def _weights_key(self):
         return (self.gate_up_proj.data_ptr(), self.gate_up_proj._version, self.down_proj.data_ptr(), self.down_proj._version)
 
     def pack_for_decode(self) -> None:
         """Keep fragment-order copies of both parameters for decode-sized steps (a second copy of the
-        expert weights in HBM). They are dropped, and the parameters read again, once a parameter has
-        been written in place (weight synchronisation) until this is called again."""
+        expert weights in HBM; opt-in).
+
+        Contract: the copies are a snapshot. Whoever writes the parameters afterwards must call
+        ``invalidate_packed()`` (or this method again) before the next forward; ``invalidate_packed_experts(model)``
+        does it for every layer after a weight synchronisation. ``load_state_dict``, ``.to()`` / ``.cuda()`` and
+        in-place tensor methods on the parameter (``mul_``, ``copy_`` ...) are noticed by the module itself. A write
+        through ``param.data`` (what the reference's weight sync does, vexact/inferencer/model_loader.py:113) or a
+        raw device copy leaves no trace a module could see, hence the explicit call."""
         if self.intermediate_size % 16 != 0 or self.gate_up_proj.dtype != torch.bfloat16:
             raise ValueError("packed expert weights need bf16 parameters and an intermediate size that is a multiple of 16")
         with torch.no_grad():
             self._packed = (ops.pack_expert_weights(self.gate_up_proj.detach()),
                             ops.pack_expert_weights(self.down_proj.detach()), self._weights_key())
+
+    def invalidate_packed(self) -> None:
+        """Forget the fragment-order copies: the next forward reads the parameters."""
+        self._packed = None
+
+    def _apply(self, fn, *args, **kwargs):  # .to() / .cuda() / .half(): new storage, the copies are void
+        self._packed = None
+        return super()._apply(fn, *args, **kwargs)
 
     def forward(self, hidden_states: torch.Tensor, expert_idx: Optional[int] = None,
                 routing_weights: Optional[torch.Tensor] = None, selected_experts: Optional[torch.Tensor] = None):
@@ -103,13 +119,36 @@ def moe_block_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
     return out.reshape(batch_size, sequence_length, hidden_dim)
 
 
+def invalidate_packed_experts(model: nn.Module) -> int:
+    """Drop the fragment-order expert copies of every layer of ``model``; call once after a weight
+    synchronisation that wrote the parameters. Returns the number of expert containers visited."""
+    n = 0
+    for m in model.modules():
+        if isinstance(m, Qwen3MoeExperts):
+            m.invalidate_packed()
+            n += 1
+    return n
+
+
 def apply_qwen3_moe_patches() -> None:
     """Swap the HuggingFace block's constructor and forward (idempotent)."""
-    global _PATCHED
-    if _PATCHED:
+    global _ORIGINAL
+    if _ORIGINAL is not None:
         return
     from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeSparseMoeBlock
 
+    _ORIGINAL = (Qwen3MoeSparseMoeBlock.__init__, Qwen3MoeSparseMoeBlock.forward)
     Qwen3MoeSparseMoeBlock.__init__ = moe_block_init
     Qwen3MoeSparseMoeBlock.forward = moe_block_forward
-    _PATCHED = True
+
+
+def remove_qwen3_moe_patches() -> None:
+    """Put the HuggingFace block's own constructor and forward back (blocks built meanwhile keep their fused
+    experts and stop working with the original forward; meant for tests and tools that need both forms)."""
+    global _ORIGINAL
+    if _ORIGINAL is None:
+        return
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeSparseMoeBlock
+
+    Qwen3MoeSparseMoeBlock.__init__, Qwen3MoeSparseMoeBlock.forward = _ORIGINAL
+    _ORIGINAL = None

@@ -429,9 +429,10 @@ def paged_attention(
     max_pages = page_table.shape[1]
     mode = {"auto": 0, "split": 3, "fused": 4}[decode_kernel] if max_seqlen_q == 1 else 1
     ws = None
-    if mode != 1:
-        need = lib.vx_paged_attn_decode_workspace_bytes(B, Hq, Hkv, Dv, max_pages * page)
-        ws = workspace if workspace is not None and workspace.numel() * workspace.element_size() >= need else _workspace(need, q.device)
+    if mode != 1:  # only the split decode form keeps chunk states in memory; the fused form needs none
+        need = lib.vx_paged_attn_decode_workspace_needed(B, Hq, Hkv, Dv, max_pages * page, mode)
+        if need > 0:
+            ws = workspace if workspace is not None and workspace.numel() * workspace.element_size() >= need else _workspace(need, q.device)
     if seq_order is not None and (mode == 1 or seq_order.dtype != torch.int32 or seq_order.numel() != B
                                   or not seq_order.is_contiguous()):
         raise ValueError("seq_order must be a contiguous int32 permutation of the sequences, for decode steps only")
