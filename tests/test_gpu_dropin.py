@@ -1,0 +1,166 @@
+"""The drop-in seen from the reference's callers: a HuggingFace ``Qwen3MoeForCausalLM`` driven the way
+``Inferencer`` drives it (vexact/inferencer/inferencer.py:52-55, 124-191, 351-383; model wrapper
+vexact/inferencer/model_loader.py:217-278): the attention function registered under the reference's name
+in ``ALL_ATTENTION_FUNCTIONS``, the MoE block patched, batch-invariant mode on, a thread-local paged KV
+context per step, packed batch of size 1. Paged prefill of three prompts, then a decode step: every
+request alone gives the bits it gives in the batch, and the logprobs agree with the CPU oracle of the
+whole decoder (the assertions of tests/test_inferencer.py:300-595 without the stored tensors of a real
+checkpoint)."""
+
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import decoder as OD
+from tests.util import assert_bitwise
+
+pytestmark = pytest.mark.gpu
+
+BF = torch.bfloat16
+
+
+def _build_model(seed):
+    from transformers.models.qwen3_moe.configuration_qwen3_moe import Qwen3MoeConfig
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeForCausalLM
+
+    cfg = Qwen3MoeConfig(
+        vocab_size=1000, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+        num_key_value_heads=2, head_dim=128, num_experts=8, num_experts_per_tok=2, moe_intermediate_size=128,
+        norm_topk_prob=True, max_position_embeddings=512, rms_norm_eps=1e-6,
+        rope_parameters={"rope_type": "default", "rope_theta": 1.0e6})
+    cfg._attn_implementation = "triton-invariant"
+    model = Qwen3MoeForCausalLM(cfg)
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if "norm" in name:
+                p.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+            else:
+                p.copy_(0.05 * torch.randn(p.shape, generator=g))
+    for p in model.parameters():  # parameters only: the rotary embedding's inv_freq buffer stays fp32, as in a
+        p.data = p.data.to(BF)    # model created by the reference's loader (model_loader.py:307-320)
+    return cfg, model.eval()
+
+
+def _oracle_weights(model):
+    layers = []
+    for l in model.model.layers:
+        a, m = l.self_attn, l.mlp
+        layers.append({k: v.detach().cpu() for k, v in dict(
+            in_norm=l.input_layernorm.weight, post_norm=l.post_attention_layernorm.weight,
+            qkv=torch.cat([a.q_proj.weight, a.k_proj.weight, a.v_proj.weight], dim=0), q_norm=a.q_norm.weight,
+            k_norm=a.k_norm.weight, o=a.o_proj.weight, router=m.gate.weight, gate_up=m.experts.gate_up_proj,
+            down=m.experts.down_proj).items()})
+    return types.SimpleNamespace(embed=model.model.embed_tokens.weight.detach().cpu(), lm_head=model.lm_head.weight.detach().cpu(),
+                                 final_norm=model.model.norm.weight.detach().cpu(), layers=layers)
+
+
+def test_huggingface_causal_lm_through_the_registered_interfaces():
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+    from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
+    from vexact_amd.batch_invariant_ops.standalone_logprobs import logprobs_from_logits_flash_attn
+    from vexact_amd.batch_invariant_ops.kv_cache_context import (KVCacheManager, KVCacheStore, clear_kv_cache_context,
+                                                                 set_kv_cache_context)
+    from vexact_amd.decoder import build_step_metadata
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+
+    page, max_blocks_per_req = 16, 32
+    cache_cfg = types.SimpleNamespace(page_size=page, max_cache_blocks=64)
+    had = ALL_ATTENTION_FUNCTIONS._global_mapping.get("triton-invariant") if hasattr(ALL_ATTENTION_FUNCTIONS, "_global_mapping") else None
+    ALL_ATTENTION_FUNCTIONS["triton-invariant"] = flash_attention_forward
+    apply_qwen3_moe_patches()
+    try:
+        hf_cfg, model = _build_model(seed=17)
+        model = model.cuda()
+        weights = _oracle_weights(model)
+        store = KVCacheStore(hf_cfg, cache_cfg, torch.device("cuda"))
+        alloc = KVCacheManager(cache_cfg)
+        rng = np.random.default_rng(18)
+        lens = [37, 5, 120]
+        prompts = [rng.integers(0, hf_cfg.vocab_size, size=n) for n in lens]
+        # blocks for prompt + one generated token, taken in turns so that the tables interleave
+        blocks = [[] for _ in lens]
+        for step in range(max(-(-(n + 1) // page) for n in lens)):
+            for s, n in enumerate(lens):
+                if step < -(-(n + 1) // page):
+                    blocks[s] += list(alloc.allocate_blocks((step + 1) * page, step))
+        routing = []
+        hooks = [l.mlp.experts.register_forward_pre_hook(lambda mod, args, kw: routing.append(kw["selected_experts"].clone()),
+                                                         with_kwargs=True) for l in model.model.layers]
+
+        def step(which, new_tokens, ids):
+            """One Inferencer step over the requests ``which``: returns (last-token logits, greedy tokens, logprobs, meta)."""
+            reqs = [dict(num_computed_tokens=done, tokens_this_step=new, block_ids=blocks[s])
+                    for s, (done, new) in zip(which, new_tokens)]
+            meta = build_step_metadata(reqs, page, max_blocks_per_req)
+            dev = {k: torch.as_tensor(v).cuda() for k, v in meta.items() if k != "max_seqlen_q"}
+            set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache,
+                                 block_tables=dev["block_tables"], context_lens=dev["context_lens"],
+                                 slot_mapping=dev["slot_mapping"], query_start_loc=dev["query_start_loc"],
+                                 max_seqlen_q=int(meta["max_seqlen_q"]))
+            routing.clear()
+            try:
+                with torch.inference_mode(), set_batch_invariant_mode(True):
+                    out = model.model(input_ids=torch.as_tensor(ids)[None].cuda(), position_ids=dev["positions"][None],
+                                      use_cache=False, return_dict=True)
+                    last = (dev["query_start_loc"][1:] - 1).long()
+                    logits = model.lm_head(out.last_hidden_state)[0, last, :]
+                    tokens = logits.argmax(-1)
+                    lp = logprobs_from_logits_flash_attn(logits.float(), tokens)
+            finally:
+                clear_kv_cache_context()
+            return logits.cpu(), tokens.cpu(), lp.cpu(), meta, [r.cpu() for r in routing]
+
+        everyone = [0, 1, 2]
+        # ---- paged prefill of the three prompts in one packed batch, then each alone
+        logits_b, tok_b, lp_b, pmeta, prouting = step(everyone, [(n, n) for n in lens], np.concatenate(prompts))
+        k_after_batch = store.key_cache[0].clone()
+        for s in everyone:
+            logits_1, tok_1, lp_1, _, _ = step([s], [(lens[s], lens[s])], prompts[s])
+            assert_bitwise(logits_1, logits_b[s: s + 1], f"prefill logits of request {s}: alone vs in the batch")
+            assert_bitwise(lp_1, lp_b[s: s + 1], f"prefill logprob of request {s}")
+        assert_bitwise(store.key_cache[0], k_after_batch, "the cache holds the same keys either way")
+        # ---- one decode step on top: batch vs alone
+        dlogits_b, dtok_b, dlp_b, dmeta, drouting = step(everyone, [(n + 1, 1) for n in lens], tok_b.numpy())
+        for s in everyone:
+            dlogits_1, dtok_1, dlp_1, _, _ = step([s], [(lens[s] + 1, 1)], tok_b.numpy()[s: s + 1])
+            assert_bitwise(dlogits_1, dlogits_b[s: s + 1], f"decode logits of request {s}: alone vs in the batch")
+            assert_bitwise(dlp_1, dlp_b[s: s + 1], f"decode logprob of request {s}")
+            assert int(dtok_1[0]) == int(dtok_b[s])
+        for h in hooks:
+            h.remove()
+
+        # ---- the CPU oracle of the whole decoder on the same weights, following the GPU's expert choice at near-ties
+        ocfg = types.SimpleNamespace(num_heads=4, num_kv_heads=2, head_dim=128, moe_intermediate=128, rms_eps=1e-6, top_k=2,
+                                     norm_topk_prob=True)
+        cos, sin = OD.rope_tables_ref(128, 1.0e6, 512)
+        kc = [torch.zeros(64, page, 2, 128, dtype=BF) for _ in range(2)]
+        vc = [torch.zeros_like(t) for t in kc]
+        report = []
+        ref_logits, _, _ = OD.decoder_step_ref(ocfg, weights, np.concatenate(prompts), pmeta, kc, vc, cos, sin, prouting, report)
+        lp_ref = torch.log_softmax(ref_logits.float(), -1).gather(-1, tok_b[:, None])[:, 0]
+        assert float((lp_b - lp_ref).abs().max()) <= 2e-2, "prefill logprob vs the decoder oracle"
+        ref_logits, _, _ = OD.decoder_step_ref(ocfg, weights, tok_b.numpy(), dmeta, kc, vc, cos, sin, drouting, report)
+        lp_ref = torch.log_softmax(ref_logits.float(), -1).gather(-1, dtok_b[:, None])[:, 0]
+        assert float((dlp_b - lp_ref).abs().max()) <= 2e-2, "decode logprob vs the decoder oracle"
+        differ, total = sum(r["differ"] for r in report), sum(r["tokens"] for r in report)
+        assert differ <= 0.1 * total, f"routing differs on {differ} of {total} (token, layer) pairs"
+        # the cache the wrapper wrote is the oracle's cache (layer 0: embedding, norm, projection, rotary only)
+        got_k, want_k = store.key_cache[0].cpu().float(), kc[0].float()
+        pair = torch.sqrt(want_k[..., :64] ** 2 + want_k[..., 64:] ** 2).repeat(1, 1, 1, 2)
+        rel = ((got_k - want_k).abs() / pair.clamp(min=1e-3))
+        print(f"layer 0 key cache vs oracle: worst |d| / pair length {float(rel.max()):.4f}, "
+              f"{int((rel > 2.0 ** -7).sum())} of {rel.numel()} beyond 2^-7", flush=True)
+        assert bool(((got_k - want_k).abs() <= 2.0 ** -6 * pair + 1e-6).all()), "layer 0 key cache vs oracle"
+    finally:
+        remove_qwen3_moe_patches()
+        if had is None:
+            try:
+                del ALL_ATTENTION_FUNCTIONS._global_mapping["triton-invariant"]
+            except Exception:
+                pass
+        else:
+            ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had

@@ -45,7 +45,9 @@ def _randomise(model, seed):
                 p.copy_(0.5 + torch.rand(p.shape, generator=g))
             else:
                 p.copy_(0.08 * torch.randn(p.shape, generator=g))
-    return model.to(BF).eval()
+    for p in model.parameters():  # parameters only: a rotary embedding's inv_freq buffer stays fp32
+        p.data = p.data.to(BF)
+    return model.eval()
 
 
 def _layer_weights(layer):

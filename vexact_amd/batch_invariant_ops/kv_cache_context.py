@@ -160,7 +160,9 @@ class KVCacheStore:
     def __init__(self, hf_config, cache_config, device: torch.device):
         self.hf_config, self.cache_config, self.device = hf_config, cache_config, device
         self.page_size, self.max_blocks = cache_config.page_size, cache_config.max_cache_blocks
-        dtype = getattr(hf_config, "torch_dtype", None) or torch.bfloat16
+        dtype = getattr(hf_config, "dtype", None) or getattr(hf_config, "torch_dtype", None) or torch.bfloat16
+        if isinstance(dtype, str):  # configs read from JSON carry the name
+            dtype = getattr(torch, dtype.replace("torch.", ""))
         layers, heads = hf_config.num_hidden_layers, hf_config.num_key_value_heads
         slabs = [torch.zeros((layers, self.max_blocks, self.page_size, heads, d), device=device, dtype=dtype)
                  for d in _kv_head_dims(hf_config)]
