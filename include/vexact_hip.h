@@ -112,6 +112,13 @@ int vx_gemm_generic(const void* a, const void* b, const void* bias, void* c, int
                     int64_t M, int64_t N, int64_t K, int64_t sab, int64_t sam, int64_t sak,
                     int64_t sbb, int64_t sbk, int64_t sbn, int64_t scb, int64_t scm, int64_t scn,
                     hipStream_t stream);
+/* C[M,N] = X[M,K] * W[N,K]^T (+ bias[N]) for float32 (dtype 0; true fp32 products, v_mfma_f32_16x16x4_f32) and
+ * float16 (dtype 2; v_mfma_f32_16x16x32_f16): fp32 accumulate, K ascending, no split-K, one kernel and one tile
+ * shape for every M, so a row's bits do not depend on the other rows. Strides in elements, K contiguous.
+ * Replaces the fp16 / fp32 configurations of matmul_persistent, batch_invariant_ops.py:158-228 (tile table
+ * :182-206; the reference's fp32 tl.dot default is TF32 on its hardware, not copied). */
+int vx_gemm_nt_mfma(const void* x, const void* w, const void* bias, void* c, int dtype, int64_t M, int64_t N, int64_t K,
+                    int64_t ldx, int64_t ldw, int64_t ldc, hipStream_t stream);
 /* out[n, k] = in[k, n] (bf16) - packs a [K, N] row-major operand for vx_gemm_bf16_nt. */
 int vx_transpose_bf16(const void* in, void* out, int64_t K, int64_t N, int64_t ld_in, int64_t ld_out,
                       hipStream_t stream);

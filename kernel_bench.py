@@ -7,7 +7,7 @@ out, and the replay is timed with events. Prints time, algorithmic bytes (or flo
 fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
 to run under ``rocprofv3 --pmc``.
 
-    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,copy
+    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,other,configs,mfma,copy
 """
 
 from __future__ import annotations
@@ -388,6 +388,13 @@ def run(a, quiet: bool = False) -> list:
             report(f"C4 fused MoE T={T} ({U} experts)", t, U * 3 * H * I * 2 + 2 * T * H * 2 + T * k * 6)
             if T == 4096 and t is not None:
                 report(f"C4 fused MoE T={T}, as flops", t, flops=T * k * 6 * H * I)
+    if "other" in what:
+        # fp32 / fp16 matrix-core GEMM (one 64 x 64 x 32 tile shape for every M)
+        for dt, nm in ((torch.float32, "fp32"), (torch.float16, "fp16")):
+            for M in (256, 4096):
+                xx = torch.randn(M, 4096, generator=g, device=dev).to(dt)
+                ww = (torch.randn(4096, 4096, generator=g, device=dev) * 0.02).to(dt)
+                report(f"{nm} gemm M={M} N=4096 K=4096", timeit(lambda li: ops.matmul(xx, ww.t()), n_layers=2), flops=2 * M * 4096 * 4096)
     if "copy" in what:
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()

@@ -120,6 +120,45 @@ def test_other_dtypes_and_layouts(dtype, tol):
     assert_bf16_close(got2, O.matmul_ref(a2, b2), max_ulp=2, what="generic bf16")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("M,N,K,bias,linear_layout", [
+    (300, 520, 256, True, True),     # nn.Linear layout, vector loads
+    (65, 100, 100, False, False),    # row-major b (made K-contiguous), ragged everything
+    (130, 77, 1031, True, True),     # K not a multiple of the vector width: scalar loads
+    (1, 2048, 2048, False, True),
+])
+def test_fp32_fp16_matrix_core_gemm(dtype, M, N, K, bias, linear_layout):
+    # the fp16 / fp32 configurations of matmul_persistent (batch_invariant_ops.py:182-206): rows do not depend on the
+    # batch (0 bits), results against an fp64 product of the same inputs
+    a = _gen((M, K), 21, dtype)
+    w = _gen((N, K), 22, dtype, scale=0.1)
+    bv = _gen((N,), 23, dtype) if bias else None
+    ag, wg = a.cuda(), w.cuda()
+    bmat = wg.t() if linear_layout else wg.t().contiguous()
+    full = matmul_persistent(ag, bmat, bv.cuda() if bias else None)
+    assert full.dtype == dtype and full.shape == (M, N)
+    want = a.double() @ w.double().t() + (bv.double() if bias else 0.0)
+    err = (full.cpu().double() - want).abs().max().item()
+    scale = want.abs().max().item()
+    if dtype == torch.float32:
+        assert err <= 2e-6 * scale * (K ** 0.5), (err, scale)   # true fp32 products and sums
+        tf32_err = ((a.double() @ w.double().t()) * 2.0 ** -11).abs().max().item()
+        assert err < 0.1 * tf32_err, "fp32 GEMM must not run at TF32 precision"
+    else:
+        got, ref16 = full.cpu(), want.to(torch.float16)
+        ulp = (got.view(torch.int16).int() - ref16.view(torch.int16).int()).abs()
+        same_sign = (got.view(torch.int16).int() ^ ref16.view(torch.int16).int()) >= 0
+        assert bool(((ulp <= 2) & same_sign | ((got.double() - want).abs() <= 2e-3 * scale)).all()), "fp16 beyond 2 ulp"
+    for m in sorted({1, 7, 33, 64, 65, M} & set(range(1, M + 1))):
+        assert_bitwise(matmul_persistent(ag[:m], bmat, bv.cuda() if bias else None), full[:m], f"{dtype} first {m} rows")
+    if M > 40:
+        assert_bitwise(matmul_persistent(ag[37:40], bmat, bv.cuda() if bias else None), full[37:40], f"{dtype} rows 37..39 alone")
+    # under the aten overrides
+    with set_batch_invariant_mode(True):
+        via_aten = torch.mm(ag, bmat) if not bias else torch.addmm(bv.cuda(), ag, bmat)
+    assert_bitwise(via_aten, full, f"{dtype} through aten::mm / addmm")
+
+
 def test_aten_overrides_and_mode_switch():
     from vexact_amd.batch_invariant_ops import (
         disable_batch_invariant_mode,

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvexact_hip.so")
-SOURCES = ["row_ops.hip", "gemm.hip", "paged_attn.hip", "attn_bwd.hip", "moe.hip", "moe_bwd.hip", "glue.hip", "sampler.hip", "host_meta.cpp"]
+SOURCES = ["row_ops.hip", "gemm.hip", "gemm_other.hip", "paged_attn.hip", "attn_bwd.hip", "moe.hip", "moe_bwd.hip", "glue.hip", "sampler.hip", "host_meta.cpp"]
 HEADERS = ["common.h", "gemm_core.h", "gemm_wide.h"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -27,6 +27,7 @@ PROTOTYPES = {
     "vx_gemm_bf16_nt_variant": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _I, _P]),
     "vx_gemm_swiglu_bf16_nt": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _L, _L, _I, _I, _P]),
     "vx_gemm_generic": (_I, [_P, _P, _P, _P, _I] + [_L] * 13 + [_P]),
+    "vx_gemm_nt_mfma": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _P]),
     "vx_transpose_bf16": (_I, [_P, _P, _L, _L, _L, _L, _P]),
     "vx_store_kvcache": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _P]),
     "vx_attn_chunk_size": (_I, []),

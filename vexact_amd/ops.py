@@ -294,9 +294,9 @@ def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None
     """``a[M,K] @ b[K,N] (+ bias[N])`` with the dtype of ``a``; any strides.
 
     bf16 operands go through the MFMA kernels: directly when ``b`` is a transposed view of an
-    ``[N, K]`` row-major weight (the ``nn.Linear`` case), after packing ``b`` otherwise. Other dtypes
-    and unaligned layouts use the generic one-thread-per-output kernel. The choice depends on dtype
-    and layout only, never on M.
+    ``[N, K]`` row-major weight (the ``nn.Linear`` case), after packing ``b`` otherwise. fp16 and fp32
+    have an MFMA kernel of their own (true fp32 products for fp32). Unaligned bf16 layouts use the
+    generic one-thread-per-output kernel. The choice depends on dtype and layout only, never on M.
     """
     assert a.ndim == 2 and b.ndim == 2, "matmul expects 2-D operands"
     assert a.shape[1] == b.shape[0], "Incompatible dimensions"
@@ -334,6 +334,16 @@ def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None
             w_nk = packed
         if _fast_ok(x, w_nk):
             return gemm_nt(x, w_nk, bias, out=c)
+    if a.dtype in (torch.float32, torch.float16):
+        # matrix cores for these too: one kernel and tile shape for every M; operands made K-contiguous if needed
+        x = a if a.stride(1) == 1 else a.contiguous()
+        w_nk = b.t() if b.stride(0) == 1 else b.t().contiguous()
+        _lib.check(
+            lib.vx_gemm_nt_mfma(x.data_ptr(), w_nk.data_ptr(), _ptr(bias), c.data_ptr(), _DT[a.dtype], M, N, K,
+                                x.stride(0), w_nk.stride(0), c.stride(0), _stream()),
+            "vx_gemm_nt_mfma",
+        )
+        return c
     _lib.check(
         lib.vx_gemm_generic(
             a.data_ptr(), b.data_ptr(), _ptr(bias), c.data_ptr(), _DT[a.dtype], 1, M, N, K,
