@@ -32,7 +32,7 @@ def parse(argv=None):
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--layers", type=int, default=6, help="independent weight / cache copies to rotate over")
     ap.add_argument("--reps", type=int, default=5)
-    ap.add_argument("--kv-layout", default="head", choices=("head", "token"),
+    ap.add_argument("--kv-layout", default="head", choices=("head", "token", "fused"),
                     help="physical KV cache layout: [blocks, Hkv, page, D] (what the decoder allocates) or [blocks, page, Hkv, D]")
     ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
     ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
@@ -141,7 +141,11 @@ def run(a, quiet: bool = False) -> list:
         for s, p in enumerate(pages):
             bt[s, :p] = perm[o : o + p]
             o += p
-        if a.kv_layout == "head":
+        if a.kv_layout == "fused":  # one kv head's K page and V page adjacent: [blocks, Hkv, 2, page, D]
+            kv = [rnd(pool, Hkv, 2, page, D, std=1.0) for _ in range(NL)]
+            kc = [t[:, :, 0].permute(0, 2, 1, 3) for t in kv]
+            vc = [t[:, :, 1].permute(0, 2, 1, 3) for t in kv]
+        elif a.kv_layout == "head":
             kc = [rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3) for _ in range(NL)]
             vc = [rnd(pool, Hkv, page, D, std=1.0).permute(0, 2, 1, 3) for _ in range(NL)]
         else:

@@ -832,6 +832,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   // offset, which keeps 64-bit per-lane address arithmetic out of the loop.
   static_assert(KPW == 8, "a wavefront's keys must stay inside one 16-key tile");
   const int ld_tt = wave >> 1;
+  int pg_cache = 0, pg_base = -64;  // SRC_FAST: page ids of this wavefront's tile for blocks [pg_base, pg_base + 64), one per lane
   auto issue_block = [&](int kb, int stage) {
     const uint32_t dst0 = lds0 + stage * PFL_STAGE + KPW * wave * 256;
     if constexpr (KIND == SRC_GENERIC) {
@@ -855,7 +856,16 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
       const bf16_t *kt, *vt;
       if constexpr (KIND == SRC_FAST) {
         key0 = tile_key <= src.last ? tile_key : 0;
-        const int pg = src.bt[key0 >> src.shift];
+        // Page id of the wavefront's tile without a memory round trip per block: lane L keeps the id for block
+        // pg_base + L (one vector load per 64 blocks), and the block's id is read from its lane. Fetched per block
+        // it cost every wavefront an L2 latency between the barrier and its loads and MFMAs.
+        const int b = kb / ATT_BLOCK;
+        if (b - pg_base >= 64) {  // wave-uniform
+          pg_base = b;
+          const int tk = (b + lane) * ATT_BLOCK + 16 * ld_tt;
+          pg_cache = src.bt[(tk <= src.last ? tk : 0) >> src.shift];
+        }
+        const int pg = __builtin_amdgcn_readlane(pg_cache, b - pg_base);
         const int off = key0 & (src.ps - 1);
         kt = src.kbase + (int64_t)pg * src.skb + (int64_t)off * src.skp;
         vt = src.vbase + (int64_t)pg * src.svb + (int64_t)off * src.svp;
