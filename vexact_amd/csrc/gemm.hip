@@ -87,8 +87,11 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
     if (nt * ((M + 63) / 64) >= 256) mt = 4;
     else if (nt * ((M + 31) / 32) >= 256) mt = 2;
   }
-  // 65 .. 512 rows: the LDS ring kernel, whose loads do not wait on one wavefront's MFMA chain
-  if (mt != 0 && M > 64 && gemm_ring_auto(p, stream)) return launch_status();
+  // 65 .. 512 rows: the LDS ring kernel, whose loads do not wait on one wavefront's MFMA chain. Up to 64 rows
+  // too when the weight matrix is small (N <= 8192): the streaming kernel then has at most 128 workgroups of
+  // dependent loads (o projection at 16 rows: 20.0 us, ring 10.8 us; router 10.9 -> 5.8; equal near N = 16384,
+  // streaming ahead from N = 32768 on).
+  if (mt != 0 && (M > 64 || nt <= 128) && gemm_ring_auto(p, stream)) return launch_status();
   if (mt != 0) {
     const dim3 grid((unsigned)nt, (unsigned)((M + 16 * mt - 1) / (16 * mt)));
     if (mt == 1) gemm_stream_kernel<1, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);

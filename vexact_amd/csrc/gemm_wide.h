@@ -523,9 +523,10 @@ static inline bool gemm_ring_launch(const GemmParams& p, int shape, hipStream_t 
   }
 }
 
-// Picks the ring configuration for a decode-sized batch (measured on M = 128 .. 512 against the
-// qkv / o / router projections of the 30B-A3B shape): enough workgroups to occupy every CU first,
-// then the largest tile (least L2 -> LDS traffic), then fewer, longer steps when K allows.
+// Picks the ring configuration for a decode-sized batch (measured on M = 1 .. 512 against the
+// qkv / o / router projections of the 30B-A3B shape and N up to 8192): enough workgroups to occupy every CU
+// first, then the largest tile (least L2 -> LDS traffic), then fewer, longer steps when K allows. The 32x32
+// configuration holds 96 KB of LDS, so one workgroup per CU: past 256 of them the 32x64 one is faster.
 static inline bool gemm_ring_auto(const GemmParams& p, hipStream_t stream) {
   const int64_t m64 = (p.M + 63) / 64, m32 = (p.M + 31) / 32;
   const int64_t n64 = (p.N + 63) / 64, n32 = (p.N + 31) / 32;
@@ -535,8 +536,8 @@ static inline bool gemm_ring_auto(const GemmParams& p, hipStream_t stream) {
   else if (m64 * n64 >= 300) shape = k2 ? 1 : 0;
   else if (m64 * n64 >= 200) shape = k2 ? 2 : 0;
   else if (m32 * n64 >= 200) shape = k2 ? 3 : 5;
+  else if (m32 * n32 > 256 && m32 * n64 >= 128) shape = k2 ? 3 : 5;
   else shape = k4 ? 4 : 6;
-  (void)n32;
   return gemm_ring_launch(p, shape, stream);
 }
 
