@@ -32,7 +32,7 @@ def parse(argv=None):
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--layers", type=int, default=6, help="independent weight / cache copies to rotate over")
     ap.add_argument("--reps", type=int, default=5)
-    ap.add_argument("--kv-layout", default="head", choices=("head", "token", "fused"),
+    ap.add_argument("--kv-layout", default="fused", choices=("head", "token", "fused"),
                     help="physical KV cache layout: [blocks, Hkv, page, D] (what the decoder allocates) or [blocks, page, Hkv, D]")
     ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
     ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
