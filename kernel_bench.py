@@ -31,7 +31,9 @@ def parse(argv=None):
     ap.add_argument("--what", default="moe,attn,gemm,small")
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--layers", type=int, default=6, help="independent weight / cache copies to rotate over")
-    ap.add_argument("--reps", type=int, default=5)
+    ap.add_argument("--reps", type=int, default=5, help="timed graph replays (at least; see --min-ms)")
+    ap.add_argument("--settle-ms", type=float, default=40.0, help="untimed replays before the timed ones")
+    ap.add_argument("--min-ms", type=float, default=10.0, help="the timed replays cover at least this long")
     ap.add_argument("--kv-layout", default="fused", choices=("head", "token", "fused"),
                     help="physical KV cache layout: [blocks, Hkv, page, D] (what the decoder allocates) or [blocks, page, Hkv, D]")
     ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
@@ -54,6 +56,9 @@ def run(a, quiet: bool = False) -> list:
         return t
 
     def timeit(fn, n_layers=NL):
+        """Seconds per call of ``fn`` inside a captured graph of ``n_layers`` calls, at steady clocks: the graph is
+        replayed for ``--settle-ms`` first (after an idle spell this machine runs heavy kernels up to 25 % slower for
+        the first ~20 ms), then ``--reps`` replays, and more until they cover ``--min-ms``, are timed as one span."""
         for li in range(n_layers):
             fn(li)
         torch.cuda.synchronize()
@@ -63,17 +68,21 @@ def run(a, quiet: bool = False) -> list:
         with torch.cuda.graph(graph):
             for li in range(n_layers):
                 fn(li)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         graph.replay()
+        e1.record()
         torch.cuda.synchronize()
-        ts = []
-        for _ in range(a.reps):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
+        one = max(e0.elapsed_time(e1), 1e-3)  # ms per replay, first estimate
+        for _ in range(min(2000, int(a.settle_ms / one) + 1)):
             graph.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            ts.append(e0.elapsed_time(e1) * 1e-3 / n_layers)
-        return float(np.mean(ts))
+        reps = max(a.reps, min(2000, int(a.min_ms / one) + 1))
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / (reps * n_layers)
 
     def report(name, t, nbytes=None, flops=None):
         say = (lambda *x, **k: None) if quiet else print
@@ -95,9 +104,9 @@ def run(a, quiet: bool = False) -> list:
         seeds = torch.arange(B, dtype=torch.int64, device=dev) + 1234
         pos = torch.arange(B, dtype=torch.int64, device=dev) + 1000
         out = torch.empty(B, dtype=torch.int64, device=dev)
-        for name, k, p in (("plain", None, 1.0), ("top-p 0.9", None, 0.9), ("top-k 50", 50, 1.0), ("top-k 50 + top-p 0.9", 50, 0.9)):
+        for name, top_k, top_p in (("plain", None, 1.0), ("top-p 0.9", None, 0.9), ("top-k 50", 50, 1.0), ("top-k 50 + top-p 0.9", 50, 0.9)):
             report(f"sampler {name} (B={B}, V={V})",
-                   timeit(lambda li: ops.sample_tokens(lg, 0.8, k, p, seeds, pos, out=out), n_layers=4), B * V * 2)
+                   timeit(lambda li: ops.sample_tokens(lg, 0.8, top_k, top_p, seeds, pos, out=out), n_layers=4), B * V * 2)
         report("greedy argmax + logprob", timeit(lambda li: ops.logprobs(lg, None, return_tokens=True), n_layers=4), B * V * 2)
     if "moe" in what:
         x = rnd(B, H, std=1.0)
