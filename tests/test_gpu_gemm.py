@@ -51,6 +51,9 @@ def test_stream_and_tiled_kernels_agree_bitwise():
         (513, 1023, 192, False),  # row stride of C not a multiple of 8 -> scalar stores
         (4352, 4096, 128, False),  # 272 tiles on 256 workgroups: some walk a second tile
         (2048, 5120, 2048, True),  # qkv-projection shape of a prefill chunk
+        (2000, 10240, 128, True),  # 8 x 40 tiles: columns from 8192 on go to 128-row tiles (ragged last row tile)
+        (256, 152000, 64, False),  # 594 column tiles: the last 82 go to 128-row tiles (ragged last column tile)
+        (8192, 5120, 64, True),  # 32 x 20 tiles: two rounds of 256-row tiles and one of 128-row tiles
     ],
 )
 def test_wide_kernel_agrees_bitwise(M, N, K, bias):
@@ -63,7 +66,8 @@ def test_wide_kernel_agrees_bitwise(M, N, K, bias):
     if M * N >= 128 * 65536:  # the default entry point picks the wide kernel here
         full = ops.gemm_nt(ag, wg, bias=bg)
         assert_bitwise(full, ref, "dispatch vs tiled")
-        assert_bitwise(ops.gemm_nt(ag[1000:1003], wg, bias=bg), full[1000:1003], "3 rows alone vs inside a chunk")
+        r0 = min(1000, M // 2)
+        assert_bitwise(ops.gemm_nt(ag[r0 : r0 + 3], wg, bias=bg), full[r0 : r0 + 3], "3 rows alone vs inside a chunk")
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 640, 2048), (100, 200, 64), (77, 333, 192), (130, 70, 320), (512, 128, 768),

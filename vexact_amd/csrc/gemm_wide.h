@@ -36,9 +36,6 @@
 namespace vx {
 
 constexpr int WD_BM = 256, WD_BN = 256, WD_BK = 64;
-constexpr int WD_XBYTES = WD_BM * WD_BK * 2;             // 32 KB
-constexpr int WD_STAGE = (WD_BM + WD_BN) * WD_BK * 2;    // 64 KB
-constexpr int WD_LDS = 2 * WD_STAGE;                     // 128 KB
 constexpr int WD_GROUP_M = 4;
 
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -63,10 +60,18 @@ struct WideTile {
 // fragments 0, 1 and the matching up columns in fragments 2, 3: LDS row 64 wn + 16 a + 4 j + b is
 // column 32 wn + 8 a + 4 (j & 1) + b of gate (j < 2) or up (j >= 2). A tile then yields 128 output
 // columns and a lane 8 consecutive ones per activation row.
-template <int EPI, bool GROUPED>
+// XI = 16-row activation tiles per wavefront: 8 (256-row tiles, the normal form) or 4 (128-row tiles: the same
+// weight panel and barriers for half the rows, for a last round of tiles that would leave half the chip idle).
+template <int EPI, bool GROUPED, int XI = 8>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t wd_lds[];
   constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;  // output columns per tile
+  constexpr int BM = 32 * XI;                             // activation rows per tile
+  constexpr int NXQ = BM / 64;                            // activation load instructions per wavefront and step
+  constexpr int NLQ = NXQ + 4;                            // all load instructions per wavefront and step
+  constexpr int XBYTES = BM * WD_BK * 2;
+  constexpr int STAGE = XBYTES + WD_BN * WD_BK * 2;
+  static_assert(XI == 8 || XI == 4, "wavefront tile heights");
 
   const int N = p.N, K = p.K;
   const int tiles = tiles_m * tiles_n;
@@ -89,8 +94,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
       const int gm0 = grp * WD_GROUP_M;
       const int gsz = min(WD_GROUP_M, tiles_m - gm0);
       const int rem = lin - grp * span;
-      t.row0 = (gm0 + rem % gsz) * WD_BM;
-      t.rows = min(WD_BM, p.M - t.row0);
+      t.row0 = (gm0 + rem % gsz) * BM;
+      t.rows = min(BM, p.M - t.row0);
       t.n0 = (rem / gsz) * NOUT;
       t.wbase = 0;
       t.ok = true;
@@ -104,23 +109,25 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   const int r16 = lane & 15, g = lane >> 4;
   const int wm = wave >> 2, wn = wave & 3;
 
-  // ---- load stream: instruction q of a step fills tile rows [8 (wave + 8 (q & 3)), +8) of X (q < 4)
-  // or W (q >= 4). Byte offsets from the operand base fit 32 bits (host check).
+  // ---- load stream: instruction q of a step fills tile rows [8 (wave + 8 q), +8) of X (q < NXQ)
+  // or rows [8 (wave + 8 (q - NXQ)), +8) of W. Byte offsets from the operand base fit 32 bits (host check).
   const int lrow = lane >> 3, lslot = lane & 7;
-  uint32_t ld_off[8];
+  uint32_t ld_off[NLQ];
   int64_t ld_wbase = 0;
   auto set_load_tile = [&](const WideTile& t) {
     ld_wbase = t.wbase;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int R = 8 * (wave + 8 * j) + lrow;
-      const int rr = t.row0 + min(R, t.rows - 1);  // rows past the tile re-read its last row (not stored)
-      const int64_t sr = (GROUPED && p.row_src) ? (int64_t)p.row_src[rr] : (int64_t)rr;
-      ld_off[j] = (uint32_t)((sr * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
+      if (j < NXQ) {
+        const int rr = t.row0 + min(R, t.rows - 1);  // rows past the tile re-read its last row (not stored)
+        const int64_t sr = (GROUPED && p.row_src) ? (int64_t)p.row_src[rr] : (int64_t)rr;
+        ld_off[j] = (uint32_t)((sr * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
+      }
       int col;
       if constexpr (EPI == EPI_SWIGLU) col = t.n0 + 32 * (R >> 6) + 8 * ((R >> 4) & 3) + 4 * ((R >> 2) & 1) + (R & 3);
       else col = t.n0 + R;
-      ld_off[4 + j] = (uint32_t)(((int64_t)min(col, N - 1) * p.ldw + (lslot ^ wd_swz_w(R)) * 8) * 2);
+      ld_off[NXQ + j] = (uint32_t)(((int64_t)min(col, N - 1) * p.ldw + (lslot ^ wd_swz_w(R)) * 8) * 2);
     }
   };
   int ld_lin = first, ld_k = 0;
@@ -133,8 +140,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   // it would wait for them (vmcnt(0)) before the first fragment read after they are issued. The
   // wait that matters is the explicit one before the barrier that precedes their first use.
   auto issue_one = [&](int q, int stage) {
-    const uint32_t dst = lds0 + stage * WD_STAGE + (q >> 2) * WD_XBYTES + (q & 3) * 8192;
-    const bf16_t* base = (q < 4 ? p.x : wsrc + ld_wbase) + ld_k;
+    const uint32_t dst = lds0 + stage * STAGE + (q < NXQ ? q * 8192 : XBYTES + (q - NXQ) * 8192);
+    const bf16_t* base = (q < NXQ ? p.x : wsrc + ld_wbase) + ld_k;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
   };
@@ -153,39 +160,39 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
     }
   };
 
-  f32x4 acc[8][4];  // [activation tile i][weight tile j]
+  f32x4 acc[XI][4];  // [activation tile i][weight tile j]
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int i = 0; i < XI; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // ---- fragment reads, k-half 0; k-half 1 is the same address with bit 6 flipped (slot ^ 4).
-  // Activation rows 128 wm + 16 i + r16: swizzle term r16 >> 1. Weight rows
+  // Activation rows 16 XI wm + 16 i + r16: swizzle term r16 >> 1. Weight rows
   // 64 wn + 16 (r16 / 4) + 4 j + r16 % 4: swizzle term 2 (r16 / 4) + (r16 % 4) / 2.
-  const int xoff = (128 * wm + r16) * 128 + ((g ^ (r16 >> 1)) * 16);
-  const int woff = WD_XBYTES + (64 * wn + 16 * (r16 >> 2) + (r16 & 3)) * 128 +
+  const int xoff = (16 * XI * wm + r16) * 128 + ((g ^ (r16 >> 1)) * 16);
+  const int woff = XBYTES + (64 * wn + 16 * (r16 >> 2) + (r16 & 3)) * 128 +
                    ((g ^ (((r16 >> 2) << 1) | ((r16 >> 1) & 1))) * 16);
-  struct Frag { uint4 w[4], x[8]; };
-  // read number r (0..11) of a fragment set: the 4 weight operands first, then the 8 activation ones
+  struct Frag { uint4 w[4], x[XI]; };
+  // read number r (0 .. 3 + XI) of a fragment set: the 4 weight operands first, then the XI activation ones
   auto read_one = [&](Frag& f, int r, const uint8_t* sb, int ks) {
     if (r < 4) f.w[r] = *(const uint4*)(sb + (woff ^ (64 * ks)) + r * 512);
     else f.x[r - 4] = *(const uint4*)(sb + (xoff ^ (64 * ks)) + (r - 4) * 2048);
   };
-  // 32 MFMAs on `cur`, interleaved with the 12 reads of `nxt` and (LOADS) the 8 global loads of a step
+  // 4 XI MFMAs on `cur`, interleaved with the 4 + XI reads of `nxt` and (LOADS) the global loads of a step
   auto half_step = [&](const Frag& cur, Frag& nxt, const uint8_t* nxt_sb, int nxt_ks, auto LOADS,
                        int ld_stage) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < XI; i++) {
 #pragma unroll
       for (int j = 0; j < 4; j++) acc[i][j] = mfma16(cur.w[j], cur.x[i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (decltype(LOADS)::value) {
-        if (i < 4) {
+        if (2 * i < NLQ) {
           issue_one(2 * i, ld_stage);
           issue_one(2 * i + 1, ld_stage);
         }
       }
-      if (i < 4) {
+      if (i < 4) {  // two reads beside each of the first four MFMA groups, one beside the others (XI = 8)
         read_one(nxt, 2 * i, nxt_sb, nxt_ks);
         read_one(nxt, 2 * i + 1, nxt_sb, nxt_ks);
       } else {
@@ -198,15 +205,15 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   const int nk = K / WD_BK;
   Frag f0, f1;
 #pragma unroll
-  for (int q = 0; q < 8; q++) issue_one(q, 0);
+  for (int q = 0; q < NLQ; q++) issue_one(q, 0);
   advance_loads();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 #pragma unroll
-  for (int q = 0; q < 8; q++) issue_one(q, 1);
+  for (int q = 0; q < NLQ; q++) issue_one(q, 1);
   advance_loads();
 #pragma unroll
-  for (int r = 0; r < 12; r++) read_one(f0, r, wd_lds, 0);
+  for (int r = 0; r < 4 + XI; r++) read_one(f0, r, wd_lds, 0);
 
   int st = 0;  // stage of the current step
   const bool vec_ok = (p.ldc & 7) == 0 && ((uintptr_t)p.c & 15) == 0;
@@ -214,8 +221,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
     const WideTile t = tile_at(lin);
     if (!t.ok) break;
     for (int kt = 0; kt < nk; kt++) {
-      const uint8_t* cur_sb = wd_lds + st * WD_STAGE;
-      const uint8_t* oth_sb = wd_lds + (st ^ 1) * WD_STAGE;
+      const uint8_t* cur_sb = wd_lds + st * STAGE;
+      const uint8_t* oth_sb = wd_lds + (st ^ 1) * STAGE;
       half_step(f0, f1, cur_sb, 1, std::false_type{}, 0);
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __syncthreads();  // the next step has landed everywhere; this stage has been read by everyone
@@ -229,8 +236,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
       // lane holds gate (fragments 0, 1) and up (2, 3) of columns n0 + 32 wn + 8 g + 4 j + c
       const int nb = t.n0 + 32 * wn + 8 * g;
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const int m = 128 * wm + 16 * i + r16;
+      for (int i = 0; i < XI; i++) {
+        const int m = 16 * XI * wm + 16 * i + r16;
         float wr = 0.f;
         if (m < t.rows) {
           const int64_t orow = t.row0 + m;
@@ -261,7 +268,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
         }
       }
     } else {
-      // lane holds C[row0 + 128 wm + 16 i + r16][n0 + 64 wn + 16 g + 4 j + c]
+      // lane holds C[row0 + 16 XI wm + 16 i + r16][n0 + 64 wn + 16 g + 4 j + c]
       const int nb = t.n0 + 64 * wn + 16 * g;
       float bv[16];
       if (p.bias) {
@@ -269,8 +276,8 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
         for (int e = 0; e < 16; e++) bv[e] = bf16_to_f32(p.bias[min(nb + e, N - 1)]);
       }
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const int m = 128 * wm + 16 * i + r16;
+      for (int i = 0; i < XI; i++) {
+        const int m = 16 * XI * wm + 16 * i + r16;
         bf16_t o[16];
 #pragma unroll
         for (int j = 0; j < 4; j++)
@@ -306,9 +313,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
 
 // Launch helper shared by the dense and the grouped entry points. x_rows = rows addressable in x
 // (bounds the 32-bit load offsets). Returns false (nothing launched) when the shape does not qualify.
-template <int EPI, bool GROUPED>
+template <int EPI, bool GROUPED, int XI = 8>
 static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int64_t x_rows, hipStream_t stream) {
   constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;
+  constexpr int LDS = 2 * (32 * XI + WD_BN) * WD_BK * 2;  // two stages of an activation and a weight tile
   if (p.K % WD_BK != 0 || p.N <= 0 || tiles_m <= 0 || x_rows <= 0) return false;
   const int64_t lim = (int64_t)1 << 32;
   if ((x_rows * p.ldx + p.K) * 2 >= lim || ((int64_t)p.N * p.ldw + p.K) * 2 >= lim) return false;
@@ -317,22 +325,48 @@ static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int6
   if (tiles > (1 << 30)) return false;
   static bool attr_set = false;  // per process and instantiation; a property of the loaded function
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, GROUPED>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, WD_LDS) != hipSuccess) {
+    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, GROUPED, XI>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
     attr_set = true;
   }
   const unsigned grid = (unsigned)(tiles >= 256 ? 256 : (tiles + 7) / 8 * 8);
-  gemm_wide_kernel<EPI, GROUPED><<<grid, 512, WD_LDS, stream>>>(p, (int)tiles_m, (int)tn);
+  gemm_wide_kernel<EPI, GROUPED, XI><<<grid, 512, LDS, stream>>>(p, (int)tiles_m, (int)tn);
   return true;
+}
+
+// Columns [0, n1) of a dense product go to 256-row tiles and [n1, N) to 128-row tiles when the 256 x 256 tiles'
+// last round would fill at most half of the 256 workgroups (640 tiles: two rounds of 256-row tiles over the
+// first 512, then one round of 256 half-height tiles instead of a third round on 128 workgroups). A half-height
+// tile pays the whole weight panel and every barrier for half the rows (measured ~0.7 of a full tile), so only
+// such a last round gains: the q/k/v projection of an 8192-token chunk 154 -> 147 us. With few row tiles the
+// kernel streams weights from HBM and a half-height tile costs what a full one does (lm_head at 256 rows:
+// 206 us either way), so those shapes are left alone. Returns N when there is nothing to split.
+static inline int64_t gemm_wide_split_col(int64_t M, int64_t N, int nout) {
+  const int64_t tm = (M + WD_BM - 1) / WD_BM, tn = (N + nout - 1) / nout;
+  const int64_t rem = (tm * tn) % 256;
+  if (tm < 4 || tm * tn < 256 || rem == 0 || rem > 128) return N;
+  // the fewest trailing column tiles whose removal leaves whole rounds
+  for (int64_t cut = 1; cut < tn && tm * cut <= 128; cut++)
+    if ((tm * (tn - cut)) % 256 == 0) return (tn - cut) * nout;
+  return N;
 }
 
 // dense: C[M, N] = X W^T (+ bias)
 static inline bool gemm_wide_launch(const GemmParams& p, hipStream_t stream) {
   if (p.M <= 0) return false;
-  return gemm_wide_launch_t<EPI_PLAIN, false>(p, ((int64_t)p.M + WD_BM - 1) / WD_BM, p.M, stream);
+  const int64_t n1 = gemm_wide_split_col(p.M, p.N, WD_BN);
+  if (n1 == p.N) return gemm_wide_launch_t<EPI_PLAIN, false>(p, ((int64_t)p.M + WD_BM - 1) / WD_BM, p.M, stream);
+  GemmParams a = p, b = p;
+  a.N = (int)n1;
+  b.N = p.N - (int)n1;
+  b.w = p.w + n1 * p.ldw;
+  b.c = p.c + n1;
+  if (p.bias) b.bias = p.bias + n1;
+  if (!gemm_wide_launch_t<EPI_PLAIN, false>(a, ((int64_t)p.M + WD_BM - 1) / WD_BM, p.M, stream)) return false;
+  return gemm_wide_launch_t<EPI_PLAIN, false, 4>(b, ((int64_t)p.M + 127) / 128, p.M, stream);
 }
 
 // dense with the SwiGLU epilogue: C[M, N] = swiglu(X Wg^T, X Wu^T)
