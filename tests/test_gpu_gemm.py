@@ -70,6 +70,27 @@ def test_wide_kernel_agrees_bitwise(M, N, K, bias):
         assert_bitwise(ops.gemm_nt(ag[r0 : r0 + 3], wg, bias=bg), full[r0 : r0 + 3], "3 rows alone vs inside a chunk")
 
 
+def test_dispatch_agrees_with_the_tiled_kernel_on_random_shapes():
+    # whatever kernel the shape-based dispatch picks (streaming, ring at 1..512 rows, 128 x 128 tiles, 256 x 256
+    # tiles with or without a half-height last round), the bits are those of the 128 x 128 tiled kernel, with
+    # strided operands and a bias as well
+    g = torch.Generator().manual_seed(77)
+    def pick(choices):
+        return choices[int(torch.randint(0, len(choices), (1,), generator=g))]
+    shapes = [(1, 2048, 4096), (16, 128, 2048), (48, 5120, 2048), (64, 8192, 256), (64, 8256, 256), (33, 1000, 192),
+              (65, 136, 72), (300, 5120, 64), (2304, 7168, 64), (1100, 10240, 128)]
+    for _ in range(14):
+        shapes.append((int(torch.randint(1, 700, (1,), generator=g)), 8 * int(torch.randint(1, 1200, (1,), generator=g)),
+                       pick([64, 72, 128, 192, 256, 320, 1024, 2048])))
+    for i, (M, N, K) in enumerate(shapes):
+        pad_x, pad_w = pick([0, 8, 64]), pick([0, 8, 64])
+        a = _gen((M, K + pad_x), 100 + i)[:, :K].cuda()
+        w = _gen((N, K + pad_w), 200 + i, scale=0.05)[:, :K].cuda()
+        bias = _gen((N,), 300 + i).cuda() if i % 2 else None
+        ref = ops.gemm_nt_variant(a.contiguous(), w.contiguous(), kind=1, bias=bias)
+        assert_bitwise(ops.gemm_nt(a, w, bias=bias), ref, f"dispatch vs tiled, {M}x{N}x{K}, row pads {pad_x}/{pad_w}")
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 640, 2048), (100, 200, 64), (77, 333, 192), (130, 70, 320), (512, 128, 768),
                                    (3000, 128, 512)])  # the last: many rows, few columns -> ring by dispatch
 def test_ring_kernel_agrees_bitwise(M, N, K):
