@@ -439,12 +439,10 @@ def other_configs():
     events (kernel_bench.py): C1 op chain at M = 1 / 7 / 64, C2 decode attention, C3 chunked prefill attention,
     C4 fused MoE block at T = 1 / 64 / 256 / 4096, and the q/k/v projection of an 8192-token prefill chunk.
     Each line carries its algorithmic bytes or flops and the fraction of the HBM / bf16 MFMA peak."""
-    import argparse as _ap
-
     import kernel_bench
 
-    res = kernel_bench.run(_ap.Namespace(what=["configs", "mfma"], batch=256, layers=2, reps=3, kv_layout="head", page=16,
-                                         nograph=False), quiet=True)
+    res = kernel_bench.run(kernel_bench.parse(["--what", "configs,mfma", "--batch", "256", "--layers", "2", "--reps", "3"]),
+                           quiet=True)
     mfma = [r for r in res if r["bound"] == "mfma"]
     return res, mfma
 

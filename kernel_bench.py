@@ -35,7 +35,7 @@ def parse(argv=None):
     ap.add_argument("--settle-ms", type=float, default=40.0, help="untimed replays before the timed ones")
     ap.add_argument("--min-ms", type=float, default=10.0, help="the timed replays cover at least this long")
     ap.add_argument("--kv-layout", default="fused", choices=("head", "token", "fused"),
-                    help="physical KV cache layout: [blocks, Hkv, page, D] (what the decoder allocates) or [blocks, page, Hkv, D]")
+                    help="physical KV cache layout: fused = [blocks, Hkv, 2, page, D] (what the decoder allocates), head = [blocks, Hkv, page, D] per tensor, token = [blocks, page, Hkv, D]")
     ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
     ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
     return ap.parse_args(argv)
