@@ -267,3 +267,24 @@ def test_bench_refuses_more_than_one_gpu():
     res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert res.returncode == 2
     assert "exactly one GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_bench_hands_kernel_bench_every_option_it_reads():
+    # bench.py's `configs` block runs kernel_bench.run() in-process: the arguments it builds must carry every
+    # option that run() reads, or the driver's bench dies after the decode step has been measured
+    import inspect
+    import os
+    import re
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, root)
+    import bench
+    import kernel_bench
+
+    call = re.search(r"kernel_bench\.parse\((\[.*?\])\)", inspect.getsource(bench.other_configs), re.S)
+    assert call, "other_configs must build its arguments with kernel_bench.parse"
+    args = kernel_bench.parse(eval(call.group(1)))
+    read = set(re.findall(r"\ba\.([a-z_]+)\b", inspect.getsource(kernel_bench.run)))
+    assert read and all(hasattr(args, name) for name in read), sorted(n for n in read if not hasattr(args, n))
+    assert "configs" in args.what and "mfma" in args.what
