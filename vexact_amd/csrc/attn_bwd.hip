@@ -588,13 +588,14 @@ template <int D>
 static int launch_attn_bwd(const AttnBwdParams& p, int64_t total_q, int num_seqs, int max_q, int max_k, hipStream_t stream) {
   attn_bwd_delta_kernel<D><<<(unsigned)((total_q * p.Hq + 15) / 16), 256, 0, stream>>>(p, total_q);
   if constexpr (D == 128) {
-    static bool attr_set = false;
-    if (!attr_set) {
+    static DeviceOnce once;
+    const int dev = once.slot();
+    if (once.need(dev)) {
       if (hipFuncSetAttribute((const void*)attn_bwd_dq_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, BWL_LDS) != hipSuccess) {
         (void)hipGetLastError();
         return VX_ERR_LAUNCH;
       }
-      attr_set = true;
+      once.mark(dev);
     }
     attn_bwd_dq_lds_kernel<<<dim3((unsigned)((max_q + 16 * BWL_WAVES - 1) / (16 * BWL_WAVES)), (unsigned)p.Hq, (unsigned)num_seqs),
                              64 * BWL_WAVES, BWL_LDS, stream>>>(p);
@@ -602,13 +603,14 @@ static int launch_attn_bwd(const AttnBwdParams& p, int64_t total_q, int num_seqs
     attn_bwd_dq_kernel<D><<<dim3((unsigned)((max_q + 63) / 64), (unsigned)p.Hq, (unsigned)num_seqs), 256, 0, stream>>>(p);
   }
   if constexpr (D == 128) {
-    static bool attr_set2 = false;
-    if (!attr_set2) {
+    static DeviceOnce once;
+    const int dev = once.slot();
+    if (once.need(dev)) {
       if (hipFuncSetAttribute((const void*)attn_bwd_dkv_lds_kernel<BWK_WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, BWK_LDS) != hipSuccess) {
         (void)hipGetLastError();
         return VX_ERR_LAUNCH;
       }
-      attr_set2 = true;
+      once.mark(dev);
     }
     attn_bwd_dkv_lds_kernel<BWK_WAVES><<<dim3((unsigned)((max_k + 16 * BWK_WAVES - 1) / (16 * BWK_WAVES)), (unsigned)p.Hkv, (unsigned)num_seqs),
                                          64 * BWK_WAVES, BWK_LDS, stream>>>(p);

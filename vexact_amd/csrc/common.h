@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace vx {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -16,6 +18,20 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef uint16_t bf16_t;  // storage type in global memory
 
 constexpr int kWave = 64;
+
+// "Done once per device" flag for host code that raises a kernel's dynamic-LDS limit before its first launch: the
+// attribute belongs to the function as loaded on one device, and several host threads may launch the same kernel.
+// slot() is the current device's index (-1 if it cannot be tracked: the caller then repeats the set-up each time).
+struct DeviceOnce {
+  std::atomic<unsigned char> done[64] = {};
+  int slot() const {
+    int d = -1;
+    if (hipGetDevice(&d) != hipSuccess || d < 0 || d >= 64) return -1;
+    return d;
+  }
+  bool need(int d) const { return d < 0 || !done[d].load(std::memory_order_acquire); }
+  void mark(int d) { if (d >= 0) done[d].store(1, std::memory_order_release); }
+};
 
 // Status codes returned over the C ABI.
 enum : int {

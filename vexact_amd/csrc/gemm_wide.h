@@ -323,14 +323,15 @@ static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int6
   const int64_t tn = ((int64_t)p.N + NOUT - 1) / NOUT;
   const int64_t tiles = tiles_m * tn;
   if (tiles > (1 << 30)) return false;
-  static bool attr_set = false;  // per process and instantiation; a property of the loaded function
-  if (!attr_set) {
+  static DeviceOnce once;  // per instantiation
+  const int dev = once.slot();
+  if (once.need(dev)) {
     if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, GROUPED, XI>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
-    attr_set = true;
+    once.mark(dev);
   }
   const unsigned grid = (unsigned)(tiles >= 256 ? 256 : (tiles + 7) / 8 * 8);
   gemm_wide_kernel<EPI, GROUPED, XI><<<grid, 512, LDS, stream>>>(p, (int)tiles_m, (int)tn);
@@ -524,14 +525,15 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmParams p) {
 template <int XF, int WF, int S, int KSUB>
 static inline bool gemm_ring_launch_t(const GemmParams& p, hipStream_t stream) {
   constexpr int BM = 32 * XF, BN = 32 * WF, LDS = S * KSUB * (BM + BN) * 128;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static DeviceOnce once;
+  const int dev = once.slot();
+  if (once.need(dev)) {
     if (hipFuncSetAttribute((const void*)gemm_ring_kernel<XF, WF, S, KSUB>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
       (void)hipGetLastError();
       return false;
     }
-    attr_set = true;
+    once.mark(dev);
   }
   const int64_t gy = ((int64_t)p.M + BM - 1) / BM, gx = ((int64_t)p.N + BN - 1) / BN;
   if (gy > 65535 || gx > 0x7fffffffLL || p.K % (64 * KSUB) != 0) return false;

@@ -1060,14 +1060,15 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
 #define VX_FUSED(KERNEL, QTV, KINDV, NW)                                                             \
   do {                                                                                             \
     constexpr int LDSB = fused_lds_bytes<DV, QTV, NW>();                                           \
-    static bool attr_set = false;                                                                  \
-    if (!attr_set) {                                                                               \
+    static DeviceOnce once;                                                                        \
+    const int dev = once.slot();                                                                   \
+    if (once.need(dev)) {                                                                          \
       if (hipFuncSetAttribute((const void*)KERNEL<DK, DV, QTV, KINDV, NW>,                         \
                               hipFuncAttributeMaxDynamicSharedMemorySize, LDSB) != hipSuccess) {   \
         (void)hipGetLastError();                                                                   \
         return VX_ERR_LAUNCH;                                                                      \
       }                                                                                            \
-      attr_set = true;                                                                             \
+      once.mark(dev);                                                                              \
     }                                                                                              \
     KERNEL<DK, DV, QTV, KINDV, NW><<<grid, 64 * NW, LDSB, stream>>>(p);                            \
   } while (0)
@@ -1123,15 +1124,16 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
       while (hp * 2 <= 8 && G % (hp * 2) == 0) hp *= 2;
       const int rb = 16 * (PFL_SLOTS / hp);
       const dim3 lgrid((rows + rb - 1) / rb, p.Hq / hp, p.num_seqs);
-      static bool attr_set = false;
-      if (!attr_set) {
+      static DeviceOnce once;
+      const int dev = once.slot();
+      if (once.need(dev)) {
         if (hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<SRC_PACKED>, hipFuncAttributeMaxDynamicSharedMemorySize, PFL_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<SRC_FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, PFL_LDS) != hipSuccess ||
             hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<SRC_GENERIC>, hipFuncAttributeMaxDynamicSharedMemorySize, PFL_LDS) != hipSuccess) {
           (void)hipGetLastError();
           return VX_ERR_LAUNCH;
         }
-        attr_set = true;
+        once.mark(dev);
       }
       if (mode == 2) attn_prefill_lds_kernel<SRC_PACKED><<<lgrid, 64 * PFL_WAVES, PFL_LDS, stream>>>(p, hp);
       else if (fast) attn_prefill_lds_kernel<SRC_FAST><<<lgrid, 64 * PFL_WAVES, PFL_LDS, stream>>>(p, hp);
