@@ -116,6 +116,32 @@ def test_log_softmax_3d_and_bf16():
     torch.testing.assert_close(gb.float(), torch.log_softmax(xb.float(), -1), atol=6e-2, rtol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_log_softmax_and_logprobs_on_ragged_and_unaligned_rows(dtype):
+    # rows that start at any element offset (column slices of a wider tensor) and lengths that are no multiple of
+    # the 4-element vectors: the vector and the element-wise form of the loads must give the same bits
+    wide = _gen((9, 9000), 21, dtype, scale=2.5).cuda()
+    g = torch.Generator().manual_seed(22)
+    for n in (8192, 8190, 4097, 4099, 5, 3):
+        labels = torch.randint(0, n, (9,), generator=g).cuda()
+        base = wide[:, :n].contiguous()
+        want_ls = ops.log_softmax(base, -1)
+        want_lp, want_tok = ops.logprobs(base, None, return_tokens=True)
+        want_lab = ops.logprobs(base, labels)
+        if dtype == torch.float32:
+            torch.testing.assert_close(want_ls.cpu(), torch.log_softmax(base.cpu(), -1), atol=2e-5, rtol=0)
+        for off in (1, 2, 3, 4):
+            view = wide[:, off : off + n]
+            shifted = wide.clone()
+            shifted[:, off : off + n] = wide[:, :n]
+            view = shifted[:, off : off + n]  # same values as `base`, rows starting `off` elements into the pitch
+            assert_bitwise(ops.log_softmax(view, -1), want_ls, f"log_softmax n={n} offset {off}")
+            lp, tok = ops.logprobs(view, None, return_tokens=True)
+            assert_bitwise(lp, want_lp, f"greedy logprob n={n} offset {off}")
+            assert torch.equal(tok, want_tok)
+            assert_bitwise(ops.logprobs(view, labels), want_lab, f"label logprob n={n} offset {off}")
+
+
 @pytest.mark.parametrize("vocab", [1000, 151936])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_logprobs_value_and_permutation_invariance(vocab, dtype):

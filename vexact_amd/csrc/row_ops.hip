@@ -227,14 +227,31 @@ struct LsPartial {
   int pad;
 };
 
+// four consecutive elements at p: one 16- or 8-byte access when `vec` (p is aligned to the four elements and all
+// four lie inside the row), element by element otherwise; same values either way
+template <int DT>
+__device__ __forceinline__ void ls_load4(const typename Elem<DT>::T* p, int left, bool vec, float* v) {
+  using T = typename Elem<DT>::T;
+  if (vec) {
+    __attribute__((aligned(16))) T t[4];
+    if constexpr (sizeof(T) == 4) *(uint4*)t = *(const uint4*)p;
+    else *(uint2*)t = *(const uint2*)p;
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[c] = Elem<DT>::ld(t + c);
+  } else {
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[c] = (c < left) ? Elem<DT>::ld(p + c) : -INFINITY;
+  }
+}
+
 template <int DT>
 __device__ __forceinline__ void ls_load(const typename Elem<DT>::T* row, int n, int c0, float* v) {
   // thread t owns vectors t, t+256, t+512, t+768 of the chunk (4 elements each)
+  const bool aligned = ((uintptr_t)row % (4 * sizeof(typename Elem<DT>::T))) == 0;  // chunk and vector starts are multiples of 4
 #pragma unroll
   for (int j = 0; j < LS_PER / 4; j++) {
     const int e0 = c0 + 4 * (threadIdx.x + LS_THREADS * j);
-#pragma unroll
-    for (int c = 0; c < 4; c++) v[4 * j + c] = (e0 + c < n) ? Elem<DT>::ld(row + e0 + c) : -INFINITY;
+    ls_load4<DT>(row + e0, n - e0, aligned && e0 + 3 < n, v + 4 * j);
   }
 }
 
@@ -276,14 +293,35 @@ __global__ __launch_bounds__(LS_THREADS) void ls_partial_kernel(
   }
 }
 
-__device__ __forceinline__ void ls_fold(const LsPartial* __restrict__ p, int nchunk, float& m,
-                                        float& logS, int& amax) {
-  m = p[0].m;
-  amax = p[0].idx;
-  for (int c = 1; c < nchunk; c++)
-    if (p[c].m > m) { m = p[c].m; amax = p[c].idx; }
+// Folds a row's chunk partials: m = max_c m_c (amax = index stored with the first chunk that attains it),
+// S = sum over ascending c of s_c * exp(m_c - m), logS = log S. One wavefront does it together: lane l takes chunks
+// l, l + 64, ... for the maximum and the terms, and the terms are then added one by one in ascending chunk order
+// (every lane carries the same running sum), so the result is the sequential sum, bit for bit, at 1/64 of its
+// exponentials per lane. All 64 lanes of the calling wavefront must be active.
+__device__ __forceinline__ void ls_fold_wave(const LsPartial* __restrict__ p, int nchunk, float& m,
+                                             float& logS, int& amax) {
+  const int lane = threadIdx.x & 63;
+  float bm = -INFINITY;
+  int bc = 0x7fffffff;  // first chunk attaining bm among this lane's chunks
+  for (int c = lane; c < nchunk; c += 64) {
+    const float v = p[c].m;
+    if (v > bm || bc == 0x7fffffff) { bm = v; bc = c; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float om = __shfl_xor(bm, o, 64);
+    const int oc = __shfl_xor(bc, o, 64);
+    if (oc != 0x7fffffff && (bc == 0x7fffffff || om > bm || (om == bm && oc < bc))) { bm = om; bc = oc; }
+  }
+  m = bm;
+  amax = p[bc].idx;
   float S = 0.f;
-  for (int c = 0; c < nchunk; c++) S += p[c].s * expf(p[c].m - m);
+  for (int base = 0; base < nchunk; base += 64) {
+    const int c = base + lane;
+    const float t = c < nchunk ? p[c].s * expf(p[c].m - m) : 0.f;
+    const int cnt = min(64, nchunk - base);
+    for (int i = 0; i < cnt; i++) S += __shfl(t, i, 64);
+  }
   logS = logf(S);
 }
 
@@ -291,19 +329,39 @@ template <int DT>
 __global__ __launch_bounds__(LS_THREADS) void ls_final_kernel(
     const typename Elem<DT>::T* __restrict__ x, typename Elem<DT>::T* __restrict__ y,
     const LsPartial* __restrict__ part, int n, int64_t xs, int64_t ys, int nchunk) {
+  __shared__ float fold[2];
   const int64_t row = blockIdx.y;
   const int c0 = blockIdx.x * LS_CHUNK;
-  float m, logS;
-  int amax;
-  ls_fold(part + row * nchunk, nchunk, m, logS, amax);
+  if (threadIdx.x < 64) {  // the first wavefront folds the row's partials for the block
+    float fm, fl;
+    int amax;
+    ls_fold_wave(part + row * nchunk, nchunk, fm, fl, amax);
+    if (threadIdx.x == 0) { fold[0] = fm; fold[1] = fl; }
+  }
+  __syncthreads();
+  const float m = fold[0], logS = fold[1];
   const typename Elem<DT>::T* xr = x + row * xs;
   typename Elem<DT>::T* yr = y + row * ys;
+  using T = typename Elem<DT>::T;
+  const bool aligned = (((uintptr_t)xr | (uintptr_t)yr) % (4 * sizeof(T))) == 0;
 #pragma unroll
   for (int j = 0; j < LS_PER / 4; j++) {
     const int e0 = c0 + 4 * (threadIdx.x + LS_THREADS * j);
+    if (e0 >= n) continue;
+    const bool vec = aligned && e0 + 3 < n;
+    float v[4];
+    ls_load4<DT>(xr + e0, n - e0, vec, v);
+    if (vec) {
+      __attribute__((aligned(16))) T t[4];
 #pragma unroll
-    for (int c = 0; c < 4; c++)
-      if (e0 + c < n) Elem<DT>::st(yr + e0 + c, (Elem<DT>::ld(xr + e0 + c) - m) - logS);
+      for (int c = 0; c < 4; c++) Elem<DT>::st(t + c, (v[c] - m) - logS);
+      if constexpr (sizeof(T) == 4) *(uint4*)(yr + e0) = *(const uint4*)t;
+      else *(uint2*)(yr + e0) = *(const uint2*)t;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+        if (e0 + c < n) Elem<DT>::st(yr + e0 + c, (v[c] - m) - logS);
+    }
   }
 }
 
@@ -314,11 +372,11 @@ __global__ __launch_bounds__(64) void logprob_final_kernel(
     const typename Elem<DT>::T* __restrict__ x, const int64_t* __restrict__ labels,
     const LsPartial* __restrict__ part, float* __restrict__ out, int64_t* __restrict__ tok_out,
     int64_t rows, int n, int64_t xs, int nchunk) {
-  const int64_t row = (int64_t)blockIdx.x * 64 + threadIdx.x;
-  if (row >= rows) return;
+  const int64_t row = blockIdx.x;  // one wavefront per row
   float m, logS;
   int amax;
-  ls_fold(part + row * nchunk, nchunk, m, logS, amax);
+  ls_fold_wave(part + row * nchunk, nchunk, m, logS, amax);
+  if (threadIdx.x != 0) return;
   int64_t lab = labels ? labels[row] : (int64_t)amax;
   if (tok_out) tok_out[row] = lab;
   float r = NAN;
@@ -496,7 +554,7 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
   int nchunk = 0;
   int rc = ls_partials(logits, dtype, rows, n, x_stride, workspace, workspace_bytes, stream, &nchunk);
   if (rc != VX_OK || rows == 0) return rc;
-  const unsigned blocks = (unsigned)((rows + 63) / 64);
+  const unsigned blocks = (unsigned)rows;  // one wavefront per row
   const LsPartial* part = (const LsPartial*)workspace;
   switch (dtype) {
     case DT_F32:
