@@ -248,3 +248,21 @@ def test_decode_on_packed_expert_weights_keeps_every_bit():
         graph.replay()
         torch.cuda.synchronize()
         assert_bitwise(b.logprobs.cpu(), lp0, "graph replay on packed expert weights")
+    # a weight update the copies know nothing about: stale until invalidated, then the new weights decide
+    with torch.no_grad():
+        w.layers[0]["down"].mul_(-0.5)
+    b.load(dmeta, tok.numpy())
+    dec.step(b, 1)
+    torch.cuda.synchronize()
+    assert_bitwise(b.logprobs.cpu(), lp0, "the copies are not tracked: an eager step still reads the old ones")
+    w.invalidate_packed()
+    b.load(dmeta, tok.numpy())
+    dec.step(b, 1)
+    torch.cuda.synchronize()
+    lp_new = b.logprobs.cpu().clone()
+    assert not torch.equal(lp_new, lp0), "after invalidate_packed the updated weights are read"
+    w.pack_experts()
+    b.load(dmeta, tok.numpy())
+    dec.step(b, 1)
+    torch.cuda.synchronize()
+    assert_bitwise(b.logprobs.cpu(), lp_new, "repacked copies of the updated weights")

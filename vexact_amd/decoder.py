@@ -120,6 +120,13 @@ class DecoderWeights:
         Costs a second copy of the expert weights in HBM; call again after the weights change."""
         self.packed = [(ops.pack_expert_weights(l["gate_up"]), ops.pack_expert_weights(l["down"])) for l in self.layers]
 
+    def invalidate_packed(self) -> None:
+        """Drop the fragment-order copies. They are plain copies that nothing tracks: after any write to
+        ``layers[i]["gate_up"]`` / ``["down"]`` call this (decode then streams the ``[E, N, K]`` tensors again)
+        or ``pack_experts()``; a decode graph captured earlier still replays the old copies and has to be
+        captured again."""
+        self.packed = None
+
     def nbytes(self) -> int:
         n = self.embed.numel() + self.lm_head.numel() + self.final_norm.numel()
         for l in self.layers:
