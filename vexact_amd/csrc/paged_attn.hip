@@ -833,6 +833,20 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   static_assert(KPW == 8, "a wavefront's keys must stay inside one 16-key tile");
   const int ld_tt = wave >> 1;
   int pg_cache = 0, pg_base = -64;  // SRC_FAST: page ids of this wavefront's tile for blocks [pg_base, pg_base + 64), one per lane
+  // Per-lane parts of a load's byte offset inside the wavefront's 16-key tile that do not change from block to block:
+  // the key's row in the tile and the swizzled 16-byte slot. Per block only the clamp of the row to the sequence's
+  // last key and one 32-bit multiply-add per load remain.
+  int row_in[KPW / 4];
+  uint32_t kslot[KPW / 4], vslot[KPW / 4];
+  if constexpr (KIND != SRC_GENERIC) {
+#pragma unroll
+    for (int j = 0; j < KPW / 4; j++) {
+      const int row = KPW * wave + 4 * j + (lane >> 4);
+      row_in[j] = row & 15;
+      kslot[j] = 16u * (uint32_t)((lane & 15) ^ (row & 15));
+      vslot[j] = 16u * (uint32_t)((lane & 15) ^ ((row & 7) << 1));
+    }
+  }
   auto issue_block = [&](int kb, int stage) {
     const uint32_t dst0 = lds0 + stage * PFL_STAGE + KPW * wave * 256;
     if constexpr (KIND == SRC_GENERIC) {
@@ -879,12 +893,13 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
                            (uint32_t)__builtin_amdgcn_readfirstlane((int)kb64);
       const uint64_t vsb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(vb64 >> 32)) << 32) |
                            (uint32_t)__builtin_amdgcn_readfirstlane((int)vb64);
+      // rows past the sequence's last key repeat it (finite data under zero weights); a tile wholly past it reads key 0
+      const int last_in = tile_key <= src.last ? src.last - tile_key : 0;  // wave-uniform
 #pragma unroll
       for (int j = 0; j < KPW / 4; j++) {
-        const int row = KPW * wave + 4 * j + (lane >> 4);
-        const int dk = tile_key <= src.last ? min(kb + row, src.last) - key0 : 0;  // 0 .. 15
-        const uint32_t koff = (uint32_t)dk * (uint32_t)(src.skp * 2) + 16u * (uint32_t)((lane & 15) ^ (row & 15));
-        const uint32_t voff = (uint32_t)dk * (uint32_t)(src.svp * 2) + 16u * (uint32_t)((lane & 15) ^ ((row & 7) << 1));
+        const uint32_t dk = (uint32_t)min(row_in[j], last_in);  // 0 .. 15
+        const uint32_t koff = dk * (uint32_t)(src.skp * 2) + kslot[j];
+        const uint32_t voff = dk * (uint32_t)(src.svp * 2) + vslot[j];
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :: "s"(dst0 + 4 * j * 256), "v"(koff), "s"(ksb) : "memory", "m0");
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
