@@ -89,7 +89,9 @@ def test_router_tie_rule():
 
 
 @pytest.mark.parametrize("T,E,k,bm", [(1, 128, 8, 32), (256, 128, 8, 32), (4096, 128, 8, 128), (700, 6, 2, 64), (33, 4, 1, 16),
-                                      (1500, 128, 8, 64), (9000, 64, 4, 256)])
+                                      (1500, 128, 8, 64), (9000, 64, 4, 256),
+                                      # whole and partial 1024-entry chunks, expert counts that are no power of two
+                                      (512, 128, 8, 32), (513, 128, 8, 32), (384, 60, 7, 16), (130, 200, 6, 64), (300, 512, 8, 32)])
 def test_routing_integers_exact(T, E, k, bm):
     g = torch.Generator().manual_seed(T)
     sel = torch.randint(0, E, (T, k), generator=g)
