@@ -39,6 +39,7 @@ constexpr int WD_BM = 256, WD_BN = 256, WD_BK = 64;
 constexpr int WD_GROUP_M = 4;
 
 typedef __attribute__((address_space(3))) void* lptr_t;
+typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int wd_swz_x(int R) { return (R >> 1) & 7; }
 __device__ __forceinline__ int wd_swz_w(int R) { return (((R >> 4) & 3) << 1) | ((R >> 1) & 1); }
@@ -115,7 +116,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   uint32_t ld_off[NLQ];
   int64_t ld_wbase = 0;
   auto set_load_tile = [&](const WideTile& t) {
-    ld_wbase = t.wbase;
+    // wave-uniform by construction; said explicitly so that the loads' scalar base stays in scalar registers
+    // whatever the surrounding code makes the compiler choose
+    ld_wbase = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)((uint64_t)t.wbase >> 32)) << 32) |
+                         (uint32_t)__builtin_amdgcn_readfirstlane((int)t.wbase));
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int R = 8 * (wave + 8 * j) + lrow;
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
           pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
           pk.z = (uint32_t)o[4] | ((uint32_t)o[5] << 16);
           pk.w = (uint32_t)o[6] | ((uint32_t)o[7] << 16);
-          *(uint4*)cp = pk;
+          __builtin_nontemporal_store(__builtin_bit_cast(u32x4_nt, pk), (u32x4_nt*)cp);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; e++)
@@ -298,7 +302,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
             pk.y = (uint32_t)o[8 * h + 2] | ((uint32_t)o[8 * h + 3] << 16);
             pk.z = (uint32_t)o[8 * h + 4] | ((uint32_t)o[8 * h + 5] << 16);
             pk.w = (uint32_t)o[8 * h + 6] | ((uint32_t)o[8 * h + 7] << 16);
-            *(uint4*)(cp + 8 * h) = pk;
+            __builtin_nontemporal_store(__builtin_bit_cast(u32x4_nt, pk), (u32x4_nt*)(cp + 8 * h));
           }
         } else {
 #pragma unroll
