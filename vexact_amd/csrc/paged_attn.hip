@@ -988,21 +988,24 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   for (int i = 0; i < PFL_NS - 1; i++)
     if (i < nblk) issue_block(i * ATT_BLOCK, i);
   int stage = 0;
-  for (int b = 0; b < nblk; b++) {
-    const int kb = b * ATT_BLOCK;
-    chunk_reset(kb);
-    // KPW / 2 loads per block and wavefront; the next block's may still be in flight
-    if (b + 1 < nblk) {
-      static_assert(KPW == 8, "the wait below counts 4 loads per block and wavefront");
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  for (int b0 = 0; b0 < nblk; b0 += ATT_CHUNK / ATT_BLOCK) {  // one chunk of keys: per-chunk state, then the fold
+    chunk_reset(b0 * ATT_BLOCK);
+    const int b1 = min(nblk, b0 + ATT_CHUNK / ATT_BLOCK);
+    for (int b = b0; b < b1; b++) {
+      const int kb = b * ATT_BLOCK;
+      // KPW / 2 loads per block and wavefront; the next block's may still be in flight
+      if (b + 1 < nblk) {
+        static_assert(KPW == 8, "the wait below counts 4 loads per block and wavefront");
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();
+      if (b + PFL_NS - 1 < nblk) issue_block(kb + (PFL_NS - 1) * ATT_BLOCK, stage == 0 ? PFL_NS - 1 : stage - 1);
+      block_compute(kb, stage);
+      stage = stage + 1 == PFL_NS ? 0 : stage + 1;
     }
-    __syncthreads();
-    if (b + PFL_NS - 1 < nblk) issue_block(kb + (PFL_NS - 1) * ATT_BLOCK, stage == 0 ? PFL_NS - 1 : stage - 1);
-    block_compute(kb, stage);
-    stage = stage + 1 == PFL_NS ? 0 : stage + 1;
-    chunk_fold(kb, b);
+    chunk_fold((b1 - 1) * ATT_BLOCK, b1 - 1);
   }
 
   // lane (r16 = query row, g) holds dims 16 f + 4 g + r of fragment f
