@@ -152,12 +152,13 @@ __device__ __forceinline__ void attn_softmax_tile(f32x4 (&st)[4], int kb, float 
 #pragma unroll
       for (int r = 0; r < 4; r++) bm = fmaxf(bm, st[tt][r]);
   } else {
+    // key kb + 16 tt + 4 g + r is visible iff 16 tt + r <= lim: the comparisons then have constant left sides
+    const int lim = qpos - kb - 4 * g;
 #pragma unroll
     for (int tt = 0; tt < 4; tt++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const int key = kb + 16 * tt + 4 * g + r;
-        const float tv = (key <= qpos) ? st[tt][r] : -INFINITY;  // exp2(fma(-inf, c, .)) = 0 below
+        const float tv = (16 * tt + r <= lim) ? st[tt][r] : -INFINITY;  // exp2(fma(-inf, c, .)) = 0 below
         st[tt][r] = tv;
         bm = fmaxf(bm, tv);
       }
