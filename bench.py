@@ -49,7 +49,10 @@ def parse():
     ap.add_argument("--no-configs", action="store_true", help="skip the reference's other configurations (C1-C4, prefill GEMM)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-packed-experts", action="store_true",
-                    help="decode reads the [E, N, K] expert tensors instead of their fragment-order copies")
+                    help="every step reads the [E, N, K] expert tensors instead of their fragment-order copies")
+    ap.add_argument("--keep-unpacked-experts", action="store_true",
+                    help="keep the [E, N, K] expert tensors beside their fragment-order copies (a second copy of the "
+                         "expert weights; the default holds the fragment-order copies only)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--seed", type=int, default=5)
     ap.add_argument("--cpu-configs", action="store_true",
@@ -120,7 +123,8 @@ def cpu_configs(seed):
     print(json.dumps({"cpu_configs": res}), flush=True)
 
 
-def build_workload(layers=48, batch=256, seed=5, min_prompt=256, max_prompt=2048, grow=1, packed=True, log=True):
+def build_workload(layers=48, batch=256, seed=5, min_prompt=256, max_prompt=2048, grow=1, packed=True, log=True,
+                   keep_unpacked=False):
     """The headline workload: random-init weights, ``batch`` prompts of random ids prefilled with the library's own
     kernels into a paged cache (page 16, block tables from a random permutation of the pool, room for ``grow``
     more tokens per sequence), and the metadata of the decode step that follows."""
@@ -149,9 +153,14 @@ def build_workload(layers=48, batch=256, seed=5, min_prompt=256, max_prompt=2048
 
     t0 = time.time()
     w = DecoderWeights(cfg, device=dev, seed=seed)
+    # Expert weights in fragment order (made once per weight update): decode streams them, and the 256-row expert
+    # tiles of the prefill chunks read them too, so the [E, N, K] tensors are freed unless asked for.
+    if packed:
+        w.pack_experts(keep_unpacked=keep_unpacked)
     dec = Qwen3MoeDecoder(cfg, w, num_cache_blocks=pool, device=dev)
     torch.cuda.synchronize()
-    say(f"[bench] weights {w.nbytes() / 1e9:.1f} GB, KV pool {pool} pages "
+    say(f"[bench] weights {w.nbytes() / 1e9:.1f} GB"
+        f"{' + a second copy of the experts in fragment order' if packed and keep_unpacked else ''}, KV pool {pool} pages "
         f"({2 * cfg.num_layers * dec.key_cache[0].numel() * 2 / 1e9:.1f} GB), init {time.time() - t0:.1f}s")
 
     # ---- prefill with the library's own kernels, several sequences per pass
@@ -175,11 +184,6 @@ def build_workload(layers=48, batch=256, seed=5, min_prompt=256, max_prompt=2048
     del dec.buffers[(PT, PB)]
     del pb
     torch.cuda.empty_cache()
-
-    # ---- decode streams the expert weights from their fragment-order copies (made once per weight update)
-    if packed:
-        w.pack_experts()
-        torch.cuda.synchronize()
 
     ctx = [int(n) + 1 for n in prompt_lens]
     reqs = [dict(num_computed_tokens=ctx[i], tokens_this_step=1, block_ids=blocks[i]) for i in range(B)]
@@ -232,7 +236,8 @@ def main():
     torch.cuda.set_device(0)
 
     wl = build_workload(args.layers, args.batch, args.seed, args.min_prompt, args.max_prompt,
-                        grow=1 + max(0, args.loop_steps), packed=not args.no_packed_experts)
+                        grow=1 + max(0, args.loop_steps), packed=not args.no_packed_experts,
+                        keep_unpacked=args.keep_unpacked_experts)
     cfg, w, dec, B = wl.cfg, wl.w, wl.dec, wl.B
     blocks, ctx, reqs, dmeta, first_tokens, max_blocks = wl.blocks, wl.ctx, wl.reqs, wl.dmeta, wl.first_tokens, wl.max_blocks
     E, k, I, H = cfg.num_experts, cfg.top_k, cfg.moe_intermediate, cfg.hidden_size
@@ -417,6 +422,8 @@ def main():
         "config": {"workload": f"Qwen3-30B-A3B-shaped decoder ({cfg.num_layers} layers, 128 experts top-8, vocab 151936), "
                                f"hipGraph decode step, batch {B}, prompts U[{args.min_prompt},{args.max_prompt}], paged KV page 16",
                    "batch": B, "sum_context": sumL, "full_model": cfg.num_layers == 48 and B == 256},
+        "weights_gb": round(w.nbytes() / 1e9, 1),
+        "expert_weight_copies": 1 if (w.packed is None or w.packed_only) else 2,
         "step_hbm_bytes": int(step_bytes["total"]),
         "step_frac_of_hbm_roofline": round(step_bytes["total"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "logprob_drift_bits_b256_vs_b1": drift_bits,
@@ -454,6 +461,7 @@ def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
 
     from oracle import decoder as OD
     from oracle.row_ops import hf_rms_norm_ref, logprobs_ref, matmul_ref
+    from vexact_amd import ops
     # threads: the harness gives a one-GPU job 16 host cores (OMP_NUM_THREADS), whatever os.cpu_count() shows
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
     torch.set_num_threads(cores)
@@ -465,7 +473,10 @@ def cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, budget_s):
                 break
     except OSError:
         pass
-    lw = {k_: v.cpu() for k_, v in w.layers[0].items()}
+    lw = {k_: v.cpu() for k_, v in w.layers[0].items() if v is not None}
+    if w.packed_only:  # the oracle wants [E, N, K]
+        lw["gate_up"] = ops.unpack_expert_weights(w.packed[0][0]).cpu()
+        lw["down"] = ops.unpack_expert_weights(w.packed[0][1]).cpu()
     kc, vc = dec.key_cache[0].cpu().contiguous(), dec.value_cache[0].cpu().contiguous()
     cos, sin = OD.rope_tables_ref(cfg.head_dim, cfg.rope_theta, cfg.max_model_len)
     x = w.embed[torch.as_tensor(first_tokens).to(w.embed.device)].cpu()

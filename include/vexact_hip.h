@@ -242,13 +242,15 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
 int vx_packed_kchunks(int64_t K);
 int vx_pack_weights(const void* w, int64_t ldw, int64_t w_gstride, int64_t G, int64_t N, int64_t K, void* out,
                     hipStream_t stream);
-/* vx_moe_gemm on packed weights, bm in {16, 32, 64} (decode sizes). w (and w2 for epi 1) point at the packed
- * image of the projection's first row, which must lie a multiple of 16 rows into the packed tensor;
- * w_gstride = elements between consecutive experts there. Same bits as vx_moe_gemm. */
+/* vx_moe_gemm on packed weights, bm in {16, 32, 64} (decode sizes) or 256 (prefill sizes: K % 64 == 0 and
+ * x_rows as for vx_moe_gemm; ignored otherwise), so that a model needs no [E, N, K] copy beside the packed one.
+ * w (and w2 for epi 1) point at the packed image of the projection's first row, which must lie a multiple of
+ * 16 rows into the packed tensor; w_gstride = elements between consecutive experts there. Same bits as
+ * vx_moe_gemm. */
 int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2, int64_t w_gstride, void* c,
                        int64_t ldc, int64_t N, int64_t K, const int* tile_group, const int* tile_row0,
                        const int* tile_rows, int64_t max_tiles, int bm, const int* row_src, const void* row_scale,
-                       const int* row_scale_idx, int epi, hipStream_t stream);
+                       const int* row_scale_idx, int epi, int64_t x_rows, hipStream_t stream);
 
 /* Grouped products of the fused-MoE backward (FusedMoeExpertFunction.backward, fused_moe.py:126-265), bf16
  * with fp32 accumulation, over the same tile table / expert offsets as the forward.

@@ -224,6 +224,41 @@ def test_sampled_decode_is_batch_invariant_and_graph_safe():
     assert torch.equal(bg.tokens.cpu()[:5], tok_e[order])
 
 
+def test_model_with_fragment_order_expert_weights_only_keeps_every_bit():
+    # one copy of the expert weights: prefill (256-row expert tiles on the packed weights instead of 128-row tiles
+    # on [E, N, K]) and decode give the bits of the model that keeps both
+    cfg, w, dec, prompts, blocks = _setup(num_seqs=10, seed=13)
+    allseq = list(range(10))
+    assert sum(len(p) for p in prompts) > 1024
+    tok, lp, meta, ids = _prefill(dec, cfg, prompts, blocks, allseq)
+    assert dec.bucket(len(ids), 10).bm == 128
+    dmeta = _decode_meta(cfg, prompts, blocks, allseq)
+    b = dec.bucket(10, 10)
+    b.load(dmeta, tok.numpy())
+    dec.step(b, 1)
+    torch.cuda.synchronize()
+    lp_d, tok_d = b.logprobs.cpu().clone(), b.tokens.cpu().clone()
+
+    w2 = DecoderWeights(cfg, device="cuda", seed=13, std=0.05, norm_std=0.1)
+    both = w2.nbytes()
+    w2.pack_experts(keep_unpacked=False)
+    assert w2.packed_only and all(l["gate_up"] is None and l["down"] is None for l in w2.layers)
+    assert w2.nbytes() >= both  # the packed image pads K to a multiple of 256
+    with pytest.raises(RuntimeError):
+        w2.invalidate_packed()
+    dec2 = Qwen3MoeDecoder(cfg, w2, num_cache_blocks=dec.key_cache[0].shape[0])
+    tok2, lp2, _, _ = _prefill(dec2, cfg, prompts, blocks, allseq)
+    assert dec2.bucket(len(ids), 10).bm == 256
+    assert_bitwise(lp2, lp, "prefill logprobs: packed-only model vs [E, N, K] model")
+    assert torch.equal(tok2, tok)
+    b2 = dec2.bucket(10, 10)
+    b2.load(dmeta, tok.numpy())
+    dec2.step(b2, 1)
+    torch.cuda.synchronize()
+    assert_bitwise(b2.logprobs.cpu(), lp_d, "decode logprobs: packed-only model vs [E, N, K] model")
+    assert torch.equal(b2.tokens.cpu(), tok_d)
+
+
 def test_decode_on_packed_expert_weights_keeps_every_bit():
     # the same decode step with the experts streamed from their fragment-order copies: eager and in a graph
     cfg, w, dec, prompts, blocks = _setup(num_seqs=6, seed=9)

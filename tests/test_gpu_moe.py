@@ -429,6 +429,7 @@ def test_pack_expert_weights_is_an_exact_permutation(E, N, K):
     pk = ops.pack_expert_weights(w.cuda())
     assert pk.kchunks == (K + 255) // 256 * 8
     assert_bitwise(pk.data.cpu(), _pack_restatement(w, pk.kchunks), "packed weights")
+    assert_bitwise(ops.unpack_expert_weights(pk).cpu(), w, "unpack(pack(w))")
 
 
 @pytest.mark.parametrize("T,H,I,E,k", [(1, 512, 256, 32, 4), (70, 512, 256, 32, 4), (256, 2048, 768, 128, 8), (33, 200, 80, 6, 2)])
@@ -448,3 +449,25 @@ def test_packed_expert_weights_give_the_same_bits(T, H, I, E, k):
         eo_p = ops.moe_gemm_packed(hw, pdn, r)
         assert_bitwise(hw_p, hw, f"gate/up + SwiGLU on packed weights, {bm}-row tiles")
         assert_bitwise(eo_p, eo, f"down projection on packed weights, {bm}-row tiles")
+
+
+@pytest.mark.parametrize("T,H,I,E,k", [(2500, 256, 128, 8, 2), (1100, 192, 64, 3, 1), (4096, 2048, 768, 16, 4)])
+def test_packed_expert_weights_on_256_row_tiles_give_the_same_bits(T, H, I, E, k):
+    # prefill-sized steps: the 256 x 256 kernel reading the fragment-order copy against the same kernel on [E, N, K]
+    # (whole tiles, tail tiles of a few rows, an expert count that is no power of two, the model's own shape)
+    x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=43)
+    xg, wg, sg, dg = x.cuda(), w.cuda(), sel.cuda(), down.cuda()
+    gu = torch.cat([gate, up], dim=1).cuda()
+    pgu, pdn = ops.pack_expert_weights(gu), ops.pack_expert_weights(dg)
+    r = ops.moe_route(sg, E, bm=256)
+    hw = ops.moe_gemm(xg, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=wg, row_scale_idx=r.sorted_flat)
+    eo = ops.moe_gemm(hw, dg, r)
+    hw_p = ops.moe_gemm_packed(xg, pgu.rows(0, I), r, w2=pgu.rows(I, 2 * I), row_src=r.sorted_token, row_scale=wg,
+                               row_scale_idx=r.sorted_flat)
+    eo_p = ops.moe_gemm_packed(hw, pdn, r)
+    assert_bitwise(hw_p, hw, "gate/up + SwiGLU on packed weights, 256-row tiles")
+    assert_bitwise(eo_p, eo, "down projection on packed weights, 256-row tiles")
+    y = ops.fused_moe(xg, wg, sg, gu[:, :I], gu[:, I:], dg, E)
+    yp = ops.fused_moe(xg, wg, sg, gu[:, :I], gu[:, I:], dg, E, packed=(pgu, pdn))
+    assert_bitwise(yp, y, "fused MoE with packed weights at a prefill size")
+

@@ -63,8 +63,17 @@ struct WideTile {
 // columns and a lane 8 consecutive ones per activation row.
 // XI = 16-row activation tiles per wavefront: 8 (256-row tiles, the normal form) or 4 (128-row tiles: the same
 // weight panel and barriers for half the rows, for a last round of tiles that would leave half the chip idle).
-template <int EPI, bool GROUPED, int XI = 8>
+// PACKED: the weights are in fragment order (pack_weights_kernel; p.ldw = 32-wide k-chunks stored per 16-row
+// block; a step advances two chunks = 1024 elements). There 16-byte piece pc (8 k-elements) of the 16 rows of a
+// block is contiguous, so the weight tile lives in LDS piece-major and in fragment order, [pc][position] with
+// position 64 wn + 16 j + rho for MFMA row rho of wavefront wn's weight fragment j: a load instruction fills
+// the 64 positions of one (pc, wn) from 4 blocks x 256 contiguous bytes (whole lines, 4 consecutive lanes on 64
+// contiguous bytes, as with row-major weights), and a fragment read takes 256 contiguous LDS bytes per 16 lanes
+// (no swizzle needed). With the SwiGLU epilogue an instruction mixes gate rows (j < 2) and up rows, so the up
+// image's distance from the gate image is part of the lane offset (host check: w2 behind w, within 4 GiB).
+template <int EPI, bool GROUPED, int XI = 8, bool PACKED = false>
 __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  static_assert(!PACKED || GROUPED, "fragment-order weights exist for the grouped form only");
   extern __shared__ __attribute__((aligned(1024))) uint8_t wd_lds[];
   constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;  // output columns per tile
   constexpr int BM = 32 * XI;                             // activation rows per tile
@@ -128,10 +137,27 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
         const int64_t sr = (GROUPED && p.row_src) ? (int64_t)p.row_src[rr] : (int64_t)rr;
         ld_off[j] = (uint32_t)((sr * p.ldx + (lslot ^ wd_swz_x(R)) * 8) * 2);
       }
+      // tile row (in the numbering of the row-major LDS layout) and 16-byte piece that this lane fetches
+      int Rw, pc;
+      if constexpr (PACKED) {
+        const int qq = wave + 8 * j;  // instruction (pc, wn) = (qq / 4, qq % 4) fills positions 64 wn + lane
+        pc = qq >> 2;
+        Rw = 64 * (qq & 3) + 16 * ((lane & 15) >> 2) + 4 * (lane >> 4) + (lane & 3);
+      } else {
+        Rw = R;
+        pc = lslot ^ wd_swz_w(R);
+      }
       int col;
-      if constexpr (EPI == EPI_SWIGLU) col = t.n0 + 32 * (R >> 6) + 8 * ((R >> 4) & 3) + 4 * ((R >> 2) & 1) + (R & 3);
-      else col = t.n0 + R;
-      ld_off[NXQ + j] = (uint32_t)(((int64_t)min(col, N - 1) * p.ldw + (lslot ^ wd_swz_w(R)) * 8) * 2);
+      if constexpr (EPI == EPI_SWIGLU) col = t.n0 + 32 * (Rw >> 6) + 8 * ((Rw >> 4) & 3) + 4 * ((Rw >> 2) & 1) + (Rw & 3);
+      else col = t.n0 + Rw;
+      if constexpr (PACKED) {
+        const int cc = min(col, N - 1);
+        int64_t off = (((int64_t)(cc >> 4) * p.ldw + (pc >> 2)) * 512 + ((cc & 15) + 16 * (pc & 3)) * 8) * 2;
+        if (EPI == EPI_SWIGLU && ((Rw >> 3) & 1)) off += (int64_t)((const uint8_t*)p.w2 - (const uint8_t*)p.w);
+        ld_off[NXQ + j] = (uint32_t)off;
+      } else {
+        ld_off[NXQ + j] = (uint32_t)(((int64_t)min(col, N - 1) * p.ldw + pc * 8) * 2);
+      }
     }
   };
   int ld_lin = first, ld_k = 0;
@@ -139,13 +165,13 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)wd_lds + wave * 1024;
   // EPI_SWIGLU: weight rows 8 q .. 8 q + 7 of load instruction q = wave + 8 j have bit 3 of the row
   // index equal to the parity of the wavefront, which says gate or up
-  const bf16_t* wsrc = (EPI == EPI_SWIGLU && (wave & 1)) ? p.w2 : p.w;
+  const bf16_t* wsrc = (EPI == EPI_SWIGLU && !PACKED && (wave & 1)) ? p.w2 : p.w;
   // The loads are written as asm so that the compiler does not track them: told that they write LDS,
   // it would wait for them (vmcnt(0)) before the first fragment read after they are issued. The
   // wait that matters is the explicit one before the barrier that precedes their first use.
   auto issue_one = [&](int q, int stage) {
     const uint32_t dst = lds0 + stage * STAGE + (q < NXQ ? q * 8192 : XBYTES + (q - NXQ) * 8192);
-    const bf16_t* base = (q < NXQ ? p.x : wsrc + ld_wbase) + ld_k;
+    const bf16_t* base = q < NXQ ? p.x + ld_k : wsrc + ld_wbase + (PACKED ? 16 * ld_k : ld_k);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
   };
@@ -174,12 +200,13 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   // Activation rows 16 XI wm + 16 i + r16: swizzle term r16 >> 1. Weight rows
   // 64 wn + 16 (r16 / 4) + 4 j + r16 % 4: swizzle term 2 (r16 / 4) + (r16 % 4) / 2.
   const int xoff = (16 * XI * wm + r16) * 128 + ((g ^ (r16 >> 1)) * 16);
-  const int woff = XBYTES + (64 * wn + 16 * (r16 >> 2) + (r16 & 3)) * 128 +
-                   ((g ^ (((r16 >> 2) << 1) | ((r16 >> 1) & 1))) * 16);
+  const int woff = PACKED ? XBYTES + g * 4096 + (64 * wn + r16) * 16
+                          : XBYTES + (64 * wn + 16 * (r16 >> 2) + (r16 & 3)) * 128 +
+                                ((g ^ (((r16 >> 2) << 1) | ((r16 >> 1) & 1))) * 16);
   struct Frag { uint4 w[4], x[XI]; };
   // read number r (0 .. 3 + XI) of a fragment set: the 4 weight operands first, then the XI activation ones
   auto read_one = [&](Frag& f, int r, const uint8_t* sb, int ks) {
-    if (r < 4) f.w[r] = *(const uint4*)(sb + (woff ^ (64 * ks)) + r * 512);
+    if (r < 4) f.w[r] = PACKED ? *(const uint4*)(sb + woff + ks * 16384 + r * 256) : *(const uint4*)(sb + (woff ^ (64 * ks)) + r * 512);
     else f.x[r - 4] = *(const uint4*)(sb + (xoff ^ (64 * ks)) + (r - 4) * 2048);
   };
   // 4 XI MFMAs on `cur`, interleaved with the 4 + XI reads of `nxt` and (LOADS) the global loads of a step
@@ -317,20 +344,27 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
 
 // Launch helper shared by the dense and the grouped entry points. x_rows = rows addressable in x
 // (bounds the 32-bit load offsets). Returns false (nothing launched) when the shape does not qualify.
-template <int EPI, bool GROUPED, int XI = 8>
+template <int EPI, bool GROUPED, int XI = 8, bool PACKED = false>
 static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int64_t x_rows, hipStream_t stream) {
   constexpr int NOUT = (EPI == EPI_SWIGLU) ? 128 : 256;
   constexpr int LDS = 2 * (32 * XI + WD_BN) * WD_BK * 2;  // two stages of an activation and a weight tile
   if (p.K % WD_BK != 0 || p.N <= 0 || tiles_m <= 0 || x_rows <= 0) return false;
   const int64_t lim = (int64_t)1 << 32;
-  if ((x_rows * p.ldx + p.K) * 2 >= lim || ((int64_t)p.N * p.ldw + p.K) * 2 >= lim) return false;
+  // bytes of one group's weights that a load offset must reach (PACKED: 16-row blocks of p.ldw 1 KB chunks)
+  int64_t wspan = PACKED ? (((int64_t)p.N + 15) / 16) * p.ldw * 1024 : ((int64_t)p.N * p.ldw + p.K) * 2;
+  if (PACKED && EPI == EPI_SWIGLU) {  // up rows are addressed from the gate image
+    const int64_t delta = (const uint8_t*)p.w2 - (const uint8_t*)p.w;
+    if (delta < 0) return false;
+    wspan += delta;
+  }
+  if ((x_rows * p.ldx + p.K) * 2 >= lim || wspan >= lim) return false;
   const int64_t tn = ((int64_t)p.N + NOUT - 1) / NOUT;
   const int64_t tiles = tiles_m * tn;
   if (tiles > (1 << 30)) return false;
   static DeviceOnce once;  // per instantiation
   const int dev = once.slot();
   if (once.need(dev)) {
-    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, GROUPED, XI>,
+    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, GROUPED, XI, PACKED>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess) {
       (void)hipGetLastError();
       return false;
@@ -338,7 +372,7 @@ static inline bool gemm_wide_launch_t(const GemmParams& p, int64_t tiles_m, int6
     once.mark(dev);
   }
   const unsigned grid = (unsigned)(tiles >= 256 ? 256 : (tiles + 7) / 8 * 8);
-  gemm_wide_kernel<EPI, GROUPED, XI><<<grid, 512, LDS, stream>>>(p, (int)tiles_m, (int)tn);
+  gemm_wide_kernel<EPI, GROUPED, XI, PACKED><<<grid, 512, LDS, stream>>>(p, (int)tiles_m, (int)tn);
   return true;
 }
 
@@ -385,6 +419,12 @@ static inline bool gemm_wide_grouped_launch(const GemmParams& p, int epi, int64_
                                             hipStream_t stream) {
   if (epi == EPI_SWIGLU) return gemm_wide_launch_t<EPI_SWIGLU, true>(p, max_m_tiles, x_rows, stream);
   return gemm_wide_launch_t<EPI_PLAIN, true>(p, max_m_tiles, x_rows, stream);
+}
+// the same on fragment-order weights (p.ldw = k-chunks per 16-row block)
+static inline bool gemm_wide_grouped_packed_launch(const GemmParams& p, int epi, int64_t max_m_tiles, int64_t x_rows,
+                                                   hipStream_t stream) {
+  if (epi == EPI_SWIGLU) return gemm_wide_launch_t<EPI_SWIGLU, true, 8, true>(p, max_m_tiles, x_rows, stream);
+  return gemm_wide_launch_t<EPI_PLAIN, true, 8, true>(p, max_m_tiles, x_rows, stream);
 }
 
 // ---------------------------------------------------------------------------------------

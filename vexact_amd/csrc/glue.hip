@@ -194,6 +194,6 @@ const char* vx_status_string(int code) {
   }
 }
 
-int vx_abi_version() { return 4; }
+int vx_abi_version() { return 5; }
 
 }  // extern "C"

@@ -691,18 +691,19 @@ int vx_pack_weights(const void* w, int64_t ldw, int64_t w_gstride, int64_t G, in
   return launch_status();
 }
 
-// vx_moe_gemm on packed weights (streaming kernel only: bm in {16, 32, 64}). w / w2 point at the packed
-// image of the first row of the gate / up (or only) projection, which must be a multiple of 16 rows into
-// the packed tensor; w_gstride = elements between consecutive experts in the packed tensor.
+// vx_moe_gemm on packed weights (bm in {16, 32, 64}: streaming kernel; 256: the 256 x 256 kernel, which needs
+// K % 64 == 0 and x_rows as vx_moe_gemm does). w / w2 point at the packed image of the first row of the gate / up
+// (or only) projection, which must be a multiple of 16 rows into the packed tensor; w_gstride = elements between
+// consecutive experts in the packed tensor.
 int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2, int64_t w_gstride, void* c,
                        int64_t ldc, int64_t N, int64_t K, const int* tile_group, const int* tile_row0,
                        const int* tile_rows, int64_t max_tiles, int bm, const int* row_src, const void* row_scale,
-                       const int* row_scale_idx, int epi, hipStream_t stream) {
+                       const int* row_scale_idx, int epi, int64_t x_rows, hipStream_t stream) {
   if (!x || !w || !c || !tile_group || !tile_row0 || !tile_rows) return VX_ERR_ARG;
   if (N <= 0 || K <= 0 || N > 0x7fffffff || K > 0x7fffffff || max_tiles < 0) return VX_ERR_ARG;
   if (epi != EPI_PLAIN && epi != EPI_SWIGLU) return VX_ERR_ARG;
   if (epi == EPI_SWIGLU && (!w2 || !row_scale)) return VX_ERR_ARG;
-  if (bm != 16 && bm != 32 && bm != 64) return VX_ERR_ARG;
+  if (bm != 16 && bm != 32 && bm != 64 && bm != 256) return VX_ERR_ARG;
   if (((uintptr_t)x % 16) != 0 || ((uintptr_t)w % 16) != 0 || (ldx % 8) != 0 || (w_gstride % 8) != 0)
     return VX_ERR_UNSUPPORTED;
   if (epi == EPI_SWIGLU && ((uintptr_t)w2 % 16) != 0) return VX_ERR_UNSUPPORTED;
@@ -716,6 +717,10 @@ int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2
   p.tile_group = tile_group; p.tile_row0 = tile_row0; p.tile_rows = tile_rows;
   p.row_src = row_src;
   p.row_scale = (const bf16_t*)row_scale; p.row_scale_idx = row_scale_idx;
+  if (bm == 256) {
+    if (x_rows <= 0 || !gemm_wide_grouped_packed_launch(p, epi, max_tiles, x_rows, stream)) return VX_ERR_UNSUPPORTED;
+    return launch_status();
+  }
   const dim3 grid((unsigned)((N + 63) / 64), (unsigned)max_tiles);
 #define VX_GP(MT)                                                                                            \
   do {                                                                                                       \

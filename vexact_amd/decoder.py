@@ -113,32 +113,59 @@ class DecoderWeights:
             )
 
         self.packed = None
+        self.packed_only = False
 
-    def pack_experts(self) -> None:
-        """Add fragment-order copies of the expert weights (``ops.pack_expert_weights``): steps whose expert
-        tiles have at most 64 rows (decode) stream those; larger steps keep reading the ``[E, N, K]`` tensors.
-        Costs a second copy of the expert weights in HBM; call again after the weights change."""
-        self.packed = [(ops.pack_expert_weights(l["gate_up"]), ops.pack_expert_weights(l["down"])) for l in self.layers]
+    def pack_experts(self, keep_unpacked: bool = True, low_peak: bool = False) -> None:
+        """Add fragment-order copies of the expert weights (``ops.pack_expert_weights``). Steps whose expert
+        tiles have at most 64 rows (decode) stream them, and so do 256-row tiles (prefill chunks); only the
+        128-row kernel needs the ``[E, N, K]`` tensors. ``keep_unpacked=False`` frees those tensors, so that the
+        model holds one copy of its expert weights (the decoder then never picks 128-row tiles; call this before
+        the first ``bucket()``); weights are then updated by loading new ``[E, N, K]`` tensors into ``layers[i]``
+        and packing again. By default every layer is packed before anything is freed and the freed memory goes
+        back to the driver, so both copies exist for a moment; ``low_peak=True`` frees layer by layer instead
+        (the packed tensors then land in recycled blocks, measured 1.5 % slower per decode step). With
+        ``keep_unpacked=True`` call this again, or ``invalidate_packed()``, after the weights change."""
+        if self.packed_only:
+            raise RuntimeError("the [E, N, K] expert tensors have been freed: nothing to pack from")
+        self.packed = []
+        for l in self.layers:
+            self.packed.append((ops.pack_expert_weights(l["gate_up"]), ops.pack_expert_weights(l["down"])))
+            if not keep_unpacked and low_peak:
+                l["gate_up"] = l["down"] = None
+        if not keep_unpacked:
+            for l in self.layers:
+                l["gate_up"] = l["down"] = None
+            torch.cuda.empty_cache()  # hand the freed tensors' memory back, so that later allocations start afresh
+        self.packed_only = not keep_unpacked
 
     def invalidate_packed(self) -> None:
         """Drop the fragment-order copies. They are plain copies that nothing tracks: after any write to
         ``layers[i]["gate_up"]`` / ``["down"]`` call this (decode then streams the ``[E, N, K]`` tensors again)
         or ``pack_experts()``; a decode graph captured earlier still replays the old copies and has to be
         captured again."""
+        if self.packed_only:
+            raise RuntimeError("the fragment-order copies are the only expert weights left")
         self.packed = None
 
     def nbytes(self) -> int:
+        """Bytes of the model's weights (one copy of each; fragment-order copies kept beside ``[E, N, K]`` tensors
+        are extra)."""
         n = self.embed.numel() + self.lm_head.numel() + self.final_norm.numel()
         for l in self.layers:
-            n += sum(t.numel() for t in l.values())
+            n += sum(t.numel() for t in l.values() if t is not None)
+        if self.packed_only:
+            n += sum(a.data.numel() + b.data.numel() for a, b in self.packed)
         return 2 * n
 
     def to_cpu(self) -> "DecoderWeights":
         c = object.__new__(DecoderWeights)
         c.cfg = self.cfg
         c.embed, c.lm_head, c.final_norm = self.embed.cpu(), self.lm_head.cpu(), self.final_norm.cpu()
+        if self.packed_only:
+            raise RuntimeError("the [E, N, K] expert tensors have been freed")
         c.layers = [{k: v.cpu() for k, v in l.items()} for l in self.layers]
         c.packed = None
+        c.packed_only = False
         return c
 
 
@@ -224,7 +251,8 @@ def capture_sizes(max_size: int) -> list[int]:
 class StepBuffers:
     """Static device buffers of one (num_tokens, num_seqs) bucket."""
 
-    def __init__(self, cfg: DecoderConfig, num_tokens: int, num_seqs: int, device):
+    def __init__(self, cfg: DecoderConfig, num_tokens: int, num_seqs: int, device, packed_only: bool = False):
+        """``packed_only``: the model holds fragment-order expert weights only (no 128-row expert tiles)."""
         T, B = num_tokens, num_seqs
         self.num_tokens, self.num_seqs = T, B
         self.max_blocks = (cfg.max_model_len + cfg.page_size - 1) // cfg.page_size
@@ -265,7 +293,8 @@ class StepBuffers:
         self.topk_idx = z(T, k, dtype=i32)
         self.hw = z(T * k, cfg.moe_intermediate, dtype=bf)
         self.eo = z(T * k, H, dtype=bf)
-        self.bm = ops.moe_tile_rows(T)
+        self.bm = ops.moe_tile_rows(T, wide_ok=(cfg.hidden_size % 64 == 0 and cfg.moe_intermediate % 64 == 0),
+                                    packed_only=packed_only)
         from . import _lib
 
         lib = _lib.load()
@@ -344,7 +373,8 @@ class Qwen3MoeDecoder:
     def bucket(self, num_tokens: int, num_seqs: int) -> StepBuffers:
         key = (num_tokens, num_seqs)
         if key not in self.buffers:
-            b = self.buffers[key] = StepBuffers(self.cfg, num_tokens, num_seqs, self.device)
+            b = self.buffers[key] = StepBuffers(self.cfg, num_tokens, num_seqs, self.device,
+                                                packed_only=self.w.packed_only)
             # Steps run one at a time on one stream, so buckets share one decode-attention workspace. A bucket
             # that needs more than the shared one holds gets a new, larger one, which later buckets share;
             # earlier buckets (and graphs captured on them) keep the tensor they were given.
@@ -378,13 +408,16 @@ class Qwen3MoeDecoder:
             if routing_log is not None:  # debugging / tests only (allocates; not for graph capture)
                 routing_log.append(b.topk_idx.clone())
             r = ops.moe_route(b.topk_idx, E, bm=b.bm, buffers=b.route_ints)
-            if w.packed is not None and r.bm <= 64:
+            if w.packed is not None and (r.bm <= 64 or r.bm == 256):
                 pgu, pdn = w.packed[li]
                 ops.moe_gemm_packed(b.h, pgu.rows(0, I), r, w2=pgu.rows(I, 2 * I), row_src=r.sorted_token,
                                     row_scale=b.topk_w, row_scale_idx=r.sorted_flat, out=b.hw)
                 ops.moe_gemm_packed(b.hw, pdn, r, out=b.eo)
             else:
                 gu = lw["gate_up"]
+                if gu is None:
+                    raise RuntimeError(f"bucket with {r.bm}-row expert tiles was made before the [E, N, K] expert "
+                                       "tensors were freed: make buckets after pack_experts(keep_unpacked=False)")
                 ops.moe_gemm(b.h, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=b.topk_w,
                              row_scale_idx=r.sorted_flat, out=b.hw)
                 ops.moe_gemm(b.hw, lw["down"], r, out=b.eo)

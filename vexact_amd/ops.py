@@ -555,13 +555,16 @@ def router_topk(
     return w, idx
 
 
-def moe_tile_rows(num_tokens: int, wide_ok: bool = True) -> int:
+def moe_tile_rows(num_tokens: int, wide_ok: bool = True, packed_only: bool = False) -> int:
     """Rows per expert tile, chosen from the token count only (any choice gives the same bits).
-    ``wide_ok``: both GEMM depths are multiples of 64, which the 256-row kernel needs."""
+    ``wide_ok``: both GEMM depths are multiples of 64, which the 256-row kernel needs.
+    ``packed_only``: only fragment-order weights exist, which the 128-row kernel does not read."""
     if num_tokens <= 256:
         return 32
     if num_tokens <= 1024:
         return 64
+    if packed_only:
+        return 256 if wide_ok else 64
     if num_tokens < 2048 or not wide_ok:
         return 128
     return 256
@@ -677,14 +680,25 @@ def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
     return pk
 
 
+def unpack_expert_weights(pk: PackedExpertWeights) -> torch.Tensor:
+    """The ``[E, N, K]`` tensor that ``pk`` was packed from (for checkpointing or inspecting a model that holds
+    fragment-order weights only; a permutation done with torch views, not a kernel)."""
+    assert pk.row0 == 0 and pk.rows_n == pk.N, "unpack the whole tensor, not a row range"
+    nb = (pk.N + 15) // 16
+    v = pk.data.view(pk.E, nb, pk.kchunks, 4, 16, 8)  # [e][row block][k-chunk][lane / 16][lane % 16][8]
+    return v.permute(0, 1, 4, 2, 3, 5).reshape(pk.E, nb * 16, pk.kchunks * 32)[:, : pk.N, : pk.K].contiguous()
+
+
 def moe_gemm_packed(
     x: torch.Tensor, w: PackedExpertWeights, routing: MoeRouting, *, w2: Optional[PackedExpertWeights] = None,
     row_src: Optional[torch.Tensor] = None, row_scale: Optional[torch.Tensor] = None,
     row_scale_idx: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """``moe_gemm`` on packed weights (tile tables of 16 / 32 / 64 rows); same bits."""
+    """``moe_gemm`` on packed weights (tile tables of 16 / 32 / 64 rows: weight-streaming kernel; 256 rows:
+    the 256 x 256 kernel, K a multiple of 64); same bits."""
     n_rows = routing.T * routing.k
-    assert x.dtype == torch.bfloat16 and x.stride(1) == 1 and routing.bm in (16, 32, 64)
+    assert x.dtype == torch.bfloat16 and x.stride(1) == 1 and routing.bm in (16, 32, 64, 256)
+    assert routing.bm != 256 or w.K % 64 == 0
     if w2 is not None:
         assert w2.data is w.data and w2.rows_n == w.rows_n and row_scale is not None
     N = w.rows_n
@@ -694,7 +708,7 @@ def moe_gemm_packed(
             x.data_ptr(), x.stride(0), w.data_ptr(), w2.data_ptr() if w2 is not None else None, w.gstride,
             c.data_ptr(), c.stride(0), N, w.K, routing.tile_group.data_ptr(), routing.tile_row0.data_ptr(),
             routing.tile_rows.data_ptr(), routing.max_tiles, routing.bm, _ptr(row_src), _ptr(row_scale),
-            _ptr(row_scale_idx), 1 if w2 is not None else 0, _stream(),
+            _ptr(row_scale_idx), 1 if w2 is not None else 0, x.shape[0], _stream(),
         ),
         "vx_moe_gemm_packed",
     )
@@ -846,7 +860,7 @@ def fused_moe(
     H_, I_ = gate_w.shape[-1], down_w.shape[-1]
     r = moe_route(selected_experts, num_experts,
                   bm=moe_tile_rows(selected_experts.shape[0], wide_ok=(H_ % 64 == 0 and I_ % 64 == 0)))
-    if packed is not None and r.bm <= 64:
+    if packed is not None and (r.bm <= 64 or r.bm == 256):
         pgu, pdn = packed
         assert pgu.rows_n == 2 * I_ and pgu.K == H_ and pdn.rows_n == down_w.shape[1] and pdn.K == I_
         hw = moe_gemm_packed(x, pgu.rows(0, I_), r, w2=pgu.rows(I_, 2 * I_), row_src=r.sorted_token, row_scale=rw,
