@@ -243,7 +243,8 @@ int vx_packed_kchunks(int64_t K);
 int vx_pack_weights(const void* w, int64_t ldw, int64_t w_gstride, int64_t G, int64_t N, int64_t K, void* out,
                     hipStream_t stream);
 /* vx_moe_gemm on packed weights, bm in {16, 32, 64} (decode sizes) or 256 (prefill sizes: K % 64 == 0 and
- * x_rows as for vx_moe_gemm; ignored otherwise), so that a model needs no [E, N, K] copy beside the packed one.
+ * x_rows as for vx_moe_gemm, and for epi 1 w2 must lie behind w within 4 GiB, as the up rows of one packed
+ * gate/up tensor do; x_rows is ignored otherwise), so that a model needs no [E, N, K] copy beside the packed one.
  * w (and w2 for epi 1) point at the packed image of the projection's first row, which must lie a multiple of
  * 16 rows into the packed tensor; w_gstride = elements between consecutive experts there. Same bits as
  * vx_moe_gemm. */
