@@ -164,3 +164,124 @@ def test_huggingface_causal_lm_through_the_registered_interfaces():
                 pass
         else:
             ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had
+
+
+def test_huggingface_decode_step_captured_the_way_the_reference_captures_it():
+    """The reference's CudaGraphManager (vexact/inferencer/cudagraph_utils.py:108-176) warms the model up and captures
+    it on static buffers with an even split of the bucket's tokens, no cache writes and max_seqlen_q = the bucket's
+    tokens; a step then copies its metadata in, padded (inferencer.py:293-349: zeroed ids and positions, slot -1,
+    zero-length padded requests whose query_start_loc is the real token count, block tables 0) and replays. The
+    same procedure on the HIP kernels: replays of a 4-token / 4-request bucket give the bits of the eager,
+    unpadded steps, for three and for two requests, and write the cache the eager step writes."""
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+    from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
+    from vexact_amd.batch_invariant_ops.kv_cache_context import (KVCacheManager, KVCacheStore, clear_kv_cache_context,
+                                                                 set_kv_cache_context)
+    from vexact_amd.decoder import build_step_metadata
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+
+    page, max_blocks_per_req, cap_t, cap_s = 16, 32, 4, 4
+    cache_cfg = types.SimpleNamespace(page_size=page, max_cache_blocks=64)
+    had = ALL_ATTENTION_FUNCTIONS._global_mapping.get("triton-invariant") if hasattr(ALL_ATTENTION_FUNCTIONS, "_global_mapping") else None
+    ALL_ATTENTION_FUNCTIONS["triton-invariant"] = flash_attention_forward
+    apply_qwen3_moe_patches()
+    try:
+        hf_cfg, model = _build_model(seed=23)
+        model = model.cuda()
+        store = KVCacheStore(hf_cfg, cache_cfg, torch.device("cuda"))
+        alloc = KVCacheManager(cache_cfg)
+        rng = np.random.default_rng(24)
+        lens = [21, 70, 9]
+        prompts = [rng.integers(0, hf_cfg.vocab_size, size=n) for n in lens]
+        blocks = [list(alloc.allocate_blocks(n + 2, 0)) for n in lens]
+
+        def forward(ids, positions):
+            out = model.model(input_ids=ids, position_ids=positions, use_cache=False, return_dict=True)
+            return model.lm_head(out.last_hidden_state)
+
+        def eager(which, new_tokens, ids):
+            reqs = [dict(num_computed_tokens=done, tokens_this_step=new, block_ids=blocks[s])
+                    for s, (done, new) in zip(which, new_tokens)]
+            meta = build_step_metadata(reqs, page, max_blocks_per_req)
+            dev = {k: torch.as_tensor(v).cuda() for k, v in meta.items() if k != "max_seqlen_q"}
+            set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache,
+                                 block_tables=dev["block_tables"], context_lens=dev["context_lens"],
+                                 slot_mapping=dev["slot_mapping"], query_start_loc=dev["query_start_loc"],
+                                 max_seqlen_q=int(meta["max_seqlen_q"]))
+            try:
+                with torch.inference_mode(), set_batch_invariant_mode(True):
+                    logits = forward(torch.as_tensor(ids)[None].cuda(), dev["positions"][None])
+                    last = (dev["query_start_loc"][1:] - 1).long()
+                    return logits[0, last, :].clone(), meta
+            finally:
+                clear_kv_cache_context()
+
+        plogits, _ = eager([0, 1, 2], [(n, n) for n in lens], np.concatenate(prompts))
+        first = plogits.argmax(-1).cpu().numpy()
+
+        # ---- static buffers of the bucket and the capture, as CudaGraphManager.capture does it
+        i32 = dict(dtype=torch.int32, device="cuda")
+        ids_s = torch.zeros(1, cap_t, dtype=torch.int64, device="cuda")
+        pos_s = torch.zeros(1, cap_t, dtype=torch.int64, device="cuda")
+        bt_s = torch.zeros(cap_s, max_blocks_per_req, **i32)
+        ctx_s = torch.zeros(cap_s, **i32)
+        slot_s = torch.full((cap_t,), -1, **i32)
+        qsl_s = torch.zeros(cap_s + 1, **i32)
+        per = torch.full((cap_s,), cap_t // cap_s, **i32)
+        per[: cap_t % cap_s] += 1
+        qsl_s[1:] = per.cumsum(0)
+        ctx_s.copy_(per)
+        set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache, block_tables=bt_s,
+                             context_lens=ctx_s, slot_mapping=slot_s, query_start_loc=qsl_s, max_seqlen_q=cap_t)
+        kcaches = list(store.key_cache.values()) if isinstance(store.key_cache, dict) else list(store.key_cache)
+        cache_before = [t.clone() for t in kcaches]
+        graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.inference_mode(), set_batch_invariant_mode(True):
+                forward(ids_s, pos_s)  # warm-up
+                with torch.cuda.graph(graph):
+                    out_s = forward(ids_s, pos_s)
+        finally:
+            clear_kv_cache_context()
+        for a, b in zip(kcaches, cache_before):
+            assert_bitwise(a, b, "capture and warm-up write nothing into the cache (slot -1)")
+
+        def replay(which, ids):
+            reqs = [dict(num_computed_tokens=lens[s] + 1, tokens_this_step=1, block_ids=blocks[s]) for s in which]
+            meta = build_step_metadata(reqs, page, max_blocks_per_req)
+            n = len(which)
+            ids_s.zero_(); pos_s.zero_(); bt_s.fill_(-1); ctx_s.zero_(); slot_s.fill_(-1); qsl_s.zero_()
+            bt_s[:n].copy_(torch.as_tensor(meta["block_tables"]))
+            ctx_s[:n].copy_(torch.as_tensor(meta["context_lens"]))
+            slot_s[:n].copy_(torch.as_tensor(meta["slot_mapping"]))
+            qsl_s[: n + 1].copy_(torch.as_tensor(meta["query_start_loc"]))
+            if cap_s > n:
+                bt_s[n:].zero_()
+                qsl_s[n + 1:] = n
+            ids_s[0, :n].copy_(torch.as_tensor(ids))
+            pos_s[0, :n].copy_(torch.as_tensor(meta["positions"]))
+            graph.replay()
+            torch.cuda.synchronize()
+            return out_s[0, :n, :].clone()
+
+        for which in ([0, 1, 2], [2, 0]):
+            store_before = [t.clone() for t in kcaches]
+            want, _ = eager(which, [(lens[s] + 1, 1) for s in which], first[which])
+            k_eager = [t.clone() for t in kcaches]
+            for t, b in zip(kcaches, store_before):
+                t.copy_(b)
+            got = replay(which, first[which])
+            assert_bitwise(got, want, f"graph replay of requests {which} in a 4 / 4 bucket vs the eager unpadded step")
+            for a, b in zip(kcaches, k_eager):
+                assert_bitwise(a, b, "the replay writes the keys the eager step writes")
+    finally:
+        remove_qwen3_moe_patches()
+        if had is None:
+            try:
+                del ALL_ATTENTION_FUNCTIONS._global_mapping["triton-invariant"]
+            except Exception:
+                pass
+        else:
+            ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had
+
