@@ -139,7 +139,12 @@ int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_
  *           (modes 3 and 4 are mode 0 with the kernel forced: 3 = one wavefront per chunk plus a
  *           combine launch, 4 = chunks folded inside one workgroup per (sequence, kv head); mode 0
  *           takes 4 when num_seqs * Hkv fills the machine. The results are bit-identical.)
- *   mode 1: paged general (chunked prefill, mixed batches) - same arithmetic per row as mode 0
+ *   mode 1: paged general (chunked prefill, mixed batches) - same arithmetic per row as mode 0. Sequences
+ *           with exactly one query row (decode tokens beside prefill chunks; a whole decode batch that a
+ *           captured graph launches with max_seqlen_q = its bucket's tokens) run on the mode-4 kernel
+ *           inside the same call when that form fits and no lse is asked for; the other sequences' row
+ *           blocks are numbered compactly when ceil(max_seqlen_q / rows per block) * num_seqs would mostly
+ *           be empty workgroups. Neither changes a bit.
  *   mode 2: packed K/V [Tk, Hkv, D] with cu_seqlens_k (skp = row stride, no block table)
  * q [total_q, Hq, Dk], k/v cache [blocks, page, Hkv, D], out [total_q, Hq, Dv];
  * query i of a sequence sits at absolute position kv_len - q_len + i.

@@ -78,6 +78,38 @@ def test_paged_correctness_and_batch_invariance(q_lens, kv_lens):
     assert_bitwise(_run_paged(q, k, v, page, pad_seqs=3), out, "padded sequence rows")
 
 
+@pytest.mark.parametrize(("qh", "kh", "d"), [(4, 2, 32), (8, 2, 128), (32, 4, 128)])
+def test_general_launch_over_prefill_chunks_and_decode_tokens(qh, kh, d):
+    # what a scheduler with chunked prefill hands over: a few chunks of very different lengths among single decode
+    # tokens. The launch numbers its (sequence, row block) pairs compactly and gives the single-token sequences to
+    # the decode kernel; every sequence keeps the bits it has alone, in the general and in the decode launch.
+    page = 16
+    q_lens = [200, 1, 1, 33, 1, 64, 1, 1, 7, 1, 1, 130]
+    prefix = [0, 700, 15, 100, 255, 1, 256, 31, 300, 1024, 0, 77]
+    kv_lens = [a + b for a, b in zip(q_lens, prefix)]
+    q = _seqs(q_lens, qh, d, 51, 0.1)
+    k = _seqs(kv_lens, kh, d, 52, 0.1)
+    v = _seqs(kv_lens, kh, d, 53, 0.1)
+    out = _run_paged(q, k, v, page)
+    ref = torch.cat([OA.eager_attention(a, b, c, d**-0.5) for a, b, c in zip(q, k, v)], dim=0)
+    torch.testing.assert_close(out.cpu(), ref, atol=3e-3, rtol=3e-3)
+    off = 0
+    for a, b, c in zip(q, k, v):
+        one = _run_paged([a], [b], [c], page)  # a single token alone runs as a decode launch
+        assert_bitwise(out[off : off + a.shape[0]], one, "alone vs in the mixed batch")
+        off += a.shape[0]
+    assert_bitwise(_run_paged(q, k, v, page, pad_seqs=5), out, "padded sequence rows")
+    assert_bitwise(_run_paged(q, k, v, page, max_seqlen_q=sum(q_lens)), out, "max_seqlen_q = the batch's tokens")
+    # a decode batch launched the general way (max_seqlen_q = the bucket's tokens, as a captured graph has it)
+    qd = [t[-1:] for t in q]
+    dec = _run_paged(qd, k, v, page)
+    assert_bitwise(_run_paged(qd, k, v, page, max_seqlen_q=64, pad_seqs=4), dec, "decode batch through a general launch")
+    off = 0
+    for i, a in enumerate(q):
+        assert_bitwise(dec[i : i + 1], out[off + a.shape[0] - 1 : off + a.shape[0]], "last chunk row vs decode step")
+        off += a.shape[0]
+
+
 def test_page_table_aliases_match():
     q, k, v = _seqs([1], 4, 32, 4), _seqs([33], 2, 32, 5), _seqs([33], 2, 32, 6)
     assert_bitwise(_run_paged(q, k, v, 16, page_kw="page_table"), _run_paged(q, k, v, 16, page_kw="block_table"), "alias")

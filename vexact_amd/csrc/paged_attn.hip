@@ -57,7 +57,34 @@ struct AttnParams {
   int max_chunks;
   const int* seq_order;  // optional [B]: decode kernels take sequence seq_order[i] as their i-th (longest first balances the tail)
   float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernels)
+  // General launches over batches whose sequences differ in their number of query rows:
+  int compact;      // != 0: blockIdx.x numbers (sequence, row block) pairs compactly, see locate_row_block
+  int single_mode;  // 0: every sequence; 1: only sequences with one query row (decode kernels inside a general
+                    // launch); 2: all others (the general kernel beside them)
 };
+
+// Which sequence and which of its row blocks (rpb query rows each) a workgroup of a general kernel works on.
+// Plain form: blockIdx.z and blockIdx.x, a grid of ceil(max_q / rpb) x num_seqs, most of it empty when one long
+// chunk shares a batch with decode tokens. Compact form: item w = blockIdx.x belongs to the last sequence s with
+// cu_q[s] / rpb + s <= w, as its row block w - (cu_q[s] / rpb + s); every sequence owns at least ceil(qlen / rpb)
+// items and there are total_q / rpb + num_seqs in all. Returns false when there is nothing to do.
+__device__ __forceinline__ bool locate_row_block(const AttnParams& p, int rpb, int& seq, int& bx) {
+  if (!p.compact) {
+    seq = blockIdx.z;
+    bx = blockIdx.x;
+    return true;
+  }
+  const int w = blockIdx.x;
+  int lo = 0, hi = p.num_seqs - 1;
+  while (lo < hi) {  // cu_q[s] / rpb + s is strictly increasing in s
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.cu_q[mid] / rpb + mid <= w) lo = mid;
+    else hi = mid - 1;
+  }
+  seq = lo;
+  bx = w - (p.cu_q[lo] / rpb + lo);
+  return bx >= 0;
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -463,6 +490,7 @@ __device__ __forceinline__ void attn_decode_fused_body(const AttnParams& p) {
   const int qlen = p.cu_q[seq + 1] - q0;
   const int kv_len = min(p.seqused_k[seq], p.max_kv);
   if (qlen <= 0 || kv_len <= 0) return;  // uniform over the block
+  if (p.single_mode == 1 && qlen != 1) return;  // inside a general launch: the general kernel takes these
   const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = tid >> 6;
   const int G = p.Hq / p.Hkv;
@@ -632,21 +660,23 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw
   // and 4 * QT / hpw row tiles: tile slot s = wave * QT + t -> head s % hpw, row tile s / hpw. With
   // hpw > 1 the wavefronts of a block walk the same keys at the same time, so K and V mostly come
   // from the CU's L1 after the first wavefront has fetched them.
-  const int seq = blockIdx.z;
+  const int rows_per_block = 16 * (4 * QT / hpw);
+  int seq, bx;
+  if (!locate_row_block(p, rows_per_block, seq, bx)) return;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
+  if (p.single_mode == 2 && qlen == 1) return;  // a decode kernel of the same launch takes these
   int kv_len, k0 = 0;
   if constexpr (KIND != SRC_PACKED) kv_len = min(p.seqused_k[seq], p.max_kv);
   else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-  const int rows_per_block = 16 * (4 * QT / hpw);
   int head_of[QT], i0_of[QT];
   bool any = false;
 #pragma unroll
   for (int t = 0; t < QT; t++) {
     const int s = wave * QT + t;
     head_of[t] = blockIdx.y * hpw + s % hpw;
-    i0_of[t] = blockIdx.x * rows_per_block + 16 * (s / hpw);
+    i0_of[t] = bx * rows_per_block + 16 * (s / hpw);
     any = any || i0_of[t] < qlen;
   }
   if (qlen <= 0 || kv_len <= 0 || !any) return;
@@ -754,16 +784,18 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   constexpr int KPW = ATT_BLOCK / PFL_WAVES;  // keys of a block that one wavefront brings in
   extern __shared__ __attribute__((aligned(1024))) uint8_t pf_lds[];
 
-  const int seq = blockIdx.z;
+  const int rows_per_block = 16 * (PFL_SLOTS / hpw);
+  int seq, bx;
+  if (!locate_row_block(p, rows_per_block, seq, bx)) return;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
+  if (p.single_mode == 2 && qlen == 1) return;  // a decode kernel of the same launch takes these
   int kv_len, k0 = 0;
   if constexpr (KIND != SRC_PACKED) kv_len = min(p.seqused_k[seq], p.max_kv);
   else { k0 = p.cu_k[seq]; kv_len = p.cu_k[seq + 1] - k0; }
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rows_per_block = 16 * (PFL_SLOTS / hpw);
-  const int i_base = blockIdx.x * rows_per_block;
+  const int i_base = bx * rows_per_block;
   if (qlen <= 0 || kv_len <= 0 || i_base >= qlen) return;  // uniform over the block
   const int shift = kv_len - qlen;  // absolute position of local row 0
   // last key any row of the block may see (uniform): every wavefront walks the blocks up to it
@@ -1064,8 +1096,24 @@ static int decode_form(int mode, int64_t num_seqs, int Hq, int Hkv, int Dv) {
 }
 
 template <int DK, int DV>
-static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hipStream_t stream) {
+static int launch_attn(const AttnParams& p_in, int mode, int max_q, int total_q, hipStream_t stream) {
+  AttnParams p = p_in;
   const bool fast = p.page_shift >= 4;  // page size a power of two >= 16
+  // A general paged launch hands its sequences of one query row (decode tokens that share the batch with prefill
+  // chunks, or a whole decode batch that a caller launches with the bucket's token count as max_seqlen_q) to the
+  // fused decode kernel and gives the general kernel the rest: the same bits (a prefill row equals the decode step
+  // of that token), a fraction of the work. Needs the fused form (chunk states in LDS, no workspace) and no lse.
+  const bool hybrid = mode == 1 && !p.lse && max_q != 1 && decode_form(4, p.num_seqs, p.Hq, p.Hkv, DV) == 1;
+  if (hybrid) {
+    AttnParams d = p;
+    d.single_mode = 1;
+    d.seq_order = nullptr;
+    const int64_t max_kv = p.max_kv;
+    d.max_chunks = (int)((max_kv + ATT_CHUNK - 1) / ATT_CHUNK);
+    const int rc = launch_attn<DK, DV>(d, 4, 1, total_q, stream);
+    if (rc != VX_OK) return rc;
+    p.single_mode = 2;
+  }
   if (mode == 0 || mode == 3 || mode == 4) {
     const int G = p.Hq / p.Hkv;
     constexpr int NW1 = 8, NW1S = 4, NW2 = 4;  // wavefronts per block for one (many / very many workgroups) / two q-tiles
@@ -1136,13 +1184,21 @@ static int launch_attn(const AttnParams& p, int mode, int max_q, int total_q, hi
     int hpw = 1;
     while (hpw * 2 <= 4 * QT && G % (hpw * 2) == 0) hpw *= 2;
     const int rpb = 16 * (4 * QT / hpw);
-    dim3 grid((rows + rpb - 1) / rpb, p.Hq / hpw, p.num_seqs);
+    // (sequence, row block) pairs: the plain grid of ceil(rows / rpb) x num_seqs, or the compact numbering when
+    // that is smaller (sequences with very different numbers of query rows)
+    auto row_grid = [&](int rb, unsigned heads) {
+      const int64_t plain = (int64_t)((rows + rb - 1) / rb) * p.num_seqs;
+      const int64_t comp = (int64_t)total_q / rb + p.num_seqs;
+      p.compact = comp < plain ? 1 : 0;
+      return p.compact ? dim3((unsigned)comp, heads, 1) : dim3((unsigned)((rows + rb - 1) / rb), heads, (unsigned)p.num_seqs);
+    };
+    dim3 grid = row_grid(rpb, (unsigned)(p.Hq / hpw));
     if constexpr (DK == 128 && DV == 128) {
       // K and V through LDS, shared by the 16 query tiles of a block
       int hp = 1;
       while (hp * 2 <= 8 && G % (hp * 2) == 0) hp *= 2;
       const int rb = 16 * (PFL_SLOTS / hp);
-      const dim3 lgrid((rows + rb - 1) / rb, p.Hq / hp, p.num_seqs);
+      const dim3 lgrid = row_grid(rb, (unsigned)(p.Hq / hp));
       static DeviceOnce once;
       const int dev = once.slot();
       if (once.need(dev)) {
