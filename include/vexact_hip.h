@@ -312,6 +312,14 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
                           void* k_cache, void* v_cache, int64_t T, int Hq, int Hkv, int D, float eps,
                           int64_t max_pos, int page_size, int64_t cache_block_stride,
                           int64_t cache_row_stride, int64_t cache_head_stride, hipStream_t stream);
+/* Rotary embedding alone, bf16: out[t, h, :] = r16(r16(x cos[t]) + r16(rotate_half(x) sin[t])) for x [T, H, D]
+ * with element strides (token, head; D contiguous, D % 8 == 0) and per-token rows cos / sin [T, D] (row stride
+ * cos_row_stride). One launch for what HuggingFace's apply_rotary_pos_emb (transformers modeling_qwen3_moe.py,
+ * called between q/k norm and the attention function that the reference registers) does in five per tensor;
+ * the reference's optional Liger patch swaps the same function (vexact/models/register.py:77-80). Same bits. */
+int vx_rope(const void* x, void* out, const void* cos_rows, const void* sin_rows, int64_t T, int H, int D,
+            int64_t x_token_stride, int64_t x_head_stride, int64_t out_token_stride, int64_t out_head_stride,
+            int64_t cos_row_stride, hipStream_t stream);
 int vx_embedding(const void* table, const void* ids, int ids_i64, void* out, int64_t T, int64_t H,
                  int64_t vocab, hipStream_t stream);
 int vx_fill_i32(int* p, int value, int64_t n, hipStream_t stream);

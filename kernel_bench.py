@@ -7,7 +7,7 @@ out, and the replay is timed with events. Prints time, algorithmic bytes (or flo
 fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
 to run under ``rocprofv3 --pmc``.
 
-    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,other,configs,mfma,copy
+    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,other,configs,mfma,copy,dropin
 """
 
 from __future__ import annotations
@@ -408,12 +408,105 @@ def run(a, quiet: bool = False) -> list:
                 xx = torch.randn(M, 4096, generator=g, device=dev).to(dt)
                 ww = (torch.randn(4096, 4096, generator=g, device=dev) * 0.02).to(dt)
                 report(f"{nm} gemm M={M} N=4096 K=4096", timeit(lambda li: ops.matmul(xx, ww.t()), n_layers=2), flops=2 * M * 4096 * 4096)
+    if "dropin" in what:
+        results.extend(dropin_decode(a, quiet))
     if "copy" in what:
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
         report("copy 1 GiB", timeit(lambda li: dst.copy_(src), n_layers=2), 2 << 30)
     return results
+
+
+def dropin_decode(a, quiet: bool = False) -> list:
+    """What a caller of the reference gets by switching imports: a HuggingFace ``Qwen3MoeForCausalLM`` of the
+    30B-A3B shape (random weights, built on the GPU) behind the registered attention function, the patched MoE
+    block and batch-invariant mode, one decode step of ``--batch`` sequences (contexts U[256, 2048], page 16)
+    captured in a HIP graph - once with ``max_seqlen_q = 1`` and once the way the reference's CudaGraphManager
+    captures it (``max_seqlen_q`` = the bucket's tokens, vexact/inferencer/cudagraph_utils.py:163)."""
+    import types
+
+    import numpy as np
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+    from transformers.models.qwen3_moe.configuration_qwen3_moe import Qwen3MoeConfig
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeForCausalLM
+
+    from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
+    from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches
+
+    say = (lambda *x, **k: None) if quiet else print
+    B, page = a.batch, a.page
+    cfg = Qwen3MoeConfig(vocab_size=151936, hidden_size=2048, intermediate_size=6144, num_hidden_layers=48,
+                         num_attention_heads=32, num_key_value_heads=4, head_dim=128, num_experts=128, num_experts_per_tok=8,
+                         moe_intermediate_size=768, norm_topk_prob=True, max_position_embeddings=40960, rms_norm_eps=1e-6,
+                         rope_parameters={"rope_type": "default", "rope_theta": 1.0e6})
+    cfg._attn_implementation = "triton-invariant"
+    ALL_ATTENTION_FUNCTIONS["triton-invariant"] = flash_attention_forward
+    apply_qwen3_moe_patches()
+    with torch.device("meta"):
+        model = Qwen3MoeForCausalLM(cfg)
+    model = model.to_empty(device="cuda").eval()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if "norm" in name:
+                p.fill_(1.0)
+            else:
+                p.normal_(0.0, 0.02, generator=g)
+    for p in model.parameters():
+        p.data = p.data.to(torch.bfloat16)
+    rot = model.model.rotary_emb  # inv_freq is a non-persistent buffer, which to_empty() leaves uninitialised
+    inv = 1.0 / (1.0e6 ** (torch.arange(0, 128, 2, device="cuda").float() / 128))
+    rot.inv_freq, rot.original_inv_freq = inv, inv.clone()
+    for layer in model.model.layers:
+        layer.mlp.experts.pack_for_decode()
+    rng = np.random.default_rng(5)
+    lens = rng.integers(256, 2049, size=B)
+    pages = [(int(n) + 2 + page - 1) // page for n in lens]
+    pool = sum(pages) + 8
+    store = KVCacheStore(cfg, types.SimpleNamespace(page_size=page, max_cache_blocks=pool), torch.device("cuda"))
+    for t in list(store.key_cache.values()) + list(store.value_cache.values()):
+        t.normal_(0, 1)
+    perm, bt, o = rng.permutation(pool), np.zeros((B, max(pages)), np.int32), 0
+    for i, pg in enumerate(pages):
+        bt[i, :pg] = perm[o:o + pg]
+        o += pg
+    i32 = dict(dtype=torch.int32, device="cuda")
+    ids = torch.randint(0, cfg.vocab_size, (1, B), device="cuda")
+    pos = torch.as_tensor(lens, device="cuda").long()[None]
+    bt_d, ctx = torch.as_tensor(bt).cuda(), torch.as_tensor(lens + 1, **i32)
+    slot = torch.as_tensor([bt[i, lens[i] // page] * page + lens[i] % page for i in range(B)], **i32)
+    qsl = torch.arange(B + 1, **i32)
+
+    def forward():
+        out = model.model(input_ids=ids, position_ids=pos, use_cache=False, return_dict=True)
+        return model.lm_head(out.last_hidden_state)
+
+    res = []
+    for msq, how in ((1, "max_seqlen_q = 1"), (B, "max_seqlen_q = bucket tokens")):
+        set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache, block_tables=bt_d,
+                             context_lens=ctx, slot_mapping=slot, query_start_loc=qsl, max_seqlen_q=msq)
+        try:
+            with torch.inference_mode(), set_batch_invariant_mode(True):
+                forward()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    forward()
+                for _ in range(3):
+                    graph.replay()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(10):
+                    graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+        finally:
+            clear_kv_cache_context()
+        ms = e0.elapsed_time(e1) / 10
+        say(f"HF Qwen3MoeForCausalLM drop-in decode, batch {B}, {how}: {ms:.2f} ms/step = {B / ms * 1e3:.0f} tok/s", flush=True)
+        res.append({"name": f"HF drop-in decode step, batch {B}, {how}", "us": round(ms * 1e3, 1), "tok_s": round(B / ms * 1e3)})
+    return res
 
 
 def main() -> None:

@@ -285,3 +285,71 @@ def test_huggingface_decode_step_captured_the_way_the_reference_captures_it():
         else:
             ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had
 
+
+def test_fused_rms_norm_patch_gives_the_bits_of_the_unfused_forward():
+    # Qwen3MoeRMSNorm.forward replaced by one kernel: hidden-size rows and head-size rows (q / k norm), bf16 and fp16,
+    # against HuggingFace's own forward run under batch-invariant mode
+    from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
+
+    from vexact_amd.batch_invariant_ops import set_batch_invariant_mode
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+    from vexact_amd.models.qwen3_moe.modeling_qwen3_moe import fused_rms_norm_forward
+
+    original = hf.Qwen3MoeRMSNorm.forward
+    apply_qwen3_moe_patches()
+    try:
+        assert hf.Qwen3MoeRMSNorm.forward is fused_rms_norm_forward
+        g = torch.Generator().manual_seed(3)
+        for shape, dtype in (((1, 37, 2048), BF), ((1, 9, 32, 128), BF), ((256, 2048), BF), ((1, 5, 4, 128), torch.float16),
+                             ((3, 200), BF)):
+            norm = hf.Qwen3MoeRMSNorm(shape[-1], eps=1e-6)
+            with torch.no_grad():
+                norm.weight.copy_(1.0 + 0.2 * torch.randn(shape[-1], generator=g))
+            norm = norm.to(dtype).cuda()
+            x = (3.0 * torch.randn(shape, generator=g)).to(dtype).cuda()
+            with torch.inference_mode(), set_batch_invariant_mode(True):
+                fused = norm(x)
+                unfused = original(norm, x)
+            assert fused.shape == unfused.shape and fused.dtype == unfused.dtype
+            assert_bitwise(fused, unfused, f"fused RMSNorm forward, shape {shape}, {dtype}")
+            with torch.inference_mode():  # outside the mode the original forward runs
+                assert_bitwise(norm(x), original(norm, x), "outside batch-invariant mode")
+    finally:
+        remove_qwen3_moe_patches()
+    assert hf.Qwen3MoeRMSNorm.forward is original
+
+
+def test_fused_rope_patch_gives_the_bits_of_apply_rotary_pos_emb():
+    from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
+
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+    from vexact_amd.models.qwen3_moe.modeling_qwen3_moe import fused_apply_rotary_pos_emb
+
+    original = hf.apply_rotary_pos_emb
+    apply_qwen3_moe_patches()
+    try:
+        assert hf.apply_rotary_pos_emb is fused_apply_rotary_pos_emb
+        g = torch.Generator().manual_seed(5)
+        for B, T, Hq, Hkv, D in ((1, 300, 32, 4, 128), (1, 1, 4, 2, 128), (3, 17, 8, 8, 64), (1, 40, 6, 2, 96)):
+            # the attention module's layout: projections [B, T, heads, D] seen as [B, heads, T, D]
+            q = (2.0 * torch.randn(B, T, Hq, D, generator=g)).to(BF).cuda().transpose(1, 2)
+            k = (2.0 * torch.randn(B, T, Hkv, D, generator=g)).to(BF).cuda().transpose(1, 2)
+            ang = 50.0 * torch.rand(B, T, D // 2, generator=g)
+            cos = torch.cat([ang.cos(), ang.cos()], -1).to(BF).cuda()
+            sin = torch.cat([ang.sin(), ang.sin()], -1).to(BF).cuda()
+            with torch.inference_mode():
+                fq, fk = hf.apply_rotary_pos_emb(q, k, cos, sin)
+                oq, ok = original(q, k, cos, sin)
+            assert fq.shape == oq.shape and fk.shape == ok.shape
+            assert_bitwise(fq, oq, f"rotated queries, B={B} T={T} D={D}")
+            assert_bitwise(fk, ok, f"rotated keys, B={B} T={T} D={D}")
+        # what the kernel does not take falls through to the original (fp32 here)
+        q = torch.randn(1, 2, 5, 64, device="cuda"); k = torch.randn(1, 2, 5, 64, device="cuda")
+        cos = torch.randn(1, 5, 64, device="cuda"); sin = torch.randn(1, 5, 64, device="cuda")
+        fq, fk = hf.apply_rotary_pos_emb(q, k, cos, sin)
+        oq, ok = original(q, k, cos, sin)
+        assert torch.equal(fq, oq) and torch.equal(fk, ok)
+    finally:
+        remove_qwen3_moe_patches()
+    assert hf.apply_rotary_pos_emb is original
+

@@ -66,6 +66,7 @@ PROTOTYPES = {
         _I,
         [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _F, _L, _I, _L, _L, _L, _P],
     ),
+    "vx_rope": (_I, [_P, _P, _P, _P, _L, _I, _I, _L, _L, _L, _L, _L, _P]),
     "vx_embedding": (_I, [_P, _P, _I, _P, _L, _L, _L, _P]),
     "vx_fill_i32": (_I, [_P, _I, _L, _P]),
     "vx_sample_tokens": (_I, [_P, _I, _L, _L, _L, _F, _I, _F, _P, _P, _P, _P]),

@@ -115,6 +115,41 @@ __global__ __launch_bounds__(256) void embedding_kernel(const bf16_t* __restrict
   for (int c = threadIdx.x; c < H / 8; c += 256) dst[c] = src[c];
 }
 
+// Rotary embedding of [T, H, D] rows from per-token cos / sin rows [T, D], HuggingFace's apply_rotary_pos_emb:
+// out = r16(r16(x cos) + r16(rotate_half(x) sin)), rotate_half(x) = (-x[D/2:], x[:D/2]). One thread per group of
+// 4 elements of the first half and their 4 partners in the second half.
+__global__ __launch_bounds__(256) void rope_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out,
+                                                   const bf16_t* __restrict__ cos_r, const bf16_t* __restrict__ sin_r,
+                                                   int64_t items, int H, int D, int64_t sxt, int64_t sxh, int64_t sot,
+                                                   int64_t soh, int64_t scs) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= items) return;
+  const int per = D / 8;  // threads per (token, head)
+  const int c4 = (int)(i % per) * 4;
+  const int64_t th = i / per;
+  const int h = (int)(th % H);
+  const int64_t t = th / H;
+  const bf16_t* xp = x + t * sxt + (int64_t)h * sxh;
+  const uint2 a = *(const uint2*)(xp + c4), b = *(const uint2*)(xp + D / 2 + c4);
+  const uint2 ca = *(const uint2*)(cos_r + t * scs + c4), cb = *(const uint2*)(cos_r + t * scs + D / 2 + c4);
+  const uint2 sa = *(const uint2*)(sin_r + t * scs + c4), sb = *(const uint2*)(sin_r + t * scs + D / 2 + c4);
+  const float x1[4] = {bf16lo(a.x), bf16hi(a.x), bf16lo(a.y), bf16hi(a.y)};
+  const float x2[4] = {bf16lo(b.x), bf16hi(b.x), bf16lo(b.y), bf16hi(b.y)};
+  const float c1[4] = {bf16lo(ca.x), bf16hi(ca.x), bf16lo(ca.y), bf16hi(ca.y)};
+  const float c2[4] = {bf16lo(cb.x), bf16hi(cb.x), bf16lo(cb.y), bf16hi(cb.y)};
+  const float s1[4] = {bf16lo(sa.x), bf16hi(sa.x), bf16lo(sa.y), bf16hi(sa.y)};
+  const float s2[4] = {bf16lo(sb.x), bf16hi(sb.x), bf16lo(sb.y), bf16hi(sb.y)};
+  float o1[4], o2[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    o1[c] = bf16_to_f32(f32_to_bf16(x1[c] * c1[c])) + bf16_to_f32(f32_to_bf16(-x2[c] * s1[c]));
+    o2[c] = bf16_to_f32(f32_to_bf16(x2[c] * c2[c])) + bf16_to_f32(f32_to_bf16(x1[c] * s2[c]));
+  }
+  bf16_t* op = out + t * sot + (int64_t)h * soh;
+  *(uint2*)(op + c4) = make_uint2(pack_bf16x2(o1[0], o1[1]), pack_bf16x2(o1[2], o1[3]));
+  *(uint2*)(op + D / 2 + c4) = make_uint2(pack_bf16x2(o2[0], o2[1]), pack_bf16x2(o2[2], o2[3]));
+}
+
 __global__ __launch_bounds__(256) void fill_i32_kernel(int* p, int v, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) p[i] = v;
@@ -156,6 +191,23 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
   if (D == 128) { if (pos_i64) VX_QK(128, int64_t); else VX_QK(128, int); }
   else { if (pos_i64) VX_QK(64, int64_t); else VX_QK(64, int); }
 #undef VX_QK
+  return launch_status();
+}
+
+int vx_rope(const void* x, void* out, const void* cos_rows, const void* sin_rows, int64_t T, int H, int D,
+            int64_t x_token_stride, int64_t x_head_stride, int64_t out_token_stride, int64_t out_head_stride,
+            int64_t cos_row_stride, hipStream_t stream) {
+  if (!x || !out || !cos_rows || !sin_rows || T < 0 || H <= 0 || D <= 0) return VX_ERR_ARG;
+  if (D % 8 != 0) return VX_ERR_UNSUPPORTED;
+  if ((x_token_stride | x_head_stride | out_token_stride | out_head_stride | cos_row_stride) % 4 != 0) return VX_ERR_UNSUPPORTED;
+  if (((uintptr_t)x | (uintptr_t)out | (uintptr_t)cos_rows | (uintptr_t)sin_rows) % 8 != 0) return VX_ERR_UNSUPPORTED;
+  if (T == 0) return VX_OK;
+  const int64_t items = T * H * (D / 8);
+  const int64_t blocks = (items + 255) / 256;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  rope_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, (const bf16_t*)cos_rows,
+                                                    (const bf16_t*)sin_rows, items, H, D, x_token_stride, x_head_stride,
+                                                    out_token_stride, out_head_stride, cos_row_stride);
   return launch_status();
 }
 

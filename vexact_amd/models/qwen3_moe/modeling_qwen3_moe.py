@@ -130,25 +130,86 @@ def invalidate_packed_experts(model: nn.Module) -> int:
     return n
 
 
-def apply_qwen3_moe_patches() -> None:
-    """Swap the HuggingFace block's constructor and forward (idempotent)."""
-    global _ORIGINAL
-    if _ORIGINAL is not None:
-        return
-    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeSparseMoeBlock
+def fused_rms_norm_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+    """``Qwen3MoeRMSNorm.forward`` as one kernel. HuggingFace's forward (cast to fp32, ``pow(2).mean(-1)``, ``rsqrt``,
+    two multiplies and two casts: eleven launches under batch-invariant mode) rounds ``x * rsqrt(var + eps)`` to
+    the input dtype and then multiplies by the weight; ``ops.rms_norm(..., hf_two_rounding=True)`` keeps both
+    roundings and the batch-invariant mean's summation order, so the bits are the ones the unfused forward gives
+    under ``set_batch_invariant_mode(True)``. Outside that mode, off the GPU or with a weight of another dtype
+    the original forward runs."""
+    from ...batch_invariant_ops import is_batch_invariant_mode_enabled
 
-    _ORIGINAL = (Qwen3MoeSparseMoeBlock.__init__, Qwen3MoeSparseMoeBlock.forward)
-    Qwen3MoeSparseMoeBlock.__init__ = moe_block_init
-    Qwen3MoeSparseMoeBlock.forward = moe_block_forward
+    w = self.weight
+    if (hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float16) and w.dtype == hidden_states.dtype
+            and not (torch.is_grad_enabled() and (hidden_states.requires_grad or w.requires_grad))
+            and is_batch_invariant_mode_enabled()):
+        return ops.rms_norm(hidden_states, w, self.variance_epsilon, hf_two_rounding=True)
+    return _ORIGINAL_NORM(self, hidden_states)
+
+
+_ORIGINAL_NORM = None  # Qwen3MoeRMSNorm.forward while the fused form is patched in
+_ORIGINAL_ROPE = None  # the module's apply_rotary_pos_emb while the fused form is patched in
+
+
+def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **kwargs):
+    """``apply_rotary_pos_emb`` of HuggingFace's Qwen3-MoE modeling file as one launch per tensor instead of five
+    (multiply, negate, concatenate, multiply, add). ``q`` / ``k`` are ``[B, heads, T, D]`` views of ``[B, T, heads, D]``
+    projections, ``cos`` / ``sin`` ``[B, T, D]``. Elementwise with the same bf16 roundings, so the bits do not change
+    in any mode; other layouts, dtypes or autograd fall through to the original."""
+    def fits(x):
+        return (x.dim() == 4 and x.is_cuda and x.dtype == torch.bfloat16 and x.stride(3) == 1 and x.shape[3] % 8 == 0
+                and (x.shape[0] == 1 or x.stride(0) == x.shape[2] * x.stride(2)) and x.stride(1) % 4 == 0 and x.stride(2) % 4 == 0)
+
+    if (not args and not kwargs and unsqueeze_dim == 1 and fits(q) and fits(k) and cos.dim() == 3 and cos.dtype == torch.bfloat16
+            and sin.dtype == torch.bfloat16 and cos.shape == sin.shape and cos.shape[0] == q.shape[0] == k.shape[0]
+            and cos.shape[1] == q.shape[2] == k.shape[2] and cos.shape[2] == q.shape[3] == k.shape[3]
+            and not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad))):
+        B, _, T, D = q.shape
+        c2, s2 = cos.reshape(B * T, D), sin.reshape(B * T, D)
+
+        def one(x):
+            H = x.shape[1]
+            rows = x.transpose(1, 2)  # [B, T, H, D]
+            flat = rows.as_strided((B * T, H, D), (rows.stride(1), rows.stride(2), 1), rows.storage_offset())
+            return ops.rope(flat, c2, s2).view(B, T, H, D).transpose(1, 2)
+
+        return one(q), one(k)
+    return _ORIGINAL_ROPE(q, k, cos, sin, *args, unsqueeze_dim=unsqueeze_dim, **kwargs)
+
+
+def apply_qwen3_moe_patches(fused_rms_norm: bool = True, fused_rope: bool = True) -> None:
+    """Swap the HuggingFace block's constructor and forward (idempotent). ``fused_rms_norm`` also replaces
+    ``Qwen3MoeRMSNorm.forward`` by ``fused_rms_norm_forward`` (same bits under batch-invariant mode, one launch
+    instead of eleven; not in the reference, whose optional Liger patch leaves RMSNorm alone because Liger's is
+    not batch invariant, vexact/models/register.py:84-87) and ``fused_rope`` the modeling file's
+    ``apply_rotary_pos_emb`` by ``fused_apply_rotary_pos_emb`` (the function that Liger patch swaps, :77-80)."""
+    global _ORIGINAL, _ORIGINAL_NORM, _ORIGINAL_ROPE
+    from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
+
+    if _ORIGINAL is None:
+        _ORIGINAL = (hf.Qwen3MoeSparseMoeBlock.__init__, hf.Qwen3MoeSparseMoeBlock.forward)
+        hf.Qwen3MoeSparseMoeBlock.__init__ = moe_block_init
+        hf.Qwen3MoeSparseMoeBlock.forward = moe_block_forward
+    if fused_rms_norm and _ORIGINAL_NORM is None:
+        _ORIGINAL_NORM = hf.Qwen3MoeRMSNorm.forward
+        hf.Qwen3MoeRMSNorm.forward = fused_rms_norm_forward
+    if fused_rope and _ORIGINAL_ROPE is None:
+        _ORIGINAL_ROPE = hf.apply_rotary_pos_emb
+        hf.apply_rotary_pos_emb = fused_apply_rotary_pos_emb
 
 
 def remove_qwen3_moe_patches() -> None:
     """Put the HuggingFace block's own constructor and forward back (blocks built meanwhile keep their fused
     experts and stop working with the original forward; meant for tests and tools that need both forms)."""
-    global _ORIGINAL
-    if _ORIGINAL is None:
-        return
-    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeSparseMoeBlock
+    global _ORIGINAL, _ORIGINAL_NORM, _ORIGINAL_ROPE
+    from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
 
-    Qwen3MoeSparseMoeBlock.__init__, Qwen3MoeSparseMoeBlock.forward = _ORIGINAL
-    _ORIGINAL = None
+    if _ORIGINAL_ROPE is not None:
+        hf.apply_rotary_pos_emb = _ORIGINAL_ROPE
+        _ORIGINAL_ROPE = None
+    if _ORIGINAL is not None:
+        hf.Qwen3MoeSparseMoeBlock.__init__, hf.Qwen3MoeSparseMoeBlock.forward = _ORIGINAL
+        _ORIGINAL = None
+    if _ORIGINAL_NORM is not None:
+        hf.Qwen3MoeRMSNorm.forward = _ORIGINAL_NORM
+        _ORIGINAL_NORM = None

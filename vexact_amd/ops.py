@@ -30,8 +30,28 @@ def _need_gpu(name: str, t: torch.Tensor) -> None:
         raise ValueError(f"{name} must be a CUDA tensor")
 
 
+def _empty(*size, **kw) -> torch.Tensor:
+    """``torch.empty`` for a tensor that the kernel about to be launched writes completely. Under
+    ``torch.use_deterministic_algorithms(True)`` (which ``enable_batch_invariant_mode`` turns on, as the
+    reference's does) ``torch.empty`` fills what it returns with NaN, one more kernel in front of every op here
+    (about 3 us each, some twenty per decoder layer); that fill is skipped for these tensors, whose every
+    element is overwritten anyway. Attention outputs keep it: rows of a sequence without any key stay unwritten."""
+    det = torch.utils.deterministic
+    if torch.are_deterministic_algorithms_enabled() and det.fill_uninitialized_memory:
+        det.fill_uninitialized_memory = False
+        try:
+            return torch.empty(*size, **kw)
+        finally:
+            det.fill_uninitialized_memory = True
+    return torch.empty(*size, **kw)
+
+
+def _empty_like(t: torch.Tensor) -> torch.Tensor:
+    return _empty(t.shape, dtype=t.dtype, device=t.device)
+
+
 def _workspace(nbytes: int, device) -> torch.Tensor:
-    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+    return _empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
 
 # ----------------------------------------------------------------------------- row ops
@@ -61,7 +81,7 @@ def mean_dim(x: torch.Tensor, dim: int, keepdim: bool = False, dtype: Optional[t
         out_shape[dim] = 1
     else:
         out_shape = shape[:dim] + shape[dim + 1 :]
-    out = torch.empty(out_shape, dtype=dtype, device=x.device)
+    out = _empty(out_shape, dtype=dtype, device=x.device)
     if M * K == 0:
         return out
     if N == 0:
@@ -99,7 +119,7 @@ def rms_norm(
     if w.dtype != x.dtype:
         w = w.to(x.dtype)
     assert w.numel() == n, "weight must have the size of the last dim"
-    y = out if out is not None else torch.empty((x2.shape[0], n), dtype=x.dtype, device=x.device)
+    y = out if out is not None else _empty((x2.shape[0], n), dtype=x.dtype, device=x.device)
     y2 = y.reshape(-1, n)
     r2 = s2 = None
     if residual is not None:
@@ -128,7 +148,7 @@ def log_softmax(x: torch.Tensor, dim: int = -1) -> torch.Tensor:
     shape = x.shape
     x2 = x.reshape(-1, shape[-1]).contiguous()
     rows, n = x2.shape
-    y = torch.empty_like(x2)
+    y = _empty_like(x2)
     if rows == 0 or n == 0:
         return y.reshape(shape)
     lib = _lib.load()
@@ -158,8 +178,8 @@ def logprobs(
     if x2.stride(-1) != 1:
         x2 = x2.contiguous()
     rows, n = x2.shape
-    out = torch.empty(rows, dtype=torch.float32, device=logits.device)
-    toks = torch.empty(rows, dtype=torch.int64, device=logits.device) if (return_tokens or labels is None) else None
+    out = _empty(rows, dtype=torch.float32, device=logits.device)
+    toks = _empty(rows, dtype=torch.int64, device=logits.device) if (return_tokens or labels is None) else None
     lab = None
     if labels is not None:
         lab = labels.reshape(-1)
@@ -204,7 +224,7 @@ def sample_tokens(
         if t.dtype != torch.int64 or t.numel() != B or not t.is_contiguous() or t.device != logits.device:
             raise ValueError(f"sample_tokens: {name} must be a contiguous int64 [B] tensor on the logits' device")
     if out is None:
-        out = torch.empty(B, dtype=torch.int64, device=logits.device)
+        out = _empty(B, dtype=torch.int64, device=logits.device)
     _lib.check(
         _lib.load().vx_sample_tokens(
             logits.data_ptr(), 0 if logits.dtype == torch.bfloat16 else 1, logits.stride(0), B, V, float(temperature),
@@ -240,7 +260,7 @@ def gemm_nt(
     """``x[M,K] @ w_nk[N,K].T (+ bias)`` in bf16 on the MFMA path (raises if the layout does not fit)."""
     M, K = x.shape
     N = w_nk.shape[0]
-    c = out if out is not None else torch.empty((M, N), dtype=x.dtype, device=x.device)
+    c = out if out is not None else _empty((M, N), dtype=x.dtype, device=x.device)
     assert c.stride(1) == 1
     _lib.check(
         _lib.load().vx_gemm_bf16_nt(
@@ -255,7 +275,7 @@ def gemm_nt(
 def gemm_nt_variant(x: torch.Tensor, w_nk: torch.Tensor, kind: int, mt: int = 1, bias=None) -> torch.Tensor:
     M, K = x.shape
     N = w_nk.shape[0]
-    c = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    c = _empty((M, N), dtype=x.dtype, device=x.device)
     _lib.check(
         _lib.load().vx_gemm_bf16_nt_variant(
             x.data_ptr(), w_nk.data_ptr(), _ptr(bias), c.data_ptr(), M, N, K, x.stride(0), w_nk.stride(0),
@@ -276,7 +296,7 @@ def gemm_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, out: 
     M, K = x.shape
     N = w_gate.shape[0]
     if out is None:
-        out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+        out = _empty(M, N, dtype=torch.bfloat16, device=x.device)
     _lib.check(
         _lib.load().vx_gemm_swiglu_bf16_nt(x.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(), out.data_ptr(), M, N, K,
                                            x.stride(0), w_gate.stride(0), out.stride(0), kind, mt, _stream()),
@@ -309,7 +329,7 @@ def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None
     N = b.shape[1]
     if bias is not None:
         bias = bias.to(a.dtype).contiguous()
-    c = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    c = _empty((M, N), dtype=a.dtype, device=a.device)
     if M == 0 or N == 0:
         return c
     if K == 0:
@@ -326,7 +346,7 @@ def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None
         if w_nk.stride(1) != 1 or w_nk.stride(0) % 8 != 0 or w_nk.data_ptr() % 16 != 0:
             # pack b[K, N] (any strides) into an [N, K] row-major buffer
             bc = b if b.stride(1) == 1 else b.contiguous()
-            packed = torch.empty((N, K), dtype=b.dtype, device=b.device)
+            packed = _empty((N, K), dtype=b.dtype, device=b.device)
             _lib.check(
                 lib.vx_transpose_bf16(bc.data_ptr(), packed.data_ptr(), K, N, bc.stride(0), K, _stream()),
                 "vx_transpose_bf16",
@@ -362,7 +382,7 @@ def bmm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     _need_gpu("a", a)
     if a.dtype not in _DT or a.dtype != b.dtype:
         raise ValueError(f"bmm: unsupported dtypes {a.dtype}, {b.dtype}")
-    c = torch.empty((B, M, N), dtype=a.dtype, device=a.device)
+    c = _empty((B, M, N), dtype=a.dtype, device=a.device)
     if c.numel() == 0:
         return c
     lib = _lib.load()
@@ -509,7 +529,7 @@ def packed_attention_backward(
         raise ValueError(f"attention backward supports equal q/k/v head sizes of 64 or 128, got {D} and {Dv}")
     if lse.dtype != torch.float32 or lse.shape != (T, Hq) or not lse.is_contiguous():
         raise ValueError("attention backward: lse must be a contiguous fp32 [tokens, heads] tensor")
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dq, dk, dv = _empty_like(q), _empty_like(k), _empty_like(v)
     if T == 0 or Tk == 0:
         return dq.zero_(), dk.zero_(), dv.zero_()
     lib = _lib.load()
@@ -542,8 +562,8 @@ def router_topk(
     if out_dtype not in (torch.float32, torch.bfloat16) or index_dtype not in (torch.int32, torch.int64):
         raise ValueError("unsupported router output dtypes")
     lg = logits if logits.stride(1) == 1 else logits.contiguous()
-    w = torch.empty((T, top_k), dtype=out_dtype, device=logits.device)
-    idx = torch.empty((T, top_k), dtype=index_dtype, device=logits.device)
+    w = _empty((T, top_k), dtype=out_dtype, device=logits.device)
+    idx = _empty((T, top_k), dtype=index_dtype, device=logits.device)
     _lib.check(
         _lib.load().vx_router_topk(
             lg.data_ptr(), w.data_ptr(), idx.data_ptr(), T, E, top_k, lg.stride(0),
@@ -593,7 +613,7 @@ def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int
     r.T, r.k, r.E, r.bm, r.max_tiles = T, k, num_experts, bm, max_tiles
     n = T * k
     if buffers is None:
-        ints = torch.empty(num_experts + (num_experts + 1) + 3 * n + 3 * max_tiles, dtype=torch.int32, device=dev)
+        ints = _empty(num_experts + (num_experts + 1) + 3 * n + 3 * max_tiles, dtype=torch.int32, device=dev)
     else:
         ints = buffers
     o = 0
@@ -632,7 +652,7 @@ def moe_gemm(
     assert x.stride(1) == 1 and w.stride(2) == 1
     if w2 is not None:
         assert w2.shape == w.shape and w2.stride() == w.stride() and row_scale is not None
-    c = out if out is not None else torch.empty((n_rows, N), dtype=torch.bfloat16, device=x.device)
+    c = out if out is not None else _empty((n_rows, N), dtype=torch.bfloat16, device=x.device)
     _lib.check(
         _lib.load().vx_moe_gemm(
             x.data_ptr(), x.stride(0), w.data_ptr(), _ptr(w2), w.stride(1), w.stride(0), c.data_ptr(), c.stride(0),
@@ -674,7 +694,7 @@ def pack_expert_weights(w: torch.Tensor) -> PackedExpertWeights:
     lib = _lib.load()
     pk = PackedExpertWeights()
     pk.E, pk.N, pk.K, pk.kchunks, pk.row0, pk.rows_n = E, N, K, lib.vx_packed_kchunks(K), 0, N
-    pk.data = torch.empty(E * pk.gstride, dtype=torch.bfloat16, device=w.device)
+    pk.data = _empty(E * pk.gstride, dtype=torch.bfloat16, device=w.device)
     _lib.check(lib.vx_pack_weights(w.data_ptr(), w.stride(1), w.stride(0), E, N, K, pk.data.data_ptr(), _stream()),
                "vx_pack_weights")
     return pk
@@ -702,7 +722,7 @@ def moe_gemm_packed(
     if w2 is not None:
         assert w2.data is w.data and w2.rows_n == w.rows_n and row_scale is not None
     N = w.rows_n
-    c = out if out is not None else torch.empty((n_rows, N), dtype=torch.bfloat16, device=x.device)
+    c = out if out is not None else _empty((n_rows, N), dtype=torch.bfloat16, device=x.device)
     _lib.check(
         _lib.load().vx_moe_gemm_packed(
             x.data_ptr(), x.stride(0), w.data_ptr(), w2.data_ptr() if w2 is not None else None, w.gstride,
@@ -733,7 +753,7 @@ def moe_gemm_nn(
         assert a2.shape == (n_rows, K2) and w2.shape[0] == E and w2.shape[2] == N
     if a_src is not None:
         assert a_src.dtype == torch.int32 and a_src.is_contiguous() and a_src.numel() == n_rows
-    c = out if out is not None else torch.empty((n_rows, N), dtype=torch.bfloat16, device=a.device)
+    c = out if out is not None else _empty((n_rows, N), dtype=torch.bfloat16, device=a.device)
     _lib.check(
         _lib.load().vx_moe_gemm_nn(
             a.data_ptr(), a.stride(0), _ptr(a_src), w.data_ptr(), w.stride(1), w.stride(0), K,
@@ -758,7 +778,7 @@ def moe_gemm_tn(
     assert cu.dtype == torch.int32 and cu.is_contiguous() and cu.numel() == num_experts + 1
     for src in (dy_src, x_src):
         assert src is None or (src.dtype == torch.int32 and src.is_contiguous())
-    dw = out if out is not None else torch.empty((num_experts, N, K), dtype=torch.bfloat16, device=dy.device)
+    dw = out if out is not None else _empty((num_experts, N, K), dtype=torch.bfloat16, device=dy.device)
     assert dw.shape == (num_experts, N, K) and dw.stride(2) == 1
     _lib.check(
         _lib.load().vx_moe_gemm_tn(
@@ -775,7 +795,7 @@ def expert_histogram(idx: torch.Tensor, num_bins: int) -> torch.Tensor:
     assert idx.dtype == torch.int32 or idx.dtype == torch.int64
     assert idx.numel() < (1 << 31) - 1, "Too many elements."
     flat = idx.flatten().contiguous()
-    out = torch.empty(num_bins, dtype=torch.int32, device=idx.device)
+    out = _empty(num_bins, dtype=torch.int32, device=idx.device)
     _lib.check(
         _lib.load().vx_expert_histogram(flat.data_ptr(), int(flat.dtype == torch.int64), flat.numel(), num_bins,
                                         out.data_ptr(), _stream()),
@@ -794,7 +814,7 @@ def moe_scatter(x: torch.Tensor, index: torch.Tensor, out_dtype=None) -> torch.T
     topk = index.shape[1]
     idx = index.to(torch.int32).contiguous()
     xs = x if x.stride(1) == 1 else x.contiguous()
-    out = torch.empty(M * topk, N, dtype=x.dtype, device=x.device)
+    out = _empty(M * topk, N, dtype=x.dtype, device=x.device)
     _lib.check(
         _lib.load().vx_moe_scatter(xs.data_ptr(), out.data_ptr(), idx.data_ptr(), M, topk, N, xs.stride(0),
                                    out.stride(0), _stream()),
@@ -819,7 +839,7 @@ def moe_gather(x: torch.Tensor, index: torch.Tensor, out_dtype=None, residual: O
     N = x.shape[1]
     idx = index if (index.dtype == torch.int32 and index.is_contiguous()) else index.to(torch.int32).contiguous()
     xs = x if x.stride(1) == 1 else x.contiguous()
-    y = out if out is not None else torch.empty(M, N, dtype=x.dtype, device=x.device)
+    y = out if out is not None else _empty(M, N, dtype=x.dtype, device=x.device)
     assert (norm_weight is None) == (norm_out is None)
     pf_bytes = 0
     if prefetch is not None:
@@ -898,10 +918,29 @@ def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, cos_table, sin_table, positions,
     )
 
 
+def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """Rotary embedding of ``x [T, H, D]`` (bf16, D contiguous, any token / head strides) with per-token rows
+    ``cos`` / ``sin [T, D]``: HuggingFace's ``x * cos + rotate_half(x) * sin`` with its bf16 roundings, one
+    launch. Returns a contiguous ``[T, H, D]`` tensor."""
+    _need_gpu("x", x)
+    assert x.dim() == 3 and x.dtype == torch.bfloat16 and x.stride(2) == 1
+    T, H, D = x.shape
+    assert cos.shape == (T, D) and sin.shape == (T, D) and cos.dtype == torch.bfloat16 and sin.dtype == torch.bfloat16
+    if cos.stride(1) != 1 or sin.stride() != cos.stride():
+        cos, sin = cos.contiguous(), sin.contiguous()
+    out = _empty((T, H, D), dtype=x.dtype, device=x.device)
+    _lib.check(
+        _lib.load().vx_rope(x.data_ptr(), out.data_ptr(), cos.data_ptr(), sin.data_ptr(), T, H, D, x.stride(0), x.stride(1),
+                            out.stride(0), out.stride(1), cos.stride(0), _stream()),
+        "vx_rope",
+    )
+    return out
+
+
 def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     T = ids.numel()
     vocab, H = table.shape
-    o = out if out is not None else torch.empty((T, H), dtype=table.dtype, device=table.device)
+    o = out if out is not None else _empty((T, H), dtype=table.dtype, device=table.device)
     _lib.check(
         _lib.load().vx_embedding(table.data_ptr(), ids.data_ptr(), int(ids.dtype == torch.int64), o.data_ptr(), T, H,
                                  vocab, _stream()),
