@@ -288,3 +288,31 @@ def test_bench_hands_kernel_bench_every_option_it_reads():
     read = set(re.findall(r"\ba\.([a-z_]+)\b", inspect.getsource(kernel_bench.run)))
     assert read and all(hasattr(args, name) for name in read), sorted(n for n in read if not hasattr(args, n))
     assert "configs" in args.what and "mfma" in args.what
+
+
+def test_expert_tile_heights_and_unfilled_outputs():
+    import torch
+
+    from vexact_amd import ops
+
+    # tile height is a function of the token count; a model that holds fragment-order expert weights only never
+    # gets 128-row tiles (the one kernel that cannot read them)
+    assert [ops.moe_tile_rows(t) for t in (1, 256, 257, 1024, 1025, 2047, 2048, 100000)] == [32, 32, 64, 64, 128, 128, 256, 256]
+    assert [ops.moe_tile_rows(t, packed_only=True) for t in (256, 1024, 1025, 2047, 2048)] == [32, 64, 256, 256, 256]
+    assert ops.moe_tile_rows(5000, wide_ok=False) == 128 and ops.moe_tile_rows(5000, wide_ok=False, packed_only=True) == 64
+    # outputs that a kernel overwrites completely skip the NaN fill of deterministic mode and leave the switch as it was
+    was = torch.are_deterministic_algorithms_enabled()
+    try:
+        torch.use_deterministic_algorithms(True)
+        assert torch.utils.deterministic.fill_uninitialized_memory
+        assert bool(torch.empty(64).isnan().all())
+        t = ops._empty((3, 5), dtype=torch.float32, device="cpu")
+        assert t.shape == (3, 5) and torch.utils.deterministic.fill_uninitialized_memory
+        assert ops._empty_like(torch.zeros(4, dtype=torch.bfloat16)).dtype == torch.bfloat16
+        torch.utils.deterministic.fill_uninitialized_memory = False
+        ops._empty(2, dtype=torch.float32, device="cpu")
+        assert not torch.utils.deterministic.fill_uninitialized_memory
+    finally:
+        torch.utils.deterministic.fill_uninitialized_memory = True
+        torch.use_deterministic_algorithms(was)
+
