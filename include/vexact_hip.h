@@ -132,6 +132,15 @@ int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_
                      int64_t v_src_stride_bytes, int64_t k_row_bytes, int64_t v_row_bytes,
                      hipStream_t stream);
 
+/* The same scatter into caches that are [blocks, page_size, heads, D] views with the given byte strides (block,
+ * in-page row, head; a head's D elements contiguous), e.g. of head-major memory [blocks, heads, page_size, D], which
+ * the decode kernels stream faster than the reference's layout. slot = block * page_size + row. */
+int vx_store_kvcache_strided(const void* key, const void* value, void* k_cache, void* v_cache, const int* slot_mapping,
+                             int64_t num_tokens, int heads, int64_t k_src_stride_bytes, int64_t v_src_stride_bytes,
+                             int64_t k_head_bytes, int64_t v_head_bytes, int page_size, int64_t k_block_stride_bytes,
+                             int64_t k_row_stride_bytes, int64_t k_head_stride_bytes, int64_t v_block_stride_bytes,
+                             int64_t v_row_stride_bytes, int64_t v_head_stride_bytes, hipStream_t stream);
+
 /* Causal GQA attention, bf16, head dims (Dk, Dv) in {(32,32),(64,64),(128,128),(192,128),(256,256)}.
  *   mode 0: paged decode - every sequence has at most one query token; KV is split into fixed
  *           256-key chunks (absolute positions) and folded in ascending order; needs

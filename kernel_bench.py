@@ -38,6 +38,8 @@ def parse(argv=None):
                     help="physical KV cache layout: fused = [blocks, Hkv, 2, page, D] (what the decoder allocates), head = [blocks, Hkv, page, D] per tensor, token = [blocks, page, Hkv, D]")
     ap.add_argument("--page", type=int, default=16, help="KV cache page size (keys)")
     ap.add_argument("--nograph", action="store_true", help="eager launches only, no timing (for rocprofv3 --pmc)")
+    ap.add_argument("--dropin-head-major", action="store_true",
+                    help="section dropin: KVCacheStore(head_major=True) instead of the reference's cache layout")
     return ap.parse_args(argv)
 
 
@@ -465,7 +467,8 @@ def dropin_decode(a, quiet: bool = False) -> list:
     lens = rng.integers(256, 2049, size=B)
     pages = [(int(n) + 2 + page - 1) // page for n in lens]
     pool = sum(pages) + 8
-    store = KVCacheStore(cfg, types.SimpleNamespace(page_size=page, max_cache_blocks=pool), torch.device("cuda"))
+    store = KVCacheStore(cfg, types.SimpleNamespace(page_size=page, max_cache_blocks=pool), torch.device("cuda"),
+                         head_major=a.dropin_head_major)
     for t in list(store.key_cache.values()) + list(store.value_cache.values()):
         t.normal_(0, 1)
     perm, bt, o = rng.permutation(pool), np.zeros((B, max(pages)), np.int32), 0

@@ -232,6 +232,59 @@ def test_attention_wrapper_shape_and_cache_write():
     assert_bitwise(kc, full_k, "wrapper wrote the new keys")
 
 
+def test_head_major_cache_views_store_and_attend_like_the_reference_layout():
+    # KVCacheStore(head_major=True) hands out [blocks, page, heads, D] views of [blocks, heads, page, D] memory:
+    # the scatter writes the same elements (slot -1 skipped) and the wrapper's attention gives the same bits
+    import types
+
+    from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore
+
+    qh, kh, d, page = 8, 2, 128, 16
+    q_lens, past = [3, 1, 40, 1], [5, 200, 0, 77]
+    kv_lens = [p + n for p, n in zip(past, q_lens)]
+    q, k, v = _seqs(q_lens, qh, d, 60, 0.1), _seqs(kv_lens, kh, d, 61, 0.1), _seqs(kv_lens, kh, d, 62, 0.1)
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, page)
+    slots, newk, newv = [], [], []
+    for s, (p, n) in enumerate(zip(past, q_lens)):
+        for pos in range(p, p + n):
+            slots.append(int(table[s, pos // page]) * page + pos % page)
+            k_cache.view(-1, kh, d)[slots[-1]] = 0
+            v_cache.view(-1, kh, d)[slots[-1]] = 0
+        newk.append(k[s][p:])
+        newv.append(v[s][p:])
+    slots[1] = -1  # one token that must not be written (its zeroed slot stays zero in both layouts)
+    hf_cfg = types.SimpleNamespace(num_hidden_layers=1, num_key_value_heads=kh, head_dim=d, hidden_size=qh * d,
+                                   num_attention_heads=qh, dtype=torch.bfloat16)
+    cache_cfg = types.SimpleNamespace(page_size=page, max_cache_blocks=k_cache.shape[0])
+    outs, caches = [], []
+    for head_major in (False, True):
+        store = KVCacheStore(hf_cfg, cache_cfg, torch.device("cuda"), head_major=head_major)
+        kc, vc = store.key_cache[0], store.value_cache[0]
+        assert kc.shape == k_cache.shape and kc.is_contiguous() != head_major
+        kc.copy_(k_cache.cuda())
+        vc.copy_(v_cache.cuda())
+        set_kv_cache_context(
+            is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache, block_tables=table.cuda(),
+            context_lens=torch.tensor(kv_lens, dtype=torch.int32).cuda(),
+            slot_mapping=torch.tensor(slots, dtype=torch.int32).cuda(), query_start_loc=_cu(q_lens).cuda(), max_seqlen_q=40,
+        )
+        try:
+            module = torch.nn.Module()
+            module.layer_idx = 0
+            qq = torch.cat(q).transpose(0, 1).unsqueeze(0).cuda()
+            kk = torch.cat(newk).transpose(0, 1).unsqueeze(0).cuda()
+            vv = torch.cat(newv).transpose(0, 1).unsqueeze(0).cuda()
+            out, _ = flash_attention_forward(module, qq, kk, vv, None, scaling=d**-0.5)
+        finally:
+            clear_kv_cache_context()
+        outs.append(out.clone())
+        caches.append((kc.contiguous().clone(), vc.contiguous().clone()))
+    assert_bitwise(outs[1], outs[0], "attention output: head-major cache views vs the reference layout")
+    assert_bitwise(caches[1][0], caches[0][0], "keys written through the strided scatter")
+    assert_bitwise(caches[1][1], caches[0][1], "values written through the strided scatter")
+    assert float(caches[0][0].view(-1, kh, d)[slots[0]].abs().sum()) > 0 and float(caches[1][0].view(-1, kh, d)[slots[2]].abs().sum()) > 0
+
+
 def test_attention_wrapper_gives_the_same_bits_for_any_memory_layout():
     # HuggingFace hands [1, heads, tokens, dim] tensors that are views of [1, tokens, heads, dim] memory; the wrapper
     # reads them through strides. A tensor that really is head-major in memory must give the same bits, in the

@@ -30,6 +30,7 @@ PROTOTYPES = {
     "vx_gemm_nt_mfma": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _P]),
     "vx_transpose_bf16": (_I, [_P, _P, _L, _L, _L, _L, _P]),
     "vx_store_kvcache": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _P]),
+    "vx_store_kvcache_strided": (_I, [_P, _P, _P, _P, _P, _L, _I, _L, _L, _L, _L, _I, _L, _L, _L, _L, _L, _L, _P]),
     "vx_attn_chunk_size": (_I, []),
     "vx_paged_attn_decode_workspace_bytes": (_L, [_L, _L, _L, _L, _L]),
     "vx_paged_attn_decode_workspace_needed": (_L, [_L, _L, _L, _L, _L, _I]),

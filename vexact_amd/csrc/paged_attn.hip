@@ -1082,6 +1082,32 @@ __global__ __launch_bounds__(256) void store_kv_kernel(const uint8_t* __restrict
       *(uint4*)(vc + (int64_t)slot * v_row_bytes + b) = *(const uint4*)(vsrc + t * vs_stride + b);
 }
 
+// The same scatter into a cache that is a [blocks, page, heads, D] view of other memory (head-major
+// [blocks, heads, page, D], which decode attention streams faster): byte strides per block, in-page row and head.
+// One wavefront per token; a lane moves 16 bytes of one head's row.
+__global__ __launch_bounds__(256) void store_kv_strided_kernel(const uint8_t* __restrict__ ksrc,
+                                                               const uint8_t* __restrict__ vsrc, uint8_t* __restrict__ kc,
+                                                               uint8_t* __restrict__ vc, const int* __restrict__ slots,
+                                                               int64_t ntok, int64_t ks_stride, int64_t vs_stride, int heads,
+                                                               int k_head_bytes, int v_head_bytes, int page, int64_t kcb,
+                                                               int64_t kcp, int64_t kch, int64_t vcb, int64_t vcp, int64_t vch) {
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= ntok) return;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t blk = slot / page, row = slot % page;
+  for (int b = lane * 16; b < heads * k_head_bytes; b += 64 * 16) {
+    const int h = b / k_head_bytes, r = b - h * k_head_bytes;
+    *(uint4*)(kc + blk * kcb + row * kcp + h * kch + r) = *(const uint4*)(ksrc + t * ks_stride + b);
+  }
+  if (vsrc)
+    for (int b = lane * 16; b < heads * v_head_bytes; b += 64 * 16) {
+      const int h = b / v_head_bytes, r = b - h * v_head_bytes;
+      *(uint4*)(vc + blk * vcb + row * vcp + h * vch + r) = *(const uint4*)(vsrc + t * vs_stride + b);
+    }
+}
+
 // Which decode form a launch takes: chunks folded inside one workgroup per (sequence, kv head) when that
 // fills the machine (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3); only the
 // latter uses the workspace. A function of the shapes alone. Returns 1 = fused, 0 = split, < 0 = error.
@@ -1363,6 +1389,29 @@ int vx_store_kvcache(const void* key, const void* value, void* k_cache, void* v_
   store_kv_kernel<<<(unsigned)blocks, 256, 0, stream>>>(
       (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping,
       num_tokens, k_src_stride_bytes, v_src_stride_bytes, (int)k_row_bytes, (int)v_row_bytes);
+  return launch_status();
+}
+
+int vx_store_kvcache_strided(const void* key, const void* value, void* k_cache, void* v_cache, const int* slot_mapping,
+                             int64_t num_tokens, int heads, int64_t k_src_stride_bytes, int64_t v_src_stride_bytes,
+                             int64_t k_head_bytes, int64_t v_head_bytes, int page_size, int64_t k_block_stride_bytes,
+                             int64_t k_row_stride_bytes, int64_t k_head_stride_bytes, int64_t v_block_stride_bytes,
+                             int64_t v_row_stride_bytes, int64_t v_head_stride_bytes, hipStream_t stream) {
+  if (!key || !k_cache || !slot_mapping || num_tokens < 0 || heads <= 0 || page_size <= 0) return VX_ERR_ARG;
+  if (value && !v_cache) return VX_ERR_ARG;
+  if (num_tokens == 0) return VX_OK;
+  if (k_head_bytes <= 0 || k_head_bytes % 16 != 0 || heads * k_head_bytes > 0x7fffffff) return VX_ERR_UNSUPPORTED;
+  if ((k_src_stride_bytes | k_block_stride_bytes | k_row_stride_bytes | k_head_stride_bytes) % 16 != 0) return VX_ERR_UNSUPPORTED;
+  if (value && (v_head_bytes <= 0 || v_head_bytes % 16 != 0 || heads * v_head_bytes > 0x7fffffff ||
+                (v_src_stride_bytes | v_block_stride_bytes | v_row_stride_bytes | v_head_stride_bytes) % 16 != 0))
+    return VX_ERR_UNSUPPORTED;
+  if (((uintptr_t)key | (uintptr_t)k_cache | (uintptr_t)value | (uintptr_t)v_cache) % 16 != 0) return VX_ERR_UNSUPPORTED;
+  const int64_t blocks = (num_tokens + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+  store_kv_strided_kernel<<<(unsigned)blocks, 256, 0, stream>>>(
+      (const uint8_t*)key, (const uint8_t*)value, (uint8_t*)k_cache, (uint8_t*)v_cache, slot_mapping, num_tokens,
+      k_src_stride_bytes, v_src_stride_bytes, heads, (int)k_head_bytes, (int)v_head_bytes, page_size, k_block_stride_bytes,
+      k_row_stride_bytes, k_head_stride_bytes, v_block_stride_bytes, v_row_stride_bytes, v_head_stride_bytes);
   return launch_status();
 }
 

@@ -405,15 +405,31 @@ def bmm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 def store_kvcache(key, value, k_cache, v_cache, slot_mapping) -> None:
     assert slot_mapping.numel() == key.shape[0]
+    strided = False
     for name, t, cache in (("key", key, k_cache), ("value", value, v_cache)):
         N, H, D = t.shape
         assert t.stride(-1) == 1
         assert t.stride(1) == D
-        assert cache.stride(1) == H * D, f"Cache stride mismatch: expected stride(1)={H * D}, got {cache.stride(1)}"
         assert cache.dtype == t.dtype, f"{name} and its cache must share a dtype"
+        if cache.dim() == 4 and cache.shape[2:] == (H, D) and cache.stride(3) == 1 and cache.stride(1) != H * D:
+            strided = True  # a [blocks, page, heads, D] view of other memory (KVCacheStore(head_major=True))
+        else:
+            assert cache.stride(1) == H * D, f"Cache stride mismatch: expected stride(1)={H * D}, got {cache.stride(1)}"
     if slot_mapping.dtype != torch.int32:
         raise ValueError(f"slot_mapping must have dtype torch.int32, got {slot_mapping.dtype}")
     es = key.element_size()
+    if strided:
+        assert k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == v_cache.shape[1]
+        _lib.check(
+            _lib.load().vx_store_kvcache_strided(
+                key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
+                key.shape[0], key.shape[1], key.stride(0) * es, value.stride(0) * es, key.shape[2] * es, value.shape[2] * es,
+                k_cache.shape[1], k_cache.stride(0) * es, k_cache.stride(1) * es, k_cache.stride(2) * es,
+                v_cache.stride(0) * es, v_cache.stride(1) * es, v_cache.stride(2) * es, _stream(),
+            ),
+            "vx_store_kvcache_strided",
+        )
+        return
     _lib.check(
         _lib.load().vx_store_kvcache(
             key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
