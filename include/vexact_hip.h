@@ -270,18 +270,23 @@ int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2
 /* Grouped products of the fused-MoE backward (FusedMoeExpertFunction.backward, fused_moe.py:126-265), bf16
  * with fp32 accumulation, over the same tile table / expert offsets as the forward.
  *   vx_moe_gemm_nn: C[rows of expert e] = A[a_src[rows]] W_e (+ A2[rows] W2_e): the data gradient through a
- *     weight stored [K, N] (N contiguous; group stride w_gstride). a_src, a2 / w2 optional. bm <= 128.
+ *     weight stored [K, N] (N contiguous; group stride w_gstride). a_src, a2 / w2 optional. bm <= 128, or
+ *     bm == 256 (tiles of the forward's wide kernel; same bits): then K and K2 must be multiples of 64 and
+ *     a_rows = rows addressable in a (a_src values, or the sorted rows, lie below it; it bounds the kernel's
+ *     32-bit offsets; ignored for bm <= 128).
  *   vx_moe_gemm_tn: dW_e[N, K] = sum over sorted rows cu[e] <= r < cu[e+1] of dY[dy_src[r], :]^T X[x_src[r], :]:
- *     the weight gradient (zeros for an expert without rows). The row gathers are optional.
+ *     the weight gradient (zeros for an expert without rows). The row gathers are optional. dy_rows / x_rows =
+ *     rows addressable in dy / x (at least 1 each; they decide whether the 256 x 256-tile kernel's 32-bit
+ *     offsets reach every row; 0 = unknown, the 128 x 128-tile kernel runs; same bits either way).
  * N, K and row strides must be multiples of 8 elements. Each output element is one ascending MFMA chain
  * (no atomics, no split contraction): results are deterministic and independent of the other experts. */
 int vx_moe_gemm_nn(const void* a, int64_t lda, const int* a_src, const void* w, int64_t ldw, int64_t w_gstride,
                    int64_t K, const void* a2, int64_t lda2, const void* w2, int64_t ldw2, int64_t w2_gstride,
                    int64_t K2, void* c, int64_t ldc, int64_t N, const int* tile_group, const int* tile_row0,
-                   const int* tile_rows, int64_t max_tiles, int bm, hipStream_t stream);
+                   const int* tile_rows, int64_t max_tiles, int bm, int64_t a_rows, hipStream_t stream);
 int vx_moe_gemm_tn(const void* dy, int64_t lddy, const int* dy_src, const void* x, int64_t ldx, const int* x_src,
                    void* dw, int64_t lddw, int64_t dw_gstride, int64_t N, int64_t K, const int* cu,
-                   int64_t num_experts, hipStream_t stream);
+                   int64_t num_experts, int64_t dy_rows, int64_t x_rows, hipStream_t stream);
 
 /* Replace expert_histogram / moe_scatter / moe_gather, group_gemm/kernel/moe.py:52-81, 304-335, 131-161.
  * vx_moe_gather: y[t] = round(sum_i x[index[t, i]]) in slot order (fp32); with residual:

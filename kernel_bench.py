@@ -201,12 +201,12 @@ def run(a, quiet: bool = False) -> list:
         report("packed attention fwd + lse 8 x 1024", timeit(lambda li: ops.packed_attention(q, kk, vv, cu, cu, D**-0.5, True, Lp, return_lse=True), n_layers=2), flops=fl)
         o, lse = ops.packed_attention(q, kk, vv, cu, cu, D**-0.5, True, Lp, return_lse=True)
         report("packed attention bwd 8 x 1024", timeit(lambda li: ops.packed_attention_backward(q, kk, vv, o, do, lse, cu, cu, D**-0.5, Lp, Lp), n_layers=2), flops=fl * 5 // 2)
-        # fused-MoE backward products at the model's expert shapes, 8192 tokens (128-row expert tiles)
+        # fused-MoE backward products at the model's expert shapes, 8192 tokens (256-row expert tiles)
         T = 8192
         x = rnd(T, H, std=1.0)
         logits = torch.randn(T, E, generator=g, device=dev)
         w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
-        r = ops.moe_route(idx, E, bm=128)
+        r = ops.moe_route(idx, E, bm=256)
         gu, dn = rnd(E, 2 * I, H), rnd(E, H, I)
         dyt, dg, du = rnd(T, H, std=1.0), rnd(T * k, I, std=1.0), rnd(T * k, I, std=1.0)
         o_i = torch.empty(T * k, I, dtype=torch.bfloat16, device=dev)

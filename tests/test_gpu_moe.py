@@ -337,6 +337,65 @@ def test_grouped_backward_products_match_per_expert_matmuls(T, k, E, N, K, bm):
     assert_bitwise(ops.moe_gemm_tn(dy.cuda(), x.cuda(), r.cu, E, x_src=r.sorted_token), got, "second launch")
 
 
+@pytest.mark.parametrize("T,k,E,N,K,K2", [(37, 2, 6, 264, 256, 0), (700, 4, 6, 520, 320, 64), (300, 8, 16, 256, 64, 128),
+                                          (2000, 2, 5, 768, 256, 256)])
+def test_wide_backward_products_give_the_bits_of_the_narrow_ones(T, k, E, N, K, K2):
+    # 256-row expert tiles (data gradient) and 256 x 256 output tiles (weight gradient) on the wide kernels'
+    # pipeline against the 128-row kernels: ragged experts, experts without rows, ragged N, both gathers, two
+    # accumulated products with different leading dimensions
+    gen = torch.Generator().manual_seed(T + N + K)
+    sel = torch.randint(0, E - 1, (T, k), generator=gen).cuda()
+    r1, r2 = ops.moe_route(sel, E, bm=128), ops.moe_route(sel, E, bm=256)
+    n = T * k
+    a = torch.randn(T, K, generator=gen).to(torch.bfloat16).cuda()
+    w = (torch.randn(E, K, N, generator=gen) * 0.1).to(torch.bfloat16).cuda()
+    print(f"[case] nn wide T={T} k={k} E={E} N={N} K={K} K2={K2}", flush=True)
+    assert_bitwise(ops.moe_gemm_nn(a, w, r2, a_src=r2.sorted_token), ops.moe_gemm_nn(a, w, r1, a_src=r1.sorted_token),
+                   "A W on 256-row tiles")
+    if K2:
+        aa = torch.randn(n, K, generator=gen).to(torch.bfloat16).cuda()
+        a2 = torch.randn(n, K2, generator=gen).to(torch.bfloat16).cuda()
+        w2 = (torch.randn(E, K2, N, generator=gen) * 0.1).to(torch.bfloat16).cuda()
+        assert_bitwise(ops.moe_gemm_nn(aa, w, r2, a2=a2, w2=w2), ops.moe_gemm_nn(aa, w, r1, a2=a2, w2=w2),
+                       "A W + A2 W2 on 256-row tiles")
+        assert_bitwise(ops.moe_gemm_nn(a, w, r2, a_src=r2.sorted_token, a2=a2, w2=w2),
+                       ops.moe_gemm_nn(a, w, r1, a_src=r1.sorted_token, a2=a2, w2=w2), "gathered A W + A2 W2")
+    if K >= 256:
+        print(f"[case] tn wide T={T} k={k} E={E} N={N} K={K}", flush=True)
+        dy = torch.randn(n, N, generator=gen).to(torch.bfloat16).cuda()
+        dyt = torch.randn(T, N, generator=gen).to(torch.bfloat16).cuda()
+        xs = torch.randn(n, K, generator=gen).to(torch.bfloat16).cuda()
+        wide = ops.moe_gemm_tn(dy, a, r1.cu, E, x_src=r1.sorted_token)
+        assert_bitwise(wide, ops.moe_gemm_tn(dy, a, r1.cu, E, x_src=r1.sorted_token, wide=False), "dY^T X[tok]")
+        assert_bitwise(ops.moe_gemm_tn(dyt, xs, r1.cu, E, dy_src=r1.sorted_token),
+                       ops.moe_gemm_tn(dyt, xs, r1.cu, E, dy_src=r1.sorted_token, wide=False), "dY[tok]^T X")
+        assert float(wide[E - 1].abs().max()) == 0.0, "an expert without rows gets zeros"
+
+
+def test_backward_on_256_row_tiles_gives_the_gradient_bits_of_128_row_tiles(monkeypatch):
+    # FusedMoeExpertFunction.backward picks the tile height from the token count; every height gives the same bits
+    from vexact_amd.batch_invariant_ops.fused_moe import fused_moe_forward
+    T, H, I, E, k = 2304, 256, 320, 8, 2
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    gw, uw = ((torch.randn(E, I, H, generator=g) * 0.08).to(torch.bfloat16) for _ in range(2))
+    dw = (torch.randn(E, H, I, generator=g) * 0.08).to(torch.bfloat16)
+    w, sel = torch.topk(torch.softmax(torch.randn(T, E, generator=g), -1), k)
+    w = (w / w.sum(-1, keepdim=True)).to(torch.bfloat16)
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).cuda()
+
+    def grads():
+        leaves = [t.cuda().requires_grad_() for t in (w, x, gw, uw, dw)]
+        fused_moe_forward(E, leaves[0], sel.cuda(), *leaves[1:]).backward(dy)
+        return [t.grad for t in leaves]
+
+    assert ops.moe_tile_rows(T) == 256
+    wide = grads()
+    monkeypatch.setattr(ops, "moe_tile_rows", lambda *a, **kw: 128)
+    for name, a, b in zip(("routing weights", "hidden states", "gate", "up", "down"), wide, grads()):
+        assert_bitwise(a, b, f"grad of {name}")
+
+
 def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
     # Qwen3MoeSparseMoeBlock after apply_qwen3_moe_patches: router + fused experts on the GPU against the CPU
     # restatements; a token alone gives the bits it gives in the batch; one expert called directly == dense MLP

@@ -56,7 +56,9 @@ class FusedMoeExpertFunction(torch.autograd.Function):
         x = hidden_states.reshape(-1, H)
         T, k = x.shape[0], selected_experts.reshape(x.shape[0], -1).shape[1]
         dy = grad_output.reshape(-1, H).to(torch.bfloat16)
-        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=False))
+        # 256-row expert tiles (the wide kernels) when every contraction depth is a multiple of 64
+        wide_ok = H % 64 == 0 and gate_w.shape[1] % 64 == 0 and up_w.shape[1] % 64 == 0
+        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok))
         flat = r.sorted_flat.long()                      # (token, slot) flat index of each sorted row
         # recomputed with the forward's kernels, so these are the values the forward used
         g = ops.moe_gemm(x, gate_w, r, row_src=r.sorted_token)

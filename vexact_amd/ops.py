@@ -756,7 +756,8 @@ def moe_gemm_nn(
     a2: Optional[torch.Tensor] = None, w2: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Grouped data gradient: ``C[rows of e] = A[a_src[rows]] @ w[e] (+ A2[rows] @ w2[e])`` with ``w [E, K, N]``
-    (N contiguous). ``routing`` must have been built with at most 128 rows per tile."""
+    (N contiguous). ``routing`` has at most 128 rows per tile, or 256 (the wide kernel: K and w2's K multiples
+    of 64); the bits do not depend on the tile height."""
     E, K, N = w.shape
     n_rows = routing.T * routing.k
     assert a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.stride(1) == 1 and w.stride(2) == 1
@@ -776,7 +777,7 @@ def moe_gemm_nn(
             _ptr(a2), a2.stride(0) if a2 is not None else 0, _ptr(w2), w2.stride(1) if w2 is not None else 0,
             w2.stride(0) if w2 is not None else 0, K2, c.data_ptr(), c.stride(0), N,
             routing.tile_group.data_ptr(), routing.tile_row0.data_ptr(), routing.tile_rows.data_ptr(),
-            routing.max_tiles, routing.bm, _stream(),
+            routing.max_tiles, routing.bm, a.shape[0], _stream(),
         ),
         "vx_moe_gemm_nn",
     )
@@ -785,10 +786,11 @@ def moe_gemm_nn(
 
 def moe_gemm_tn(
     dy: torch.Tensor, x: torch.Tensor, cu: torch.Tensor, num_experts: int, *, dy_src: Optional[torch.Tensor] = None,
-    x_src: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+    x_src: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None, wide: bool = True,
 ) -> torch.Tensor:
     """Grouped weight gradient: ``dW[e] = dY[dy_src[r]]^T @ X[x_src[r]]`` summed over the sorted rows
-    ``cu[e] <= r < cu[e + 1]``; returns ``[E, N, K]`` (zeros for an expert without rows)."""
+    ``cu[e] <= r < cu[e + 1]``; returns ``[E, N, K]`` (zeros for an expert without rows). ``wide=False`` keeps
+    the 128 x 128-tile kernel where the 256 x 256-tile one would run (same bits)."""
     N, K = dy.shape[1], x.shape[1]
     assert dy.dtype == torch.bfloat16 and x.dtype == torch.bfloat16 and dy.stride(1) == 1 and x.stride(1) == 1
     assert cu.dtype == torch.int32 and cu.is_contiguous() and cu.numel() == num_experts + 1
@@ -796,10 +798,13 @@ def moe_gemm_tn(
         assert src is None or (src.dtype == torch.int32 and src.is_contiguous())
     dw = out if out is not None else _empty((num_experts, N, K), dtype=torch.bfloat16, device=dy.device)
     assert dw.shape == (num_experts, N, K) and dw.stride(2) == 1
+    if dy.shape[0] == 0 or x.shape[0] == 0:  # no rows at all: every expert's gradient is zero
+        return dw.zero_()
     _lib.check(
         _lib.load().vx_moe_gemm_tn(
             dy.data_ptr(), dy.stride(0), _ptr(dy_src), x.data_ptr(), x.stride(0), _ptr(x_src), dw.data_ptr(),
-            dw.stride(1), dw.stride(0), N, K, cu.data_ptr(), num_experts, _stream(),
+            dw.stride(1), dw.stride(0), N, K, cu.data_ptr(), num_experts, dy.shape[0] if wide else 0, x.shape[0] if wide else 0,
+            _stream(),
         ),
         "vx_moe_gemm_tn",
     )
