@@ -317,7 +317,8 @@ int vx_moe_gather_norm_prefetch(const void* x, const int* index, const void* res
  * [max_pos, D], q -> q_out [T, Hq, D], k -> k_out (optional) and k_cache slot, v -> v_cache slot.
  * Both caches are [blocks, page_size, Hkv, D] views with the given element strides (block, in-page
  * row, head; D contiguous), so a head-major physical layout [blocks, Hkv, page_size, D] can be used.
- * qkv rows are [q heads | k heads | v heads]. The scatter is store_kvcache
+ * qkv rows are [q heads | k heads | v heads]. positions may be null: row t of the tables is then token t's
+ * (per-token cos / sin rows as HuggingFace's rotary module returns them). The scatter is store_kvcache
  * (kv_cache_context.py:294-314); norm + rotary are the HuggingFace Qwen3 attention prologue the
  * reference runs between its q/k/v projections and its attention call. */
 int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, const void* k_norm_w,

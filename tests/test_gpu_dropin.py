@@ -353,3 +353,97 @@ def test_fused_rope_patch_gives_the_bits_of_apply_rotary_pos_emb():
         remove_qwen3_moe_patches()
     assert hf.apply_rotary_pos_emb is original
 
+
+
+def test_fused_attention_and_residual_patches_give_the_bits_of_the_unfused_forwards():
+    # Qwen3MoeAttention.forward over the paged cache as one q/k/v projection + one norm/rotary/store kernel + attention,
+    # and Qwen3MoeDecoderLayer.forward with its residual additions inside the norm and the MoE combine, against
+    # HuggingFace's own forwards (three projections, q / k norm, apply_rotary_pos_emb, the registered attention
+    # function's cache write, two additions): logits and both layers' caches, for a packed prefill of three prompts
+    # and a decode step
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+    from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
+
+    from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
+    from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
+    from vexact_amd.decoder import build_step_metadata
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+    from vexact_amd.models.qwen3_moe.modeling_qwen3_moe import fused_attention_forward, fused_decoder_layer_forward
+
+    page, max_blocks_per_req = 16, 16
+    cache_cfg = types.SimpleNamespace(page_size=page, max_cache_blocks=40)
+    had = ALL_ATTENTION_FUNCTIONS._global_mapping.get("triton-invariant") if hasattr(ALL_ATTENTION_FUNCTIONS, "_global_mapping") else None
+    ALL_ATTENTION_FUNCTIONS["triton-invariant"] = flash_attention_forward
+    original, original_layer = hf.Qwen3MoeAttention.forward, hf.Qwen3MoeDecoderLayer.forward
+    apply_qwen3_moe_patches()
+    try:
+        assert hf.Qwen3MoeAttention.forward is fused_attention_forward
+        assert hf.Qwen3MoeDecoderLayer.forward is fused_decoder_layer_forward
+        hf_cfg, model = _build_model(seed=23)
+        model = model.cuda()
+        rng = np.random.default_rng(24)
+        lens = [37, 5, 120]
+        prompts = [rng.integers(0, hf_cfg.vocab_size, size=n) for n in lens]
+        blocks, nxt = [], 0
+        for n in lens:
+            need = -(-(n + 1) // page)
+            blocks.append(list(range(nxt, nxt + need)))
+            nxt += need
+
+        def run(fused, which_store):
+            hf.Qwen3MoeAttention.forward = fused_attention_forward if fused else original
+            hf.Qwen3MoeDecoderLayer.forward = fused_decoder_layer_forward if fused else original_layer
+            outs = []
+            for new_tokens, ids in (([(n, n) for n in lens], np.concatenate(prompts)), ([(n + 1, 1) for n in lens], np.array([3, 1, 4]))):
+                reqs = [dict(num_computed_tokens=done, tokens_this_step=new, block_ids=blocks[s]) for s, (done, new) in enumerate(new_tokens)]
+                meta = build_step_metadata(reqs, page, max_blocks_per_req)
+                dev = {k: torch.as_tensor(v).cuda() for k, v in meta.items() if k != "max_seqlen_q"}
+                set_kv_cache_context(is_paged_attn=True, key_cache=which_store.key_cache, value_cache=which_store.value_cache,
+                                     block_tables=dev["block_tables"], context_lens=dev["context_lens"],
+                                     slot_mapping=dev["slot_mapping"], query_start_loc=dev["query_start_loc"],
+                                     max_seqlen_q=int(meta["max_seqlen_q"]))
+                try:
+                    with torch.inference_mode(), set_batch_invariant_mode(True):
+                        out = model.model(input_ids=torch.as_tensor(ids)[None].cuda(), position_ids=dev["positions"][None],
+                                          use_cache=False, return_dict=True)
+                        outs.append(model.lm_head(out.last_hidden_state)[0].clone())
+                finally:
+                    clear_kv_cache_context()
+            return outs
+
+        stores = [KVCacheStore(hf_cfg, cache_cfg, torch.device("cuda")) for _ in range(2)]
+        for s in stores:
+            for t in list(s.key_cache.values()) + list(s.value_cache.values()):
+                t.zero_()
+        unfused = run(False, stores[0])
+        fused = run(True, stores[1])
+        attn = model.model.layers[0].self_attn
+        assert attn.q_proj.weight.data_ptr() == attn._vx_qkv_weight.data_ptr(), "the parameters are views of the fused weight"
+        for name, a, b in zip(("prefill", "decode"), fused, unfused):
+            assert_bitwise(a, b, f"{name} logits, fused attention forward vs HuggingFace's")
+        for layer in range(2):
+            assert_bitwise(stores[1].key_cache[layer], stores[0].key_cache[layer], f"key cache of layer {layer}")
+            assert_bitwise(stores[1].value_cache[layer], stores[0].value_cache[layer], f"value cache of layer {layer}")
+        # a parameter written in place (what a weight synchronisation does) reaches the fused weight; one that gets
+        # new storage makes the module rebuild it
+        with torch.no_grad():
+            attn.k_proj.weight.data.mul_(0.5)
+        again_fused, again_unfused = run(True, stores[1]), run(False, stores[0])
+        assert_bitwise(again_fused[1], again_unfused[1], "after an in-place weight update")
+        assert not torch.equal(again_fused[1], fused[1])
+        attn.v_proj.weight.data = attn.v_proj.weight.data.clone() * 2
+        again_fused, again_unfused = run(True, stores[1]), run(False, stores[0])
+        assert_bitwise(again_fused[1], again_unfused[1], "after a parameter got new storage")
+        assert attn.v_proj.weight.data_ptr() == attn._vx_qkv_weight[attn.q_proj.weight.shape[0] + attn.k_proj.weight.shape[0]].data_ptr()
+    finally:
+        hf.Qwen3MoeAttention.forward = fused_attention_forward  # what remove_qwen3_moe_patches expects to undo
+        hf.Qwen3MoeDecoderLayer.forward = fused_decoder_layer_forward
+        remove_qwen3_moe_patches()
+        if had is None:
+            try:
+                del ALL_ATTENTION_FUNCTIONS._global_mapping["triton-invariant"]
+            except Exception:
+                pass
+        else:
+            ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had
+    assert hf.Qwen3MoeAttention.forward is original and hf.Qwen3MoeDecoderLayer.forward is original_layer

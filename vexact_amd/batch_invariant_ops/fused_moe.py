@@ -94,12 +94,15 @@ def fused_moe_forward(
     fc2_weight: torch.Tensor,
     fc1_1_2_weight: Optional[torch.Tensor] = None,
     packed_weights: Optional[tuple] = None,
+    residual: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """``hidden_states [T,H]``, ``routing_weights/selected_experts [T,k]``; expert weights either as
     ``fc1_1_weight`` (gate) + ``fc1_2_weight`` (up), each ``[E,I,H]``, or fused ``fc1_1_2_weight [E,2I,H]``
     (gate rows first); ``fc2_weight [E,H,I]``. Returns ``[T,H]`` bf16. ``packed_weights`` (not in the
     reference; inference only): fragment-order copies of the same weights, ``(ops.pack_expert_weights(
-    fc1_1_2_weight), ops.pack_expert_weights(fc2_weight))``, streamed instead at decode sizes."""
+    fc1_1_2_weight), ops.pack_expert_weights(fc2_weight))``, streamed instead at decode sizes. ``residual`` (not
+    in the reference; bf16, the shape of ``hidden_states``): returns ``residual + output`` with the rounding of a
+    separate bf16 add, inside the combine kernel."""
     routing_weights = routing_weights.bfloat16()
     hidden_states = hidden_states.bfloat16()
     gate_w, up_w = _split_weights(fc1_1_weight, fc1_2_weight, fc1_1_2_weight)
@@ -110,12 +113,18 @@ def fused_moe_forward(
         down_w = down_w.contiguous()
     shape = hidden_states.shape
     if torch.is_grad_enabled() and any(t.requires_grad for t in (routing_weights, hidden_states, gate_w, up_w, down_w)):
-        return FusedMoeExpertFunction.apply(num_experts, routing_weights, selected_experts, hidden_states, gate_w, up_w,
-                                            down_w)
+        out = FusedMoeExpertFunction.apply(num_experts, routing_weights, selected_experts, hidden_states, gate_w, up_w,
+                                           down_w)
+        return out if residual is None else residual + out
     x = hidden_states.reshape(-1, shape[-1])
+    res = None
+    if residual is not None:
+        res = residual.reshape(-1, shape[-1])
+        if res.dtype != torch.bfloat16 or res.stride(1) != 1 or res.shape != x.shape:
+            raise ValueError("residual must be a bf16 tensor of the shape of hidden_states, contiguous in its last dim")
     out = ops.fused_moe(
         x, routing_weights.reshape(x.shape[0], -1), selected_experts.reshape(x.shape[0], -1), gate_w, up_w, down_w,
-        num_experts, packed=packed_weights,
+        num_experts, packed=packed_weights, residual=res,
     )
     return out.reshape(shape)
 

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   // position, norm weight and rotary rows are requested before the reduction so that their
   // latency overlaps it
   const bf16_t* w = (h < Hq) ? qw : kw;
-  int64_t pos = (int64_t)positions[t];
+  int64_t pos = positions ? (int64_t)positions[t] : t;  // no positions: row t of the tables belongs to token t
   pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
   uint2 wr = make_uint2(0, 0), cr = make_uint2(0, 0), sr = make_uint2(0, 0);
   if (own) {
@@ -167,7 +167,7 @@ int vx_qk_norm_rope_store(const void* qkv, int64_t ld, const void* q_norm_w, con
                           void* k_cache, void* v_cache, int64_t T, int Hq, int Hkv, int D, float eps,
                           int64_t max_pos, int page_size, int64_t cache_block_stride,
                           int64_t cache_row_stride, int64_t cache_head_stride, hipStream_t stream) {
-  if (!qkv || !q_norm_w || !k_norm_w || !cos_table || !sin_table || !positions || !q_out) return VX_ERR_ARG;
+  if (!qkv || !q_norm_w || !k_norm_w || !cos_table || !sin_table || !q_out) return VX_ERR_ARG;
   if (T < 0 || Hq <= 0 || Hkv <= 0 || max_pos <= 0) return VX_ERR_ARG;
   if (D != 128 && D != 64) return VX_ERR_UNSUPPORTED;
   if (ld % 4 != 0) return VX_ERR_UNSUPPORTED;

@@ -68,8 +68,10 @@ class Qwen3MoeExperts(nn.Module):
         return super()._apply(fn, *args, **kwargs)
 
     def forward(self, hidden_states: torch.Tensor, expert_idx: Optional[int] = None,
-                routing_weights: Optional[torch.Tensor] = None, selected_experts: Optional[torch.Tensor] = None):
+                routing_weights: Optional[torch.Tensor] = None, selected_experts: Optional[torch.Tensor] = None,
+                residual: Optional[torch.Tensor] = None):
         if expert_idx is not None:  # one expert as a dense SwiGLU MLP
+            assert residual is None
             inter = self.intermediate_size
             w = self.gate_up_proj[expert_idx]
             x = hidden_states.reshape(-1, self.hidden_dim)
@@ -86,7 +88,7 @@ class Qwen3MoeExperts(nn.Module):
         return fused_moe_forward(
             num_experts=self.num_experts, routing_weights=routing_weights, selected_experts=selected_experts,
             hidden_states=hidden_states, fc1_1_weight=None, fc1_2_weight=None, fc2_weight=self.down_proj,
-            fc1_1_2_weight=self.gate_up_proj, packed_weights=packed,
+            fc1_1_2_weight=self.gate_up_proj, packed_weights=packed, residual=residual,
         )
 
 
@@ -104,8 +106,9 @@ def moe_block_init(self, config):
     self.experts = Qwen3MoeExperts(config)
 
 
-def moe_block_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
-    """Replacement for ``Qwen3MoeSparseMoeBlock.forward``; returns the hidden states only."""
+def moe_block_forward(self, hidden_states: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Replacement for ``Qwen3MoeSparseMoeBlock.forward``; returns the hidden states only. ``residual`` (not in
+    the reference): the block returns ``residual + output``, added inside the combine kernel."""
     if not isinstance(self.experts, Qwen3MoeExperts):
         raise AssertionError(
             "Qwen3-MoE experts are not fused. Ensure apply_qwen3_moe_patches() is called before loading the model."
@@ -115,7 +118,8 @@ def moe_block_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
     router_logits = self.gate(x)  # aten::mm -> the batch-invariant GEMM when the mode is on
     routing_weights, selected_experts = ops.router_topk(
         router_logits, self.top_k, renorm=bool(self.norm_topk_prob), out_dtype=x.dtype, index_dtype=torch.int64)
-    out = self.experts(x, routing_weights=routing_weights, selected_experts=selected_experts)
+    res = None if residual is None else residual.reshape(-1, hidden_dim)
+    out = self.experts(x, routing_weights=routing_weights, selected_experts=selected_experts, residual=res)
     return out.reshape(batch_size, sequence_length, hidden_dim)
 
 
@@ -177,13 +181,125 @@ def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **
     return _ORIGINAL_ROPE(q, k, cos, sin, *args, unsqueeze_dim=unsqueeze_dim, **kwargs)
 
 
-def apply_qwen3_moe_patches(fused_rms_norm: bool = True, fused_rope: bool = True) -> None:
+_ORIGINAL_ATTN = None  # Qwen3MoeAttention.forward while the fused form is patched in
+
+
+def _fused_qkv_weight(attn) -> torch.Tensor:
+    """``[q_proj.weight; k_proj.weight; v_proj.weight]`` as one tensor, made once per module: the three
+    parameters are then re-pointed at row ranges of it, so there is still one copy of the weights in memory and
+    an in-place write to a parameter (``param.data.copy_``, what the reference's weight sync does,
+    vexact/inferencer/model_loader.py:113) lands in the fused tensor. A parameter that has been given new
+    storage since is noticed by its address and the fused tensor is rebuilt."""
+    ws = (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
+    fused = getattr(attn, "_vx_qkv_weight", None)
+    if fused is not None:
+        row = 0
+        for w in ws:
+            if w.data_ptr() != fused[row].data_ptr() or w.dtype != fused.dtype:
+                fused = None
+                break
+            row += w.shape[0]
+    if fused is None:
+        with torch.no_grad():
+            fused = torch.cat([w.detach() for w in ws], dim=0)
+            row = 0
+            for w in ws:
+                w.data = fused[row:row + w.shape[0]]
+                row += w.shape[0]
+        attn._vx_qkv_weight = fused
+    return fused
+
+
+def fused_attention_forward(self, hidden_states, position_embeddings, attention_mask=None, past_key_values=None, **kwargs):
+    """``Qwen3MoeAttention.forward`` for a step over the paged cache as four launches in front of the output
+    projection instead of twelve: one q/k/v projection on the concatenated weight, one kernel for the per-head
+    q / k RMSNorm, the rotary embedding and the cache write (``ops.qk_norm_rope_store``; it computes what
+    ``q_norm`` / ``k_norm``, ``apply_rotary_pos_emb`` and ``store_kvcache`` compute, rounding for rounding), the
+    attention kernel, then ``o_proj``. A row of a product depends on its own weight row only, so the concatenated
+    projection gives the three projections' bits. Taken only under batch-invariant mode with a paged context,
+    the registered attention function of this package, bf16 tensors of batch 1 and no autograd, bias, HuggingFace
+    cache object or sliding window; anything else runs the original forward."""
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+    from ...batch_invariant_ops import flash_attention_forward, flash_attn_varlen_func, is_batch_invariant_mode_enabled
+    from ...batch_invariant_ops.kv_cache_context import get_kv_cache_context
+
+    ctx = get_kv_cache_context()
+    cos, sin = position_embeddings
+    D = self.head_dim
+    fits = (
+        ctx is not None and ctx.is_paged_attn and past_key_values is None and not self.training
+        and is_batch_invariant_mode_enabled() and not torch.is_grad_enabled()
+        and hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 3
+        and hidden_states.shape[0] == 1 and D in (64, 128) and getattr(self, "sliding_window", None) is None
+        and self.q_proj.bias is None and self.k_proj.bias is None and self.v_proj.bias is None
+        and self.q_proj.weight.dtype == torch.bfloat16 and self.q_norm.weight.dtype == torch.bfloat16
+        and cos.dtype == torch.bfloat16 and sin.dtype == torch.bfloat16 and cos.shape == sin.shape
+        and cos.shape == (1, hidden_states.shape[1], D) and cos.is_contiguous() and sin.is_contiguous()
+        and ALL_ATTENTION_FUNCTIONS.get(self.config._attn_implementation) is flash_attention_forward
+    )
+    if not fits:
+        return _ORIGINAL_ATTN(self, hidden_states, position_embeddings, attention_mask, past_key_values, **kwargs)
+    T = hidden_states.shape[1]
+    Hq, Hkv = self.q_proj.weight.shape[0] // D, self.k_proj.weight.shape[0] // D
+    x = hidden_states[0]
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    qkv = ops.gemm_nt(x, _fused_qkv_weight(self))
+    q = ops._empty((T, Hq, D), dtype=torch.bfloat16, device=x.device)
+    ops.qk_norm_rope_store(qkv, self.q_norm.weight, self.k_norm.weight, cos[0], sin[0], None, ctx.slot_mapping, q,
+                           ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx], Hq, Hkv, D,
+                           self.q_norm.variance_epsilon)
+    out, _ = flash_attn_varlen_func(
+        q, ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx], cu_seqlens_q=ctx.query_start_loc,
+        max_seqlen_q=ctx.max_seqlen_q, seqused_k=ctx.context_lens, page_table=ctx.block_tables, dropout_p=0.0,
+        softmax_scale=self.scaling, causal=True)
+    return self.o_proj(out.reshape(1, T, Hq * D)), None
+
+
+_ORIGINAL_LAYER = None  # Qwen3MoeDecoderLayer.forward while the fused form is patched in
+
+
+def fused_decoder_layer_forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_values=None,
+                                use_cache=False, position_embeddings=None, **kwargs):
+    """``Qwen3MoeDecoderLayer.forward`` with its two residual additions folded into the kernels next to them:
+    ``residual + attention output`` into the post-attention RMSNorm's launch (which also writes the sum) and
+    ``residual + MoE output`` into the MoE combine. Each sum is rounded to bf16 exactly where the separate
+    addition rounds it, so the bits do not change. Taken under batch-invariant mode for bf16 GPU tensors without
+    autograd when the layer's MLP is the patched sparse block; otherwise the original forward runs."""
+    from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
+
+    from ...batch_invariant_ops import is_batch_invariant_mode_enabled
+
+    norm = self.post_attention_layernorm
+    if not (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 3
+            and not torch.is_grad_enabled() and is_batch_invariant_mode_enabled()
+            and isinstance(self.mlp, hf.Qwen3MoeSparseMoeBlock) and isinstance(getattr(self.mlp, "experts", None), Qwen3MoeExperts)
+            and hf.Qwen3MoeSparseMoeBlock.forward is moe_block_forward and norm.weight.dtype == torch.bfloat16):
+        return _ORIGINAL_LAYER(self, hidden_states, attention_mask=attention_mask, position_ids=position_ids,
+                               past_key_values=past_key_values, use_cache=use_cache,
+                               position_embeddings=position_embeddings, **kwargs)
+    residual = hidden_states if hidden_states.stride(2) == 1 else hidden_states.contiguous()
+    attn_out, _ = self.self_attn(
+        hidden_states=self.input_layernorm(hidden_states), attention_mask=attention_mask, position_ids=position_ids,
+        past_key_values=past_key_values, use_cache=use_cache, position_embeddings=position_embeddings, **kwargs)
+    summed = ops._empty_like(residual)
+    normed = ops.rms_norm(attn_out, norm.weight, norm.variance_epsilon, hf_two_rounding=True, residual=residual,
+                          sum_out=summed)
+    return self.mlp(normed, residual=summed)
+
+
+def apply_qwen3_moe_patches(fused_rms_norm: bool = True, fused_rope: bool = True, fused_attention: bool = True,
+                            fused_residual: bool = True) -> None:
     """Swap the HuggingFace block's constructor and forward (idempotent). ``fused_rms_norm`` also replaces
     ``Qwen3MoeRMSNorm.forward`` by ``fused_rms_norm_forward`` (same bits under batch-invariant mode, one launch
     instead of eleven; not in the reference, whose optional Liger patch leaves RMSNorm alone because Liger's is
     not batch invariant, vexact/models/register.py:84-87) and ``fused_rope`` the modeling file's
-    ``apply_rotary_pos_emb`` by ``fused_apply_rotary_pos_emb`` (the function that Liger patch swaps, :77-80)."""
-    global _ORIGINAL, _ORIGINAL_NORM, _ORIGINAL_ROPE
+    ``apply_rotary_pos_emb`` by ``fused_apply_rotary_pos_emb`` (the function that Liger patch swaps, :77-80).
+    ``fused_attention`` replaces ``Qwen3MoeAttention.forward`` by ``fused_attention_forward`` (same bits; it
+    applies to steps over the paged cache and falls through to the original otherwise) and ``fused_residual``
+    ``Qwen3MoeDecoderLayer.forward`` by ``fused_decoder_layer_forward`` (same bits, two launches fewer)."""
+    global _ORIGINAL, _ORIGINAL_NORM, _ORIGINAL_ROPE, _ORIGINAL_ATTN, _ORIGINAL_LAYER
     from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
 
     if _ORIGINAL is None:
@@ -196,14 +312,26 @@ def apply_qwen3_moe_patches(fused_rms_norm: bool = True, fused_rope: bool = True
     if fused_rope and _ORIGINAL_ROPE is None:
         _ORIGINAL_ROPE = hf.apply_rotary_pos_emb
         hf.apply_rotary_pos_emb = fused_apply_rotary_pos_emb
+    if fused_attention and _ORIGINAL_ATTN is None:
+        _ORIGINAL_ATTN = hf.Qwen3MoeAttention.forward
+        hf.Qwen3MoeAttention.forward = fused_attention_forward
+    if fused_residual and _ORIGINAL_LAYER is None:
+        _ORIGINAL_LAYER = hf.Qwen3MoeDecoderLayer.forward
+        hf.Qwen3MoeDecoderLayer.forward = fused_decoder_layer_forward
 
 
 def remove_qwen3_moe_patches() -> None:
     """Put the HuggingFace block's own constructor and forward back (blocks built meanwhile keep their fused
     experts and stop working with the original forward; meant for tests and tools that need both forms)."""
-    global _ORIGINAL, _ORIGINAL_NORM, _ORIGINAL_ROPE
+    global _ORIGINAL, _ORIGINAL_NORM, _ORIGINAL_ROPE, _ORIGINAL_ATTN, _ORIGINAL_LAYER
     from transformers.models.qwen3_moe import modeling_qwen3_moe as hf
 
+    if _ORIGINAL_LAYER is not None:
+        hf.Qwen3MoeDecoderLayer.forward = _ORIGINAL_LAYER
+        _ORIGINAL_LAYER = None
+    if _ORIGINAL_ATTN is not None:
+        hf.Qwen3MoeAttention.forward = _ORIGINAL_ATTN
+        _ORIGINAL_ATTN = None
     if _ORIGINAL_ROPE is not None:
         hf.apply_rotary_pos_emb = _ORIGINAL_ROPE
         _ORIGINAL_ROPE = None

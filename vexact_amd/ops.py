@@ -918,10 +918,16 @@ def fused_moe(
 
 def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, cos_table, sin_table, positions, slot_mapping, q_out,
                        k_cache, v_cache, Hq: int, Hkv: int, D: int, eps: float, k_out=None) -> None:
-    """Caches are ``[blocks, page, Hkv, D]`` views (any block / row / head strides, D contiguous)."""
+    """Caches are ``[blocks, page, Hkv, D]`` views (any block / row / head strides, D contiguous).
+    ``positions=None``: ``cos_table`` / ``sin_table`` hold one row per token."""
     T = qkv.shape[0]
     assert qkv.stride(1) == 1 and qkv.shape[1] == (Hq + 2 * Hkv) * D
-    assert positions.dtype in (torch.int32, torch.int64)
+    assert cos_table.is_contiguous() and sin_table.is_contiguous() and cos_table.shape == sin_table.shape
+    assert cos_table.shape[1] == D and cos_table.dtype == torch.bfloat16 and sin_table.dtype == torch.bfloat16
+    if positions is None:
+        assert cos_table.shape[0] >= T
+    else:
+        assert positions.dtype in (torch.int32, torch.int64)
     page, sb, sp, sh = 1, 0, 0, 0
     if k_cache is not None:
         assert k_cache.dim() == 4 and k_cache.shape[2] == Hkv and k_cache.shape[3] == D and k_cache.stride(3) == 1
@@ -931,7 +937,8 @@ def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, cos_table, sin_table, positions,
     _lib.check(
         _lib.load().vx_qk_norm_rope_store(
             qkv.data_ptr(), qkv.stride(0), q_norm_w.data_ptr(), k_norm_w.data_ptr(), cos_table.data_ptr(),
-            sin_table.data_ptr(), positions.data_ptr(), int(positions.dtype == torch.int64), _ptr(slot_mapping),
+            sin_table.data_ptr(), _ptr(positions), int(positions is not None and positions.dtype == torch.int64),
+            _ptr(slot_mapping),
             q_out.data_ptr(), _ptr(k_out), _ptr(k_cache), _ptr(v_cache), T, Hq, Hkv, D, float(eps),
             cos_table.shape[0], page, sb, sp, sh, _stream(),
         ),
