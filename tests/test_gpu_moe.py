@@ -372,6 +372,36 @@ def test_wide_backward_products_give_the_bits_of_the_narrow_ones(T, k, E, N, K, 
         assert float(wide[E - 1].abs().max()) == 0.0, "an expert without rows gets zeros"
 
 
+@pytest.mark.parametrize("n,I,T,k", [(520, 64, 130, 4), (4096, 768, 512, 8), (7, 8, 7, 1)])
+def test_backward_elementwise_kernel_equals_the_tensor_operations(n, I, T, k):
+    # vx_moe_swiglu_bwd against the bf16 tensor operations the reference's backward runs (fused_moe.py:150-250): every
+    # elementwise output bit for bit (same rounding points), the routing-weight gradient within 1 bf16 ulp of torch.sum
+    gen = torch.Generator().manual_seed(n + I)
+    g = (torch.randn(n, I, generator=gen) * 2).to(torch.bfloat16).cuda()
+    u = torch.randn(n, I, generator=gen).to(torch.bfloat16).cuda()
+    d = torch.randn(n, I, generator=gen).to(torch.bfloat16).cuda()
+    rw = torch.rand(T, k, generator=gen).to(torch.bfloat16).cuda()
+    flat = torch.randperm(n, generator=gen).to(torch.int32).cuda()
+    hw, d_g, d_u, d_rw = ops.moe_swiglu_backward(g, u, d, rw, flat)
+    fl = flat.long()
+    a = torch.ops.aten.silu(g)
+    act = a * u
+    ws = rw.reshape(-1)[fl].unsqueeze(1)
+    d_act = d * ws
+    want_rw = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    want_rw[fl] = torch.sum(act * d, dim=-1)
+    assert_bitwise(hw, act * ws, "hw = silu(g) u w")
+    assert_bitwise(d_u, a * d_act, "d_u")
+    assert_bitwise(d_g, torch.ops.aten.silu_backward(d_act * u, g), "d_g")
+    assert d_rw.shape == rw.shape
+    assert_bf16_close(d_rw.reshape(-1), want_rw, max_ulp=1, atol_frac=1e-3, what="routing-weight gradient")
+    # a row's outputs do not depend on the other rows
+    one = ops.moe_swiglu_backward(g[3:4].contiguous(), u[3:4].contiguous(), d[3:4].contiguous(),
+                                  rw.reshape(-1)[fl[3]].reshape(1, 1), torch.zeros(1, dtype=torch.int32, device="cuda"))
+    assert_bitwise(one[1], d_g[3:4], "row alone")
+    assert_bitwise(one[3].reshape(-1), d_rw.reshape(-1)[fl[3]].reshape(1), "row sum alone")
+
+
 def test_backward_on_256_row_tiles_gives_the_gradient_bits_of_128_row_tiles(monkeypatch):
     # FusedMoeExpertFunction.backward picks the tile height from the token count; every height gives the same bits
     from vexact_amd.batch_invariant_ops.fused_moe import fused_moe_forward

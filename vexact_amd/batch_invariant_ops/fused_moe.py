@@ -59,23 +59,27 @@ class FusedMoeExpertFunction(torch.autograd.Function):
         # 256-row expert tiles (the wide kernels) when every contraction depth is a multiple of 64
         wide_ok = H % 64 == 0 and gate_w.shape[1] % 64 == 0 and up_w.shape[1] % 64 == 0
         r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok))
-        flat = r.sorted_flat.long()                      # (token, slot) flat index of each sorted row
         # recomputed with the forward's kernels, so these are the values the forward used
         g = ops.moe_gemm(x, gate_w, r, row_src=r.sorted_token)
         u = ops.moe_gemm(x, up_w, r, row_src=r.sorted_token)
-        a = torch.ops.aten.silu(g)
-        act = a * u
-        w_sorted = routing_weights.reshape(-1)[flat].unsqueeze(1)
-        hw = act * w_sorted
         # grouped products on the HIP kernels; the row gathers x[tok], dy[tok] happen inside them
         d_hw = ops.moe_gemm_nn(dy, down_w, r, a_src=r.sorted_token)                # dgrad of the down projection
+        if g.shape[1] % 8 == 0 and routing_weights.dtype == torch.bfloat16:
+            # silu, its derivative, the routing-weight gradient and the scatter back to (token, slot) in one launch
+            hw, d_g, d_u, grad_rw = ops.moe_swiglu_backward(g, u, d_hw, routing_weights.reshape(T, k), r.sorted_flat)
+        else:
+            flat = r.sorted_flat.long()                  # (token, slot) flat index of each sorted row
+            a = torch.ops.aten.silu(g)
+            act = a * u
+            w_sorted = routing_weights.reshape(-1)[flat].unsqueeze(1)
+            hw = act * w_sorted
+            d_act = d_hw * w_sorted
+            d_w_sorted = torch.sum(act * d_hw, dim=-1)
+            grad_rw = torch.empty_like(d_w_sorted)
+            grad_rw[flat] = d_w_sorted
+            d_a, d_u = d_act * u, a * d_act
+            d_g = torch.ops.aten.silu_backward(d_a, g)
         d_d_w = ops.moe_gemm_tn(dy, hw, r.cu, E, dy_src=r.sorted_token) if ctx.needs_input_grad[6] else None
-        d_act = d_hw * w_sorted
-        d_w_sorted = torch.sum(act * d_hw, dim=-1)
-        grad_rw = torch.empty_like(d_w_sorted)
-        grad_rw[flat] = d_w_sorted
-        d_a, d_u = d_act * u, a * d_act
-        d_g = torch.ops.aten.silu_backward(d_a, g)
         d_xs = ops.moe_gemm_nn(d_g, gate_w, r, a2=d_u, w2=up_w)
         d_g_w = ops.moe_gemm_tn(d_g, x, r.cu, E, x_src=r.sorted_token) if ctx.needs_input_grad[4] else None
         d_u_w = ops.moe_gemm_tn(d_u, x, r.cu, E, x_src=r.sorted_token) if ctx.needs_input_grad[5] else None

@@ -663,6 +663,64 @@ __global__ __launch_bounds__(512) void moe_gemm_tn_wide_kernel(MoeTnParams p) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // loads past the last step still target our LDS
 }
 
+// ---------------------------------------------------------------------------------------
+// The elementwise part of the backward pass between the grouped products (fused_moe.py:150-250 of the
+// reference runs it as separate bf16 tensor operations; every rounding to bf16 below stands where one of those
+// operations rounds). Per sorted row r with routing weight w = rw[flat[r]], from g, u (recomputed gate / up
+// projections) and d_hw (gradient of the weighted activation):
+//   a = silu(g)   act = a u   hw = act w                       (the forward's values)
+//   d_act = d_hw w   d_rw[flat[r]] = sum_i r16(act d_hw)   d_u = a d_act   d_g = silu'(g) (d_act u)
+// One wavefront per row; the row sum runs lane-sequentially over the lane's 8-element pieces, then through the
+// wavefront butterfly: the order depends on I only.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float rb(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+
+__global__ __launch_bounds__(256) void moe_swiglu_bwd_kernel(const bf16_t* __restrict__ g, const bf16_t* __restrict__ u,
+                                                             const bf16_t* __restrict__ d_hw, int64_t ldg, int64_t ldu,
+                                                             int64_t ldd, const bf16_t* __restrict__ rw,
+                                                             const int* __restrict__ flat, bf16_t* __restrict__ hw,
+                                                             bf16_t* __restrict__ d_g, bf16_t* __restrict__ d_u,
+                                                             bf16_t* __restrict__ d_rw, int64_t rows, int I) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int f = flat[r];
+  const float w = bf16_to_f32(rw[f]);
+  float part = 0.f;
+  for (int v = lane; v < I / 8; v += 64) {
+    const uint4 gv = ldg16_raw(g + r * ldg + 8 * v), uv = ldg16_raw(u + r * ldu + 8 * v), dv = ldg16_raw(d_hw + r * ldd + 8 * v);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w}, dw[4] = {dv.x, dv.y, dv.z, dv.w};
+    uint32_t oh[4], og[4], ou[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      float res[3][2];
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const float gf = h ? bf16hi(gw[j]) : bf16lo(gw[j]);
+        const float uf = h ? bf16hi(uw[j]) : bf16lo(uw[j]);
+        const float df = h ? bf16hi(dw[j]) : bf16lo(dw[j]);
+        const float s = 1.0f / (1.0f + expf(-gf));
+        const float a = rb(gf * s);
+        const float act = rb(a * uf);
+        const float d_act = rb(df * w);
+        part += rb(act * df);
+        const float d_a = rb(d_act * uf);
+        res[0][h] = act * w;
+        res[1][h] = d_a * s * (1.0f + gf * (1.0f - s));
+        res[2][h] = a * d_act;
+      }
+      oh[j] = pack_bf16x2(res[0][0], res[0][1]);
+      og[j] = pack_bf16x2(res[1][0], res[1][1]);
+      ou[j] = pack_bf16x2(res[2][0], res[2][1]);
+    }
+    *(uint4*)(hw + r * (int64_t)I + 8 * v) = make_uint4(oh[0], oh[1], oh[2], oh[3]);
+    *(uint4*)(d_g + r * (int64_t)I + 8 * v) = make_uint4(og[0], og[1], og[2], og[3]);
+    *(uint4*)(d_u + r * (int64_t)I + 8 * v) = make_uint4(ou[0], ou[1], ou[2], ou[3]);
+  }
+  part = wave_sum(part);
+  if (lane == 0) d_rw[f] = f32_to_bf16(part);
+}
+
 static inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace vx
@@ -718,6 +776,22 @@ int vx_moe_gemm_nn(const void* a, int64_t lda, const int* a_src, const void* w, 
     return launch_status();
   }
   moe_gemm_nn_kernel<NN_ROWS><<<dim3((unsigned)((N + 127) / 128), (unsigned)max_tiles), 256, 0, stream>>>(p);
+  return launch_status();
+}
+
+int vx_moe_swiglu_bwd(const void* g, const void* u, const void* d_hw, int64_t ldg, int64_t ldu, int64_t ldd,
+                      const void* rw, const int* flat, void* hw, void* d_g, void* d_u, void* d_rw, int64_t rows,
+                      int64_t I, hipStream_t stream) {
+  if (!g || !u || !d_hw || !rw || !flat || !hw || !d_g || !d_u || !d_rw) return VX_ERR_ARG;
+  if (rows < 0 || I <= 0 || I > 0x7fffffff) return VX_ERR_ARG;
+  if (I % 8 || ldg % 8 || ldu % 8 || ldd % 8 || !al16(g) || !al16(u) || !al16(d_hw) || !al16(hw) || !al16(d_g) || !al16(d_u))
+    return VX_ERR_UNSUPPORTED;
+  if (rows == 0) return VX_OK;
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_UNSUPPORTED;
+  moe_swiglu_bwd_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)g, (const bf16_t*)u, (const bf16_t*)d_hw, ldg,
+                                                              ldu, ldd, (const bf16_t*)rw, flat, (bf16_t*)hw, (bf16_t*)d_g,
+                                                              (bf16_t*)d_u, (bf16_t*)d_rw, rows, (int)I);
   return launch_status();
 }
 

@@ -811,6 +811,28 @@ def moe_gemm_tn(
     return dw
 
 
+def moe_swiglu_backward(g: torch.Tensor, u: torch.Tensor, d_hw: torch.Tensor, routing_weights: torch.Tensor,
+                        sorted_flat: torch.Tensor):
+    """The elementwise step of the fused-MoE backward in one launch. ``g``, ``u``, ``d_hw`` are ``[T k, I]`` in
+    sorted-row order, ``routing_weights [T, k]`` bf16, ``sorted_flat`` the (token, slot) flat index of each sorted
+    row. Returns ``(hw, d_g, d_u, d_routing_weights [T, k])``."""
+    n, I = g.shape
+    for t in (g, u, d_hw):
+        assert t.dtype == torch.bfloat16 and t.shape == (n, I) and t.stride(1) == 1
+    rw = routing_weights.contiguous()
+    assert rw.dtype == torch.bfloat16 and rw.numel() == n and sorted_flat.dtype == torch.int32 and sorted_flat.numel() == n
+    hw, d_g, d_u = (_empty((n, I), dtype=torch.bfloat16, device=g.device) for _ in range(3))
+    d_rw = _empty(rw.shape, dtype=torch.bfloat16, device=g.device)
+    _lib.check(
+        _lib.load().vx_moe_swiglu_bwd(
+            g.data_ptr(), u.data_ptr(), d_hw.data_ptr(), g.stride(0), u.stride(0), d_hw.stride(0), rw.data_ptr(),
+            sorted_flat.data_ptr(), hw.data_ptr(), d_g.data_ptr(), d_u.data_ptr(), d_rw.data_ptr(), n, I, _stream(),
+        ),
+        "vx_moe_swiglu_bwd",
+    )
+    return hw, d_g, d_u, d_rw
+
+
 def expert_histogram(idx: torch.Tensor, num_bins: int) -> torch.Tensor:
     assert idx.is_cuda
     assert idx.dtype == torch.int32 or idx.dtype == torch.int64
