@@ -287,11 +287,12 @@ int vx_moe_gemm_nn(const void* a, int64_t lda, const int* a_src, const void* w, 
 /* The elementwise step of the same backward between the products (fused_moe.py:150-250: silu, its derivative, the
  * routing-weight gradient), one launch, bf16 with a rounding wherever one of the reference's tensor operations
  * rounds. For sorted row r, w = rw[flat[r]]: hw = silu(g) u w; d_rw[flat[r]] = sum_i (silu(g) u)(d_hw);
- * d_u = silu(g) (d_hw w); d_g = silu'(g) ((d_hw w) u). g, u, d_hw: [rows, I] with row strides; hw, d_g, d_u:
- * [rows, I] contiguous; rw, d_rw: bf16 arrays indexed by flat (every flat index occurs once). I % 8 == 0. */
+ * d_u = silu(g) (d_hw w); d_g = silu'(g) ((d_hw w) u). g, u, d_hw and the outputs hw, d_g, d_u: [rows, I] with
+ * row strides (multiples of 8; d_g and d_u may be the halves of one [rows, 2 I] buffer); rw, d_rw: bf16 arrays
+ * indexed by flat (every flat index occurs once). I % 8 == 0. */
 int vx_moe_swiglu_bwd(const void* g, const void* u, const void* d_hw, int64_t ldg, int64_t ldu, int64_t ldd,
-                      const void* rw, const int* flat, void* hw, void* d_g, void* d_u, void* d_rw, int64_t rows,
-                      int64_t I, hipStream_t stream);
+                      const void* rw, const int* flat, void* hw, void* d_g, void* d_u, void* d_rw, int64_t ld_hw,
+                      int64_t ld_dg, int64_t ld_du, int64_t rows, int64_t I, hipStream_t stream);
 int vx_moe_gemm_tn(const void* dy, int64_t lddy, const int* dy_src, const void* x, int64_t ldx, const int* x_src,
                    void* dw, int64_t lddw, int64_t dw_gstride, int64_t N, int64_t K, const int* cu,
                    int64_t num_experts, int64_t dy_rows, int64_t x_rows, hipStream_t stream);

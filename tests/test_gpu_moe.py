@@ -426,6 +426,37 @@ def test_backward_on_256_row_tiles_gives_the_gradient_bits_of_128_row_tiles(monk
         assert_bitwise(a, b, f"grad of {name}")
 
 
+@pytest.mark.parametrize("T,H,I,E,k", [(48, 128, 64, 8, 2), (2304, 256, 320, 8, 2), (300, 64, 24, 4, 4)])
+def test_stacked_gate_up_backward_gives_the_bits_of_the_split_backward(T, H, I, E, k):
+    # fc1_1_2_weight = one [E, 2I, H] parameter: FusedMoeStackedFunction (one recompute, one data-gradient product over
+    # K = 2I, one weight-gradient launch into the stacked gradient) against FusedMoeExpertFunction on the two slices,
+    # whose gradients autograd scatters back into the same leaf
+    from vexact_amd.batch_invariant_ops.fused_moe import fused_moe_forward
+    g = torch.Generator().manual_seed(T + I)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    gu = (torch.randn(E, 2 * I, H, generator=g) * 0.08).to(torch.bfloat16)
+    dw = (torch.randn(E, H, I, generator=g) * 0.08).to(torch.bfloat16)
+    w, sel = torch.topk(torch.softmax(torch.randn(T, E, generator=g), -1), k)
+    w = (w / w.sum(-1, keepdim=True)).to(torch.bfloat16)
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).cuda()
+
+    def grads(stacked):
+        lw, lx, lgu, ldw = (t.cuda().requires_grad_() for t in (w, x, gu, dw))
+        if stacked:
+            out = fused_moe_forward(E, lw, sel.cuda(), lx, None, None, ldw, fc1_1_2_weight=lgu)
+        else:
+            out = fused_moe_forward(E, lw, sel.cuda(), lx, lgu[:, :I], lgu[:, I:], ldw)
+        out.backward(dy)
+        return out.detach(), [t.grad for t in (lw, lx, lgu, ldw)]
+
+    out_s, gs = grads(True)
+    out_p, gp = grads(False)
+    assert_bitwise(out_s, out_p, "forward")
+    for name, a, b in zip(("routing weights", "hidden states", "stacked gate/up", "down"), gs, gp):
+        assert a.shape == b.shape
+        assert_bitwise(a, b, f"grad of {name}")
+
+
 def test_patched_sparse_moe_block_matches_oracle_and_is_batch_invariant():
     # Qwen3MoeSparseMoeBlock after apply_qwen3_moe_patches: router + fused experts on the GPU against the CPU
     # restatements; a token alone gives the bits it gives in the batch; one expert called directly == dense MLP

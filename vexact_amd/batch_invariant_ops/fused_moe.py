@@ -6,8 +6,9 @@ Mirrors ``fused_moe_forward`` of ``vexact/batch_invariant_ops/fused_moe.py:459-4
 ``FusedMoeExpertFunction.forward`` (fused_moe.py:24-102): bf16 gate/up projections, bf16
 ``silu(g) * u``, routing weight applied before the down projection, fp32 sum over a token's slots
 in slot order. The backward (``FusedMoeExpertFunction.backward``, fused_moe.py:126-265) recomputes
-the gate / up projections with the same grouped kernel and runs the dgrad / wgrad products as plain
-per-expert library GEMMs: only the forward has to match the rollout bit for bit.
+the gate / up projections with the forward's grouped kernel and runs the data- and weight-gradient
+products on the grouped kernels of ``csrc/moe_bwd.hip``; only the forward has to match the rollout bit
+for bit.
 """
 
 from __future__ import annotations
@@ -88,6 +89,47 @@ class FusedMoeExpertFunction(torch.autograd.Function):
                 d_x.reshape(hidden_states.shape), d_g_w, d_u_w, d_d_w)
 
 
+class FusedMoeStackedFunction(torch.autograd.Function):
+    """``FusedMoeExpertFunction`` for gate and up projections stacked in one tensor ``[E, 2I, H]`` (the layout of
+    ``Qwen3MoeExperts.gate_up_proj``; not in the reference, which slices the stacked parameter and lets autograd
+    scatter the two gradients back into a zero-filled ``[E, 2I, H]`` each). Same forward; the backward treats
+    gate and up as one projection of width 2 I: one recompute launch, one data-gradient product over K = 2 I
+    (the accumulation chain of ``d_g W_gate + d_u W_up``, so the same bits) and one weight-gradient launch that
+    writes the stacked gradient directly."""
+
+    @staticmethod
+    def forward(ctx, num_experts, routing_weights, selected_experts, hidden_states, gate_up_w, down_w):
+        x = hidden_states.reshape(-1, hidden_states.shape[-1])
+        inter = gate_up_w.shape[1] // 2
+        out = ops.fused_moe(x, routing_weights.reshape(x.shape[0], -1), selected_experts.reshape(x.shape[0], -1),
+                            gate_up_w[:, :inter], gate_up_w[:, inter:], down_w, num_experts)
+        ctx.num_experts = num_experts
+        ctx.save_for_backward(routing_weights, selected_experts, hidden_states, gate_up_w, down_w)
+        return out.reshape(hidden_states.shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        routing_weights, selected_experts, hidden_states, gate_up_w, down_w = ctx.saved_tensors
+        E = ctx.num_experts
+        H, inter = hidden_states.shape[-1], gate_up_w.shape[1] // 2
+        x = hidden_states.reshape(-1, H)
+        T, k = x.shape[0], selected_experts.reshape(x.shape[0], -1).shape[1]
+        dy = grad_output.reshape(-1, H).to(torch.bfloat16)
+        wide_ok = H % 64 == 0 and inter % 64 == 0
+        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok))
+        gu = ops.moe_gemm(x, gate_up_w, r, row_src=r.sorted_token)                 # [T k, 2I]: gate | up, as the forward
+        d_hw = ops.moe_gemm_nn(dy, down_w, r, a_src=r.sorted_token)
+        d_gu = torch.empty_like(gu)
+        hw, _, _, grad_rw = ops.moe_swiglu_backward(gu[:, :inter], gu[:, inter:], d_hw, routing_weights.reshape(T, k),
+                                                    r.sorted_flat, d_g_out=d_gu[:, :inter], d_u_out=d_gu[:, inter:])
+        d_d_w = ops.moe_gemm_tn(dy, hw, r.cu, E, dy_src=r.sorted_token) if ctx.needs_input_grad[5] else None
+        d_xs = ops.moe_gemm_nn(d_gu, gate_up_w, r)
+        d_gu_w = ops.moe_gemm_tn(d_gu, x, r.cu, E, x_src=r.sorted_token) if ctx.needs_input_grad[4] else None
+        d_x = ops.moe_gather(d_xs, r.scatter_index)
+        return (None, grad_rw.reshape(routing_weights.shape).to(routing_weights.dtype), None,
+                d_x.reshape(hidden_states.shape), d_gu_w, d_d_w)
+
+
 def fused_moe_forward(
     num_experts: int,
     routing_weights: torch.Tensor,
@@ -117,6 +159,11 @@ def fused_moe_forward(
         down_w = down_w.contiguous()
     shape = hidden_states.shape
     if torch.is_grad_enabled() and any(t.requires_grad for t in (routing_weights, hidden_states, gate_w, up_w, down_w)):
+        stacked = fc1_1_2_weight
+        if (stacked is not None and stacked.dtype == torch.bfloat16 and stacked.stride(2) == 1
+                and stacked.shape[1] % 16 == 0 and stacked.shape[2] % 8 == 0):
+            out = FusedMoeStackedFunction.apply(num_experts, routing_weights, selected_experts, hidden_states, stacked, down_w)
+            return out if residual is None else residual + out
         out = FusedMoeExpertFunction.apply(num_experts, routing_weights, selected_experts, hidden_states, gate_w, up_w,
                                            down_w)
         return out if residual is None else residual + out

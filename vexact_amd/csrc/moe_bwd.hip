@@ -680,7 +680,8 @@ __global__ __launch_bounds__(256) void moe_swiglu_bwd_kernel(const bf16_t* __res
                                                              int64_t ldd, const bf16_t* __restrict__ rw,
                                                              const int* __restrict__ flat, bf16_t* __restrict__ hw,
                                                              bf16_t* __restrict__ d_g, bf16_t* __restrict__ d_u,
-                                                             bf16_t* __restrict__ d_rw, int64_t rows, int I) {
+                                                             bf16_t* __restrict__ d_rw, int64_t ldh, int64_t ldog,
+                                                             int64_t ldou, int64_t rows, int I) {
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= rows) return;
@@ -713,9 +714,9 @@ __global__ __launch_bounds__(256) void moe_swiglu_bwd_kernel(const bf16_t* __res
       og[j] = pack_bf16x2(res[1][0], res[1][1]);
       ou[j] = pack_bf16x2(res[2][0], res[2][1]);
     }
-    *(uint4*)(hw + r * (int64_t)I + 8 * v) = make_uint4(oh[0], oh[1], oh[2], oh[3]);
-    *(uint4*)(d_g + r * (int64_t)I + 8 * v) = make_uint4(og[0], og[1], og[2], og[3]);
-    *(uint4*)(d_u + r * (int64_t)I + 8 * v) = make_uint4(ou[0], ou[1], ou[2], ou[3]);
+    *(uint4*)(hw + r * ldh + 8 * v) = make_uint4(oh[0], oh[1], oh[2], oh[3]);
+    *(uint4*)(d_g + r * ldog + 8 * v) = make_uint4(og[0], og[1], og[2], og[3]);
+    *(uint4*)(d_u + r * ldou + 8 * v) = make_uint4(ou[0], ou[1], ou[2], ou[3]);
   }
   part = wave_sum(part);
   if (lane == 0) d_rw[f] = f32_to_bf16(part);
@@ -780,18 +781,18 @@ int vx_moe_gemm_nn(const void* a, int64_t lda, const int* a_src, const void* w, 
 }
 
 int vx_moe_swiglu_bwd(const void* g, const void* u, const void* d_hw, int64_t ldg, int64_t ldu, int64_t ldd,
-                      const void* rw, const int* flat, void* hw, void* d_g, void* d_u, void* d_rw, int64_t rows,
-                      int64_t I, hipStream_t stream) {
+                      const void* rw, const int* flat, void* hw, void* d_g, void* d_u, void* d_rw, int64_t ld_hw,
+                      int64_t ld_dg, int64_t ld_du, int64_t rows, int64_t I, hipStream_t stream) {
   if (!g || !u || !d_hw || !rw || !flat || !hw || !d_g || !d_u || !d_rw) return VX_ERR_ARG;
   if (rows < 0 || I <= 0 || I > 0x7fffffff) return VX_ERR_ARG;
-  if (I % 8 || ldg % 8 || ldu % 8 || ldd % 8 || !al16(g) || !al16(u) || !al16(d_hw) || !al16(hw) || !al16(d_g) || !al16(d_u))
+  if (I % 8 || ldg % 8 || ldu % 8 || ldd % 8 || ld_hw % 8 || ld_dg % 8 || ld_du % 8 || !al16(g) || !al16(u) || !al16(d_hw) || !al16(hw) || !al16(d_g) || !al16(d_u))
     return VX_ERR_UNSUPPORTED;
   if (rows == 0) return VX_OK;
   const int64_t blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffffLL) return VX_ERR_UNSUPPORTED;
   moe_swiglu_bwd_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)g, (const bf16_t*)u, (const bf16_t*)d_hw, ldg,
                                                               ldu, ldd, (const bf16_t*)rw, flat, (bf16_t*)hw, (bf16_t*)d_g,
-                                                              (bf16_t*)d_u, (bf16_t*)d_rw, rows, (int)I);
+                                                              (bf16_t*)d_u, (bf16_t*)d_rw, ld_hw, ld_dg, ld_du, rows, (int)I);
   return launch_status();
 }
 

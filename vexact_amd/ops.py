@@ -812,21 +812,26 @@ def moe_gemm_tn(
 
 
 def moe_swiglu_backward(g: torch.Tensor, u: torch.Tensor, d_hw: torch.Tensor, routing_weights: torch.Tensor,
-                        sorted_flat: torch.Tensor):
+                        sorted_flat: torch.Tensor, d_g_out: Optional[torch.Tensor] = None,
+                        d_u_out: Optional[torch.Tensor] = None):
     """The elementwise step of the fused-MoE backward in one launch. ``g``, ``u``, ``d_hw`` are ``[T k, I]`` in
-    sorted-row order, ``routing_weights [T, k]`` bf16, ``sorted_flat`` the (token, slot) flat index of each sorted
-    row. Returns ``(hw, d_g, d_u, d_routing_weights [T, k])``."""
+    sorted-row order (any row strides), ``routing_weights [T, k]`` bf16, ``sorted_flat`` the (token, slot) flat
+    index of each sorted row. Returns ``(hw, d_g, d_u, d_routing_weights [T, k])``; ``d_g_out`` / ``d_u_out`` may
+    be the two halves of one ``[T k, 2 I]`` buffer."""
     n, I = g.shape
-    for t in (g, u, d_hw):
+    hw = _empty((n, I), dtype=torch.bfloat16, device=g.device)
+    d_g = d_g_out if d_g_out is not None else _empty((n, I), dtype=torch.bfloat16, device=g.device)
+    d_u = d_u_out if d_u_out is not None else _empty((n, I), dtype=torch.bfloat16, device=g.device)
+    for t in (g, u, d_hw, d_g, d_u):
         assert t.dtype == torch.bfloat16 and t.shape == (n, I) and t.stride(1) == 1
     rw = routing_weights.contiguous()
     assert rw.dtype == torch.bfloat16 and rw.numel() == n and sorted_flat.dtype == torch.int32 and sorted_flat.numel() == n
-    hw, d_g, d_u = (_empty((n, I), dtype=torch.bfloat16, device=g.device) for _ in range(3))
     d_rw = _empty(rw.shape, dtype=torch.bfloat16, device=g.device)
     _lib.check(
         _lib.load().vx_moe_swiglu_bwd(
             g.data_ptr(), u.data_ptr(), d_hw.data_ptr(), g.stride(0), u.stride(0), d_hw.stride(0), rw.data_ptr(),
-            sorted_flat.data_ptr(), hw.data_ptr(), d_g.data_ptr(), d_u.data_ptr(), d_rw.data_ptr(), n, I, _stream(),
+            sorted_flat.data_ptr(), hw.data_ptr(), d_g.data_ptr(), d_u.data_ptr(), d_rw.data_ptr(), hw.stride(0),
+            d_g.stride(0), d_u.stride(0), n, I, _stream(),
         ),
         "vx_moe_swiglu_bwd",
     )
