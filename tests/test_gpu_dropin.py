@@ -314,6 +314,37 @@ def test_fused_rms_norm_patch_gives_the_bits_of_the_unfused_forward():
             assert_bitwise(fused, unfused, f"fused RMSNorm forward, shape {shape}, {dtype}")
             with torch.inference_mode():  # outside the mode the original forward runs
                 assert_bitwise(norm(x), original(norm, x), "outside batch-invariant mode")
+        # Rows of small entries reach arguments where the GPU's torch.rsqrt and the kernel's 1 / sqrt (the CPU's
+        # torch.rsqrt) differ by an fp32 ulp: a few elements in 10^5 then round to the neighbouring bf16 value
+        for n in (64, 320, 2048):
+            norm = hf.Qwen3MoeRMSNorm(n, eps=1e-6).to(BF).cuda()
+            x = (0.05 * torch.randn(600, n, generator=g)).to(BF).cuda()
+            with torch.inference_mode(), set_batch_invariant_mode(True):
+                fused, unfused = norm(x), original(norm, x)
+            ulp = (fused.view(torch.int16).int() - unfused.view(torch.int16).int()).abs()
+            assert int(ulp.max()) <= 1 and int((ulp > 0).sum()) <= 1e-4 * ulp.numel(), f"n={n}: {int((ulp > 0).sum())} elements differ"
+        # with autograd the same kernel runs (the trainer's forward is the rollout's), and its backward is the
+        # derivative of the original forward
+        norm = hf.Qwen3MoeRMSNorm(256, eps=1e-6)
+        with torch.no_grad():
+            norm.weight.copy_(1.0 + 0.2 * torch.randn(256, generator=g))
+        norm = norm.to(BF).cuda()
+        x = torch.randn(2, 50, 256, generator=g).to(BF).cuda()
+        dy = torch.randn(2, 50, 256, generator=g).to(BF).cuda()
+        with torch.inference_mode(), set_batch_invariant_mode(True):
+            rollout = norm(x)
+        xa = x.clone().requires_grad_()
+        with set_batch_invariant_mode(True):
+            ya = norm(xa)
+        assert_bitwise(ya.detach(), rollout, "forward under autograd")
+        ya.backward(dy)
+        got_x, got_w = xa.grad, norm.weight.grad.clone()
+        norm.weight.grad = None
+        xb = x.clone().requires_grad_()
+        original(norm, xb).backward(dy)
+        for name, a, b in (("input", got_x, xb.grad), ("weight", got_w, norm.weight.grad)):
+            err, scale = (a.float() - b.float()).abs(), float(b.float().abs().max())
+            assert float(err.max()) <= 2e-2 * scale, f"RMSNorm gradient of the {name}: {float(err.max()):.4g} vs scale {scale:.4g}"
     finally:
         remove_qwen3_moe_patches()
     assert hf.Qwen3MoeRMSNorm.forward is original
@@ -447,3 +478,144 @@ def test_fused_attention_and_residual_patches_give_the_bits_of_the_unfused_forwa
         else:
             ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had
     assert hf.Qwen3MoeAttention.forward is original and hf.Qwen3MoeDecoderLayer.forward is original_layer
+
+
+def _fp32_reference_logits(P, ids, lens, selected, cfg):
+    """The tiny model in plain fp32 tensor operations on the CPU (autograd-friendly): RMSNorm, q/k/v, per-head norm,
+    rotary embedding, causal attention per sequence with grouped kv heads, the MoE block on the GPU's expert choice."""
+    Hq, Hkv, D, k = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.num_experts_per_tok
+
+    def rms(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + cfg.rms_norm_eps) * w
+
+    def rot(x, cos, sin):
+        x1, x2 = x[..., : D // 2], x[..., D // 2:]
+        return x * cos[:, None, :] + torch.cat([-x2, x1], -1) * sin[:, None, :]
+
+    T = len(ids)
+    h = P["model.embed_tokens.weight"][torch.as_tensor(ids)]
+    pos = torch.cat([torch.arange(n) for n in lens]).float()
+    inv = 1.0 / (1.0e6 ** (torch.arange(0, D, 2).float() / D))
+    ang = pos[:, None] * inv[None, :]
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1), torch.cat([ang.sin(), ang.sin()], -1)
+    for l in range(cfg.num_hidden_layers):
+        pre = f"model.layers.{l}."
+        x = rms(h, P[pre + "input_layernorm.weight"])
+        q = (x @ P[pre + "self_attn.q_proj.weight"].t()).view(T, Hq, D)
+        kk = (x @ P[pre + "self_attn.k_proj.weight"].t()).view(T, Hkv, D)
+        v = (x @ P[pre + "self_attn.v_proj.weight"].t()).view(T, Hkv, D)
+        q, kk = rot(rms(q, P[pre + "self_attn.q_norm.weight"]), cos, sin), rot(rms(kk, P[pre + "self_attn.k_norm.weight"]), cos, sin)
+        outs, o = [], 0
+        for n in lens:
+            qs = q[o:o + n].transpose(0, 1)                                        # [Hq, n, D]
+            ks = kk[o:o + n].transpose(0, 1).repeat_interleave(Hq // Hkv, dim=0)
+            vs = v[o:o + n].transpose(0, 1).repeat_interleave(Hq // Hkv, dim=0)
+            s = (qs @ ks.transpose(1, 2)) * D ** -0.5
+            s = s.masked_fill(torch.ones(n, n, dtype=torch.bool).triu(1), float("-inf"))
+            outs.append((torch.softmax(s, -1) @ vs).transpose(0, 1).reshape(n, Hq * D))
+            o += n
+        h = h + torch.cat(outs) @ P[pre + "self_attn.o_proj.weight"].t()
+        x = rms(h, P[pre + "post_attention_layernorm.weight"])
+        probs = torch.softmax(x @ P[pre + "mlp.gate.weight"].t(), -1)
+        sel = selected[l]
+        w = probs.gather(-1, sel)
+        w = w / w.sum(-1, keepdim=True)
+        gu, dn = P[pre + "mlp.experts.gate_up_proj"], P[pre + "mlp.experts.down_proj"]
+        inter = gu.shape[1] // 2
+        moe = torch.zeros_like(h)
+        for i in range(k):
+            e = sel[:, i]
+            gate = torch.einsum("th,tih->ti", x, gu[e, :inter])
+            up = torch.einsum("th,tih->ti", x, gu[e, inter:])
+            moe = moe + w[:, i: i + 1] * torch.einsum("ti,thi->th", torch.nn.functional.silu(gate) * up, dn[e])
+        h = h + moe
+    return rms(h, P["model.norm.weight"]) @ P["lm_head.weight"].t()
+
+
+def test_training_forward_gives_the_rollout_bits_and_its_gradients_match_an_fp32_model():
+    """The property the reference exists for: the trainer's forward (packed sequences, no cache, autograd on, the packed
+    attention and fused-MoE autograd functions) reproduces the rollout's logits (paged prefill, inference mode, every fused
+    patch) bit for bit, so on-policy logprobs are exact; and its backward gives the gradients of the model (against the
+    same model in fp32 tensor operations on the CPU, following the GPU's expert choice), router weights included."""
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+    from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
+    from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
+    from vexact_amd.decoder import build_step_metadata
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+
+    page = 16
+    cache_cfg = types.SimpleNamespace(page_size=page, max_cache_blocks=40)
+    had = ALL_ATTENTION_FUNCTIONS._global_mapping.get("triton-invariant") if hasattr(ALL_ATTENTION_FUNCTIONS, "_global_mapping") else None
+    ALL_ATTENTION_FUNCTIONS["triton-invariant"] = flash_attention_forward
+    apply_qwen3_moe_patches()
+    try:
+        hf_cfg, model = _build_model(seed=31)
+        model = model.cuda()
+        rng = np.random.default_rng(32)
+        lens = [37, 5, 120]
+        ids = np.concatenate([rng.integers(0, hf_cfg.vocab_size, size=n) for n in lens])
+        targets = torch.as_tensor(rng.integers(0, hf_cfg.vocab_size, size=len(ids)))
+        ids_d = torch.as_tensor(ids)[None].cuda()
+        # ---- rollout: paged prefill in inference mode
+        blocks, nxt = [], 0
+        for n in lens:
+            blocks.append(list(range(nxt, nxt + -(-n // page))))
+            nxt += len(blocks[-1])
+        meta = build_step_metadata([dict(num_computed_tokens=n, tokens_this_step=n, block_ids=b) for n, b in zip(lens, blocks)], page, 16)
+        dev = {k: torch.as_tensor(v).cuda() for k, v in meta.items() if k != "max_seqlen_q"}
+        store = KVCacheStore(hf_cfg, cache_cfg, torch.device("cuda"))
+        set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache,
+                             block_tables=dev["block_tables"], context_lens=dev["context_lens"], slot_mapping=dev["slot_mapping"],
+                             query_start_loc=dev["query_start_loc"], max_seqlen_q=int(meta["max_seqlen_q"]))
+        try:
+            with torch.inference_mode(), set_batch_invariant_mode(True):
+                out = model.model(input_ids=ids_d, position_ids=dev["positions"][None], use_cache=False, return_dict=True)
+                rollout = model.lm_head(out.last_hidden_state)[0].clone()
+        finally:
+            clear_kv_cache_context()
+        # ---- trainer: the same tokens as a packed batch, gradients on
+        selected = []
+        hooks = [l.mlp.experts.register_forward_pre_hook(lambda mod, args, kw: selected.append(kw["selected_experts"].detach().cpu()),
+                                                         with_kwargs=True) for l in model.model.layers]
+        for p in model.parameters():
+            p.requires_grad_(True)
+        set_kv_cache_context(is_paged_attn=False, context_lens=dev["context_lens"], query_start_loc=dev["query_start_loc"],
+                             max_seqlen_q=int(meta["max_seqlen_q"]))
+        try:
+            with set_batch_invariant_mode(True):
+                out = model.model(input_ids=ids_d, position_ids=dev["positions"][None], use_cache=False, return_dict=True)
+                logits = model.lm_head(out.last_hidden_state)[0]
+                assert logits.requires_grad
+                assert_bitwise(logits.detach(), rollout, "trainer's logits vs the rollout's")
+                lp = torch.log_softmax(logits.float(), -1).gather(-1, targets.cuda()[:, None])[:, 0]
+                (-lp.sum()).backward()
+        finally:
+            clear_kv_cache_context()
+            for h in hooks:
+                h.remove()
+        # ---- the same model in fp32 on the CPU
+        P = {n: p.detach().cpu().float().requires_grad_() for n, p in model.named_parameters()}
+        ref_logits = _fp32_reference_logits(P, ids, lens, selected, hf_cfg)
+        ref_lp = torch.log_softmax(ref_logits, -1).gather(-1, targets[:, None])[:, 0]
+        assert float((lp.detach().cpu() - ref_lp.detach()).abs().max()) <= 0.1, "logprobs vs the fp32 model"
+        (-ref_lp.sum()).backward()
+        worst = []
+        for n, p in model.named_parameters():
+            assert p.grad is not None, f"no gradient for {n}"
+            want = P[n].grad
+            err, scale = (p.grad.detach().cpu().float() - want).abs(), float(want.abs().max())
+            worst.append((float(err.max()) / max(scale, 1e-12), n))
+            assert float(err.max()) <= 0.08 * scale + 1e-6 and float(err.mean()) <= 0.01 * scale + 1e-7, (
+                f"grad of {n}: max err {float(err.max()):.4g}, mean {float(err.mean()):.4g}, scale {scale:.4g}")
+        worst.sort(reverse=True)
+        print("largest gradient errors relative to the largest entry:", [(round(e, 4), n) for e, n in worst[:4]], flush=True)
+    finally:
+        remove_qwen3_moe_patches()
+        if had is None:
+            try:
+                del ALL_ATTENTION_FUNCTIONS._global_mapping["triton-invariant"]
+            except Exception:
+                pass
+        else:
+            ALL_ATTENTION_FUNCTIONS["triton-invariant"] = had

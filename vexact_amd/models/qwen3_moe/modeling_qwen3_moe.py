@@ -92,6 +92,34 @@ class Qwen3MoeExperts(nn.Module):
         )
 
 
+class RouterTopKFunction(torch.autograd.Function):
+    """``ops.router_topk`` with a gradient for the router logits, for the training side. The reference's block
+    runs softmax -> top-k -> renormalise -> cast as tensor operations (modeling_qwen3_moe.py:128-134), which
+    autograd differentiates; here the forward stays the one kernel of the rollout (same bits) and the backward
+    applies the derivative of those operations to the recomputed fp32 softmax."""
+
+    @staticmethod
+    def forward(ctx, router_logits, top_k, renorm, out_dtype):
+        weights, selected = ops.router_topk(router_logits, top_k, renorm=renorm, out_dtype=out_dtype, index_dtype=torch.int64)
+        ctx.save_for_backward(router_logits, selected)
+        ctx.renorm = renorm
+        ctx.mark_non_differentiable(selected)
+        return weights, selected
+
+    @staticmethod
+    def backward(ctx, d_weights, _):
+        router_logits, selected = ctx.saved_tensors
+        p = torch.softmax(router_logits.float(), dim=-1)
+        d_sel = d_weights.float()
+        if ctx.renorm:
+            sel = p.gather(-1, selected)
+            s = sel.sum(-1, keepdim=True)
+            d_sel = (d_sel - (d_sel * (sel / s)).sum(-1, keepdim=True)) / s
+        d_p = torch.zeros_like(p).scatter_(-1, selected, d_sel)
+        d_logits = p * (d_p - (d_p * p).sum(-1, keepdim=True))
+        return d_logits.to(router_logits.dtype), None, None, None
+
+
 def moe_block_init(self, config):
     """Replacement for ``Qwen3MoeSparseMoeBlock.__init__``: a plain linear router and fused experts."""
     nn.Module.__init__(self)
@@ -116,8 +144,11 @@ def moe_block_forward(self, hidden_states: torch.Tensor, residual: Optional[torc
     batch_size, sequence_length, hidden_dim = hidden_states.shape
     x = hidden_states.view(-1, hidden_dim)
     router_logits = self.gate(x)  # aten::mm -> the batch-invariant GEMM when the mode is on
-    routing_weights, selected_experts = ops.router_topk(
-        router_logits, self.top_k, renorm=bool(self.norm_topk_prob), out_dtype=x.dtype, index_dtype=torch.int64)
+    if torch.is_grad_enabled() and router_logits.requires_grad:
+        routing_weights, selected_experts = RouterTopKFunction.apply(router_logits, self.top_k, bool(self.norm_topk_prob), x.dtype)
+    else:
+        routing_weights, selected_experts = ops.router_topk(
+            router_logits, self.top_k, renorm=bool(self.norm_topk_prob), out_dtype=x.dtype, index_dtype=torch.int64)
     res = None if residual is None else residual.reshape(-1, hidden_dim)
     out = self.experts(x, routing_weights=routing_weights, selected_experts=selected_experts, residual=res)
     return out.reshape(batch_size, sequence_length, hidden_dim)
@@ -134,19 +165,49 @@ def invalidate_packed_experts(model: nn.Module) -> int:
     return n
 
 
+class RmsNormFunction(torch.autograd.Function):
+    """The fused RMSNorm with a backward, so that a trainer's forward runs the kernel the rollout ran (the same
+    bits, which the tensor-operation forward does not give in every element: its ``torch.rsqrt`` on the GPU and the
+    kernel's ``1 / sqrt`` differ by an fp32 ulp now and then). Backward: the RMSNorm derivative in fp32 tensor
+    operations, ``d_x = inv (d_h - h mean(d_h h))`` with ``h = x inv``, ``d_h = d_y w``, ``d_w = sum d_y r(h)``."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, weight, eps):
+        ctx.save_for_backward(hidden_states, weight)
+        ctx.eps = eps
+        return ops.rms_norm(hidden_states, weight, eps, hf_two_rounding=True)
+
+    @staticmethod
+    def backward(ctx, d_y):
+        x, w = ctx.saved_tensors
+        x32, dy32 = x.float(), d_y.float()
+        inv = torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + ctx.eps)
+        h = x32 * inv
+        d_w = None
+        if ctx.needs_input_grad[1]:
+            d_w = (dy32 * h.to(x.dtype).float()).reshape(-1, x.shape[-1]).sum(0).to(w.dtype)
+        d_x = None
+        if ctx.needs_input_grad[0]:
+            d_h = dy32 * w.float()
+            d_x = (inv * (d_h - h * (d_h * h).mean(-1, keepdim=True))).to(x.dtype)
+        return d_x, d_w, None
+
+
 def fused_rms_norm_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
     """``Qwen3MoeRMSNorm.forward`` as one kernel. HuggingFace's forward (cast to fp32, ``pow(2).mean(-1)``, ``rsqrt``,
     two multiplies and two casts: eleven launches under batch-invariant mode) rounds ``x * rsqrt(var + eps)`` to
     the input dtype and then multiplies by the weight; ``ops.rms_norm(..., hf_two_rounding=True)`` keeps both
-    roundings and the batch-invariant mean's summation order, so the bits are the ones the unfused forward gives
-    under ``set_batch_invariant_mode(True)``. Outside that mode, off the GPU or with a weight of another dtype
-    the original forward runs."""
+    roundings and the batch-invariant mean's summation order. Its ``1 / sqrt`` is the CPU's ``torch.rsqrt``; the
+    GPU's differs from it by an fp32 ulp now and then, which shows in about one output element in 10^5. With
+    autograd the same kernel runs (``RmsNormFunction``), so rollout and trainer agree bit for bit. Outside
+    batch-invariant mode, off the GPU or with a weight of another dtype the original forward runs."""
     from ...batch_invariant_ops import is_batch_invariant_mode_enabled
 
     w = self.weight
     if (hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float16) and w.dtype == hidden_states.dtype
-            and not (torch.is_grad_enabled() and (hidden_states.requires_grad or w.requires_grad))
             and is_batch_invariant_mode_enabled()):
+        if torch.is_grad_enabled() and (hidden_states.requires_grad or w.requires_grad):
+            return RmsNormFunction.apply(hidden_states, w, self.variance_epsilon)
         return ops.rms_norm(hidden_states, w, self.variance_epsilon, hf_two_rounding=True)
     return _ORIGINAL_NORM(self, hidden_states)
 
@@ -200,7 +261,9 @@ def _fused_qkv_weight(attn) -> torch.Tensor:
                 break
             row += w.shape[0]
     if fused is None:
-        with torch.no_grad():
+        # outside inference mode: tensors made inside it could never take part in autograd again, and these
+        # become the parameters' storage
+        with torch.inference_mode(False), torch.no_grad():
             fused = torch.cat([w.detach() for w in ws], dim=0)
             row = 0
             for w in ws:
