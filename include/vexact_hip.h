@@ -67,6 +67,13 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
                 int64_t rows, int64_t n, int64_t x_stride, void* workspace, int64_t workspace_bytes,
                 hipStream_t stream);
 
+/* Gradient of vx_logprobs with respect to the logits (the backward of the cross-entropy kernel behind the
+ * reference's logprobs_from_logits_flash_attn, standalone_logprobs.py:28-55, whose inplace_backward writes it into the
+ * logits): d_logits[i, j] = d_out[i] ((j == labels[i]) - softmax(logits[i])[j]), from the forward's out (which fixes
+ * logsumexp). d_logits may be logits itself. At most 65535 rows per call. */
+int vx_logprobs_bwd(const void* logits, const int64_t* labels, const float* out, const float* d_out, void* d_logits,
+                    int dtype, int64_t rows, int64_t n, int64_t x_stride, int64_t d_stride, hipStream_t stream);
+
 /* vx_logprobs for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc): no workspace argument, no counterpart in the reference. The chunk partials live in a
  * 1 MiB array inside the library's device image (VX_LOGPROBS_STATIC_BYTES; every GPU the library runs on holds

@@ -541,6 +541,7 @@ def test_training_forward_gives_the_rollout_bits_and_its_gradients_match_an_fp32
 
     from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
     from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
+    from vexact_amd.batch_invariant_ops.standalone_logprobs import logprobs_from_logits_flash_attn
     from vexact_amd.decoder import build_step_metadata
     from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
 
@@ -572,6 +573,7 @@ def test_training_forward_gives_the_rollout_bits_and_its_gradients_match_an_fp32
             with torch.inference_mode(), set_batch_invariant_mode(True):
                 out = model.model(input_ids=ids_d, position_ids=dev["positions"][None], use_cache=False, return_dict=True)
                 rollout = model.lm_head(out.last_hidden_state)[0].clone()
+                rollout_lp = logprobs_from_logits_flash_attn(rollout.float(), targets.cuda())
         finally:
             clear_kv_cache_context()
         # ---- trainer: the same tokens as a packed batch, gradients on
@@ -588,7 +590,8 @@ def test_training_forward_gives_the_rollout_bits_and_its_gradients_match_an_fp32
                 logits = model.lm_head(out.last_hidden_state)[0]
                 assert logits.requires_grad
                 assert_bitwise(logits.detach(), rollout, "trainer's logits vs the rollout's")
-                lp = torch.log_softmax(logits.float(), -1).gather(-1, targets.cuda()[:, None])[:, 0]
+                lp = logprobs_from_logits_flash_attn(logits.float(), targets.cuda(), inplace_backward=True)
+                assert_bitwise(lp.detach(), rollout_lp, "trainer's logprobs vs the rollout's")
                 (-lp.sum()).backward()
         finally:
             clear_kv_cache_context()

@@ -167,3 +167,30 @@ def test_greedy_token_is_first_argmax():
     ref_tok = torch.tensor([int(torch.nonzero(r == r.max())[0]) for r in logits])
     assert torch.equal(tok.cpu(), ref_tok)
     torch.testing.assert_close(lp.cpu(), O.logprobs_ref(logits, ref_tok), atol=2e-5, rtol=0)
+
+
+@pytest.mark.parametrize("rows,n,dtype", [(5, 1000, torch.bfloat16), (64, 151936, torch.bfloat16), (300, 4097, torch.float32),
+                                         (3, 77, torch.float16)])
+def test_logprobs_backward_matches_autograd_of_log_softmax(rows, n, dtype):
+    # logprobs_from_logits_flash_attn under autograd: forward = the inference kernel's bits, backward = d_out (onehot - softmax)
+    # against autograd through an fp32 log_softmax; the in-place form writes the same gradient into the logits
+    from vexact_amd.batch_invariant_ops.standalone_logprobs import logprobs_from_logits_flash_attn
+    g = torch.Generator().manual_seed(rows + n)
+    logits = (3.0 * torch.randn(rows, n, generator=g)).to(dtype).cuda()
+    labels = torch.randint(0, n, (rows,), generator=g).cuda()
+    d_out = torch.randn(rows, generator=g).cuda()
+    plain = logprobs_from_logits_flash_attn(logits, labels)
+    x = logits.clone().requires_grad_()
+    lp = logprobs_from_logits_flash_attn(x, labels)
+    assert_bitwise(lp.detach(), plain, "forward under autograd")
+    lp.backward(d_out)
+    ref_x = logits.float().clone().requires_grad_()
+    torch.log_softmax(ref_x, -1).gather(-1, labels[:, None])[:, 0].backward(d_out)
+    want = ref_x.grad.to(dtype)
+    err = (x.grad.float() - want.float()).abs()
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -7
+    assert float((err / (want.float().abs() + 1e-3)).max()) <= tol, f"gradient: worst relative error {float((err / (want.float().abs() + 1e-3)).max()):.3g}"
+    y = logits.clone().requires_grad_()
+    z = y.clone()                                 # a non-leaf whose memory the in-place backward may take
+    logprobs_from_logits_flash_attn(z, labels, inplace_backward=True).backward(d_out)
+    assert_bitwise(y.grad, x.grad, "in-place backward")

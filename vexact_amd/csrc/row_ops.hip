@@ -5,6 +5,8 @@
 // size depends on the row length only; a thread owns the 4-element vectors t, t+G, t+2G, ...
 // and adds their elements in ascending order, then a lane butterfly and an ascending
 // wave-order pass finish the sum. The schedule never looks at the number of rows.
+#include <algorithm>
+
 #include "common.h"
 #include <math.h>
 #include <atomic>
@@ -411,6 +413,29 @@ static int static_scratch(void** out) {
   return VX_OK;
 }
 
+// Gradient of out[i] = logits[i, label_i] - logsumexp(logits[i, :]) with respect to the logits, from the forward's
+// output: lse_i = logits[i, label_i] - out[i], d_logits[i, j] = d_out[i] ((j == label_i) - exp(logits[i, j] - lse_i)).
+// Elementwise over the row; d_logits may be the logits' own memory (every element is read before it is written).
+template <int DT>
+__global__ __launch_bounds__(256) void logprob_bwd_kernel(const typename Elem<DT>::T* __restrict__ logits,
+                                                          const int64_t* __restrict__ labels,
+                                                          const float* __restrict__ out, const float* __restrict__ d_out,
+                                                          typename Elem<DT>::T* d_logits, int n, int64_t x_stride,
+                                                          int64_t d_stride) {
+  const int64_t row = blockIdx.y;
+  const int64_t lab = labels[row];
+  const typename Elem<DT>::T* x = logits + row * x_stride;
+  typename Elem<DT>::T* d = d_logits + row * d_stride;
+  const float g = d_out[row];
+  const bool has = lab >= 0 && lab < n;
+  const float lse = has ? Elem<DT>::ld(x + lab) - out[row] : 0.f;
+  __syncthreads();  // in place: everyone has read the label's logit before anyone overwrites it
+  for (int j = blockIdx.x * 256 + threadIdx.x; j < n; j += gridDim.x * 256) {
+    const float p = has ? expf(Elem<DT>::ld(x + j) - lse) : 0.f;
+    Elem<DT>::st(d + j, g * ((j == lab ? 1.f : 0.f) - p));
+  }
+}
+
 extern "C" {
 
 int vx_mean_dim(const void* in, void* out, int dtype, int64_t M, int64_t N, int64_t K, int64_t s0,
@@ -571,6 +596,35 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
       logprob_final_kernel<DT_F16><<<blocks, 64, 0, stream>>>((const _Float16*)logits, labels, part,
                                                               out, tokens_out, rows, (int)n,
                                                               x_stride, nchunk);
+      break;
+    default: return VX_ERR_UNSUPPORTED;
+  }
+  return launch_status();
+}
+
+int vx_logprobs_bwd(const void* logits, const int64_t* labels, const float* out, const float* d_out, void* d_logits,
+                    int dtype, int64_t rows, int64_t n, int64_t x_stride, int64_t d_stride, hipStream_t stream) {
+  if (!logits || !labels || !out || !d_out || !d_logits) return VX_ERR_ARG;
+  if (rows < 0 || n <= 0 || n > 0x7fffffff) return VX_ERR_ARG;
+  if (rows == 0) return VX_OK;
+  if (rows > 65535) return VX_ERR_UNSUPPORTED;
+  // Every workgroup must read the label's logit before any workgroup of the row overwrites it when the gradient goes
+  // into the logits' memory: one workgroup per row then; else enough workgroups per row to fill the chip
+  const bool inplace = d_logits == logits;
+  const unsigned gx = inplace ? 1u : (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 2047) / 2048, 2048 / rows + 1));
+  const dim3 grid(gx, (unsigned)rows);
+  switch (dtype) {
+    case DT_F32:
+      logprob_bwd_kernel<DT_F32><<<grid, 256, 0, stream>>>((const float*)logits, labels, out, d_out, (float*)d_logits, (int)n,
+                                                           x_stride, d_stride);
+      break;
+    case DT_BF16:
+      logprob_bwd_kernel<DT_BF16><<<grid, 256, 0, stream>>>((const bf16_t*)logits, labels, out, d_out, (bf16_t*)d_logits,
+                                                            (int)n, x_stride, d_stride);
+      break;
+    case DT_F16:
+      logprob_bwd_kernel<DT_F16><<<grid, 256, 0, stream>>>((const _Float16*)logits, labels, out, d_out,
+                                                           (_Float16*)d_logits, (int)n, x_stride, d_stride);
       break;
     default: return VX_ERR_UNSUPPORTED;
   }

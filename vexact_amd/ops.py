@@ -205,6 +205,28 @@ def logprobs(
     return (out, toks) if return_tokens else out
 
 
+def logprobs_backward(logits: torch.Tensor, labels: torch.Tensor, out: torch.Tensor, d_out: torch.Tensor,
+                      inplace: bool = False) -> torch.Tensor:
+    """Gradient of ``logprobs(logits, labels)`` with respect to ``logits [rows, n]`` given the forward's ``out`` and
+    the incoming ``d_out`` (both fp32 ``[rows]``); ``inplace`` writes it over the logits."""
+    _need_gpu("logits", logits)
+    assert logits.dim() == 2 and logits.stride(1) == 1 and logits.dtype in _DT
+    rows, n = logits.shape
+    lab = labels.reshape(-1).to(torch.int64).contiguous()
+    o, g = out.reshape(-1).float().contiguous(), d_out.reshape(-1).float().contiguous()
+    assert lab.numel() == rows and o.numel() == rows and g.numel() == rows
+    d = logits if inplace else _empty_like(logits)
+    lib = _lib.load()
+    for r0 in range(0, rows, 65535):
+        r = min(65535, rows - r0)
+        _lib.check(
+            lib.vx_logprobs_bwd(logits[r0:].data_ptr(), lab[r0:].data_ptr(), o[r0:].data_ptr(), g[r0:].data_ptr(),
+                                d[r0:].data_ptr(), _DT[logits.dtype], r, n, logits.stride(0), d.stride(0), _stream()),
+            "vx_logprobs_bwd",
+        )
+    return d
+
+
 def sample_tokens(
     logits: torch.Tensor, temperature: float, top_k: Optional[int], top_p: float, seeds: torch.Tensor,
     positions: torch.Tensor, out: Optional[torch.Tensor] = None,
