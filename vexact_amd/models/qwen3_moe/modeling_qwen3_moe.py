@@ -245,12 +245,14 @@ def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **
 _ORIGINAL_ATTN = None  # Qwen3MoeAttention.forward while the fused form is patched in
 
 
-def _fused_qkv_weight(attn) -> torch.Tensor:
+def _fused_qkv_weight(attn) -> Optional[torch.Tensor]:
     """``[q_proj.weight; k_proj.weight; v_proj.weight]`` as one tensor, made once per module: the three
     parameters are then re-pointed at row ranges of it, so there is still one copy of the weights in memory and
     an in-place write to a parameter (``param.data.copy_``, what the reference's weight sync does,
     vexact/inferencer/model_loader.py:113) lands in the fused tensor. A parameter that has been given new
-    storage since is noticed by its address and the fused tensor is rebuilt."""
+    storage since is noticed by its address and the fused tensor is rebuilt. Returns None when it would have to
+    be built while a graph is being captured (its memory would belong to the graph's pool): the caller then runs
+    the unfused forward, as it does for every other case it does not take."""
     ws = (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
     fused = getattr(attn, "_vx_qkv_weight", None)
     if fused is not None:
@@ -260,6 +262,8 @@ def _fused_qkv_weight(attn) -> torch.Tensor:
                 fused = None
                 break
             row += w.shape[0]
+    if fused is None and torch.cuda.is_current_stream_capturing():
+        return None
     if fused is None:
         # outside inference mode: tensors made inside it could never take part in autograd again, and these
         # become the parameters' storage
@@ -301,14 +305,15 @@ def fused_attention_forward(self, hidden_states, position_embeddings, attention_
         and cos.shape == (1, hidden_states.shape[1], D) and cos.is_contiguous() and sin.is_contiguous()
         and ALL_ATTENTION_FUNCTIONS.get(self.config._attn_implementation) is flash_attention_forward
     )
-    if not fits:
+    w_qkv = _fused_qkv_weight(self) if fits else None
+    if w_qkv is None:
         return _ORIGINAL_ATTN(self, hidden_states, position_embeddings, attention_mask, past_key_values, **kwargs)
     T = hidden_states.shape[1]
     Hq, Hkv = self.q_proj.weight.shape[0] // D, self.k_proj.weight.shape[0] // D
     x = hidden_states[0]
     if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
         x = x.contiguous()
-    qkv = ops.gemm_nt(x, _fused_qkv_weight(self))
+    qkv = ops.gemm_nt(x, w_qkv)
     q = ops._empty((T, Hq, D), dtype=torch.bfloat16, device=x.device)
     ops.qk_norm_rope_store(qkv, self.q_norm.weight, self.k_norm.weight, cos[0], sin[0], None, ctx.slot_mapping, q,
                            ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx], Hq, Hkv, D,
