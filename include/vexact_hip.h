@@ -67,6 +67,15 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
                 int64_t rows, int64_t n, int64_t x_stride, void* workspace, int64_t workspace_bytes,
                 hipStream_t stream);
 
+/* Backward of vx_rms_norm without residual (the training side of batch_invariant_rms_norm / of the HuggingFace
+ * RMSNorm forward that mode 1 restates), bf16 or fp16, n % 8 == 0, n <= 8192: d_x = inv (d_h - h mean(d_h h)) with
+ * h = x inv, d_h = d_y w; d_w = sum over rows of d_y r(h) (mode 1) or d_y h (mode 0), accumulated in fp32 in a fixed
+ * order (deterministic for a given number of rows). Workspace: vx_rms_norm_bwd_workspace_bytes(rows, n). */
+int64_t vx_rms_norm_bwd_workspace_bytes(int64_t rows, int64_t n);
+int vx_rms_norm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dw, int dtype, int64_t rows,
+                    int64_t n, int64_t x_stride, int64_t dy_stride, int64_t dx_stride, float eps, int mode,
+                    void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
 /* Gradient of vx_logprobs with respect to the logits (the backward of the cross-entropy kernel behind the
  * reference's logprobs_from_logits_flash_attn, standalone_logprobs.py:28-55, whose inplace_backward writes it into the
  * logits): d_logits[i, j] = d_out[i] ((j == labels[i]) - softmax(logits[i])[j]), from the forward's out (which fixes

@@ -374,6 +374,20 @@ def test_fused_rope_patch_gives_the_bits_of_apply_rotary_pos_emb():
             assert fq.shape == oq.shape and fk.shape == ok.shape
             assert_bitwise(fq, oq, f"rotated queries, B={B} T={T} D={D}")
             assert_bitwise(fk, ok, f"rotated keys, B={B} T={T} D={D}")
+        # with autograd the kernel runs in both directions: the original's output and gradient bits
+        q0 = (2.0 * torch.randn(1, 50, 8, 128, generator=g)).to(BF).cuda()
+        k0 = (2.0 * torch.randn(1, 50, 2, 128, generator=g)).to(BF).cuda()
+        ang = 50.0 * torch.rand(1, 50, 64, generator=g)
+        cos, sin = torch.cat([ang.cos(), ang.cos()], -1).to(BF).cuda(), torch.cat([ang.sin(), ang.sin()], -1).to(BF).cuda()
+        dq, dk = torch.randn(1, 8, 50, 128, generator=g).to(BF).cuda(), torch.randn(1, 2, 50, 128, generator=g).to(BF).cuda()
+        grads = []
+        for fn in (hf.apply_rotary_pos_emb, original):
+            ql, kl = q0.clone().requires_grad_(), k0.clone().requires_grad_()
+            oq, ok = fn(ql.transpose(1, 2), kl.transpose(1, 2), cos, sin)
+            torch.autograd.backward([oq, ok], [dq, dk])
+            grads.append((oq.detach(), ok.detach(), ql.grad, kl.grad))
+        for name, a, b in zip(("rotated queries", "rotated keys", "query gradient", "key gradient"), *grads):
+            assert_bitwise(a, b, f"{name} under autograd")
         # what the kernel does not take falls through to the original (fp32 here)
         q = torch.randn(1, 2, 5, 64, device="cuda"); k = torch.randn(1, 2, 5, 64, device="cuda")
         cos = torch.randn(1, 5, 64, device="cuda"); sin = torch.randn(1, 5, 64, device="cuda")

@@ -194,3 +194,27 @@ def test_logprobs_backward_matches_autograd_of_log_softmax(rows, n, dtype):
     z = y.clone()                                 # a non-leaf whose memory the in-place backward may take
     logprobs_from_logits_flash_attn(z, labels, inplace_backward=True).backward(d_out)
     assert_bitwise(y.grad, x.grad, "in-place backward")
+
+
+@pytest.mark.parametrize("rows,n,dtype", [(37, 2048, torch.bfloat16), (1000, 128, torch.bfloat16), (5, 8192, torch.bfloat16),
+                                         (3000, 256, torch.float16), (1, 64, torch.bfloat16), (70000, 128, torch.bfloat16)])
+def test_rms_norm_backward_matches_autograd(rows, n, dtype):
+    # vx_rms_norm_bwd against autograd through the fp32 formula of the HuggingFace forward (both roundings); deterministic
+    g = torch.Generator().manual_seed(rows + n)
+    x = torch.randn(rows, n, generator=g).to(dtype).cuda()
+    w = (1.0 + 0.2 * torch.randn(n, generator=g)).to(dtype).cuda()
+    dy = torch.randn(rows, n, generator=g).to(dtype).cuda()
+    d_x, d_w = ops.rms_norm_backward(x, w, dy, 1e-6, hf_two_rounding=True)
+    xr, wr = x.float().requires_grad_(), w.float().requires_grad_()
+    h = xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + 1e-6)
+    (wr * h).backward(dy.float())
+    for name, got, want in (("input", d_x, xr.grad), ("weight", d_w, wr.grad)):
+        err, scale = (got.float() - want).abs(), float(want.abs().max())
+        assert float(err.max()) <= 2.0 ** -6 * scale, f"{name} gradient: max err {float(err.max()):.4g} vs scale {scale:.4g}"
+    again = ops.rms_norm_backward(x, w, dy, 1e-6, hf_two_rounding=True)
+    assert_bitwise(again[0], d_x, "second launch, input gradient")
+    assert_bitwise(again[1], d_w, "second launch, weight gradient")
+    # a row's input gradient does not depend on the other rows
+    one = ops.rms_norm_backward(x[rows // 2: rows // 2 + 1].contiguous(), w, dy[rows // 2: rows // 2 + 1].contiguous(), 1e-6,
+                                hf_two_rounding=True)
+    assert_bitwise(one[0], d_x[rows // 2: rows // 2 + 1], "row alone")

@@ -57,6 +57,8 @@ PROTOTYPES = {
     "vx_pack_weights": (_I, [_P, _L, _L, _L, _L, _L, _P, _P]),
     "vx_moe_gemm_packed": (_I, [_P, _L, _P, _P, _L, _P, _L, _L, _L, _P, _P, _P, _L, _I, _P, _P, _P, _I, _L, _P]),
     "vx_moe_gemm_nn": (_I, [_P, _L, _P, _P, _L, _L, _L, _P, _L, _P, _L, _L, _L, _P, _L, _L, _P, _P, _P, _L, _I, _L, _P]),
+    "vx_rms_norm_bwd_workspace_bytes": (_L, [_L, _L]),
+    "vx_rms_norm_bwd": (_I, [_P, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _F, _I, _P, _L, _P]),
     "vx_logprobs_bwd": (_I, [_P, _P, _P, _P, _P, _I, _L, _L, _L, _L, _P]),
     "vx_moe_swiglu_bwd": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _P]),
     "vx_moe_gemm_tn": (_I, [_P, _L, _P, _P, _L, _P, _P, _L, _L, _L, _L, _P, _L, _L, _L, _P]),

@@ -119,7 +119,7 @@ class FusedMoeStackedFunction(torch.autograd.Function):
         r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok))
         gu = ops.moe_gemm(x, gate_up_w, r, row_src=r.sorted_token)                 # [T k, 2I]: gate | up, as the forward
         d_hw = ops.moe_gemm_nn(dy, down_w, r, a_src=r.sorted_token)
-        d_gu = torch.empty_like(gu)
+        d_gu = ops._empty_like(gu)
         hw, _, _, grad_rw = ops.moe_swiglu_backward(gu[:, :inter], gu[:, inter:], d_hw, routing_weights.reshape(T, k),
                                                     r.sorted_flat, d_g_out=d_gu[:, :inter], d_u_out=d_gu[:, inter:])
         d_d_w = ops.moe_gemm_tn(dy, hw, r.cu, E, dy_src=r.sorted_token) if ctx.needs_input_grad[5] else None

@@ -413,6 +413,113 @@ static int static_scratch(void** out) {
   return VX_OK;
 }
 
+// Backward of RMSNorm y = w r(x inv) (mode 1: h = x inv is rounded to the storage type before the weight is applied,
+// as in HuggingFace's forward) or y = r(w x inv) (mode 0), inv = 1 / sqrt(mean(x^2) + eps), for 16-bit storage types:
+//   d_h = d_y w,  d_x = inv (d_h - h mean(d_h h)),  d_w = sum over rows of d_y r(h).
+// G lanes share a row (8-element pieces, up to MAXV per lane); a workgroup's 256 / G row slots walk the rows with the
+// grid's stride and keep d_w sums for their own columns in registers; at the end the slots add them in slot order into
+// LDS and the workgroup writes one fp32 partial row. rms_norm_bwd_finish_kernel adds the partial rows in workgroup
+// order: run-to-run deterministic for a given number of rows.
+template <int DT, int G, int MAXV>
+__global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const typename Elem<DT>::T* __restrict__ x,
+                                                           const typename Elem<DT>::T* __restrict__ w,
+                                                           const typename Elem<DT>::T* __restrict__ dy,
+                                                           typename Elem<DT>::T* __restrict__ dx, float* __restrict__ dw_part,
+                                                           int64_t rows, int n, int64_t xs, int64_t dys, int64_t dxs,
+                                                           float eps, int mode) {
+  using E = Elem<DT>;
+  using T = typename E::T;
+  constexpr int SLOTS = 256 / G;
+  extern __shared__ float rb_red[];  // n floats
+  const int slot = threadIdx.x / G, l = threadIdx.x % G;
+  const int nv = n >> 3;
+  auto ld8 = [](const T* p, float (&f)[8]) {
+    const uint4 raw = *(const uint4*)p;
+    const T* e = (const T*)&raw;
+#pragma unroll
+    for (int c = 0; c < 8; c++) f[c] = E::ld(e + c);
+  };
+  float wf[MAXV][8], acc[MAXV][8];
+#pragma unroll
+  for (int i = 0; i < MAXV; i++) {
+    const int v = l + i * G;
+#pragma unroll
+    for (int c = 0; c < 8; c++) { wf[i][c] = 0.f; acc[i][c] = 0.f; }
+    if (v < nv) ld8(w + 8 * v, wf[i]);
+  }
+  for (int64_t r = (int64_t)blockIdx.x * SLOTS + slot; r < rows; r += (int64_t)gridDim.x * SLOTS) {
+    float xf[MAXV][8], gf[MAXV][8];
+    float ssq = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+      const int v = l + i * G;
+      if (v < nv) {
+        ld8(x + r * xs + 8 * v, xf[i]);
+        ld8(dy + r * dys + 8 * v, gf[i]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 8; c++) { xf[i][c] = 0.f; gf[i][c] = 0.f; }
+      }
+#pragma unroll
+      for (int c = 0; c < 8; c++) ssq += xf[i][c] * xf[i][c];
+    }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o, 64);
+    const float inv = 1.0f / sqrtf(ssq / (float)n + eps);
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXV; i++)
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const float h = xf[i][c] * inv;
+        T hb;
+        E::st(&hb, h);
+        acc[i][c] += gf[i][c] * (mode == 1 ? E::ld(&hb) : h);
+        gf[i][c] *= wf[i][c];  // d_h
+        xf[i][c] = h;
+        dot += gf[i][c] * h;
+      }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
+    const float cm = dot / (float)n;
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+      const int v = l + i * G;
+      if (v < nv) {
+        uint4 o4;
+        T* e = (T*)&o4;
+#pragma unroll
+        for (int c = 0; c < 8; c++) E::st(e + c, inv * (gf[i][c] - xf[i][c] * cm));
+        *(uint4*)(dx + r * dxs + 8 * v) = o4;
+      }
+    }
+  }
+  for (int s = 0; s < SLOTS; s++) {
+    if (slot == s) {
+#pragma unroll
+      for (int i = 0; i < MAXV; i++) {
+        const int v = l + i * G;
+        if (v < nv) {
+#pragma unroll
+          for (int c = 0; c < 8; c++) rb_red[8 * v + c] = (s == 0 ? 0.f : rb_red[8 * v + c]) + acc[i][c];
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int j = threadIdx.x; j < n; j += 256) dw_part[(int64_t)blockIdx.x * n + j] = rb_red[j];
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void rms_norm_bwd_finish_kernel(const float* __restrict__ dw_part, int nblocks, int n,
+                                                                  typename Elem<DT>::T* __restrict__ dw) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= n) return;
+  float s = 0.f;
+  for (int b = 0; b < nblocks; b++) s += dw_part[(int64_t)b * n + j];
+  Elem<DT>::st(dw + j, s);
+}
+
 // Gradient of out[i] = logits[i, label_i] - logsumexp(logits[i, :]) with respect to the logits, from the forward's
 // output: lse_i = logits[i, label_i] - out[i], d_logits[i, j] = d_out[i] ((j == label_i) - exp(logits[i, j] - lse_i)).
 // Elementwise over the row; d_logits may be the logits' own memory (every element is read before it is written).
@@ -599,6 +706,49 @@ int vx_logprobs(const void* logits, const int64_t* labels, float* out, int64_t* 
       break;
     default: return VX_ERR_UNSUPPORTED;
   }
+  return launch_status();
+}
+
+static inline int64_t rms_bwd_blocks(int64_t rows, int64_t n) {
+  const int64_t slots = n <= 128 ? 16 : 4;
+  return std::max<int64_t>(1, std::min<int64_t>((rows + slots - 1) / slots, 512));
+}
+int64_t vx_rms_norm_bwd_workspace_bytes(int64_t rows, int64_t n) {
+  if (rows < 0 || n <= 0) return 0;
+  return rms_bwd_blocks(rows, n) * n * 4;
+}
+int vx_rms_norm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dw, int dtype, int64_t rows,
+                    int64_t n, int64_t x_stride, int64_t dy_stride, int64_t dx_stride, float eps, int mode,
+                    void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  if (!x || !weight || !dy || !dx || !dw || rows < 0 || n <= 0) return VX_ERR_ARG;
+  if (mode != 0 && mode != 1) return VX_ERR_ARG;
+  if ((dtype != DT_BF16 && dtype != DT_F16) || n % 8 != 0 || n > 8192 || (x_stride | dy_stride | dx_stride) % 8 != 0 ||
+      (((uintptr_t)x | (uintptr_t)weight | (uintptr_t)dy | (uintptr_t)dx) % 16 != 0))
+    return VX_ERR_UNSUPPORTED;
+  const int64_t blocks = rms_bwd_blocks(rows, n);
+  if (!workspace || workspace_bytes < blocks * n * 4) return VX_ERR_WORKSPACE;
+  const size_t lds = (size_t)n * 4;
+#define VX_RB(DT, G, MV)                                                                                            \
+  rms_norm_bwd_kernel<DT, G, MV><<<(unsigned)blocks, 256, lds, stream>>>(                                          \
+      (const Elem<DT>::T*)x, (const Elem<DT>::T*)weight, (const Elem<DT>::T*)dy, (Elem<DT>::T*)dx, (float*)workspace, \
+      rows, (int)n, x_stride, dy_stride, dx_stride, eps, mode)
+#define VX_RB_ANY(DT)                      \
+  do {                                     \
+    if (n <= 128) VX_RB(DT, 16, 1);        \
+    else if (n <= 2048) VX_RB(DT, 64, 4);  \
+    else VX_RB(DT, 64, 16);                \
+  } while (0)
+  if (rows > 0) {
+    if (dtype == DT_BF16) VX_RB_ANY(DT_BF16); else VX_RB_ANY(DT_F16);
+  }
+#undef VX_RB_ANY
+#undef VX_RB
+  // no rows: the weight gradient is zero (no partial rows are read)
+  const int nb = rows > 0 ? (int)blocks : 0;
+  if (dtype == DT_BF16)
+    rms_norm_bwd_finish_kernel<DT_BF16><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const float*)workspace, nb, (int)n, (bf16_t*)dw);
+  else
+    rms_norm_bwd_finish_kernel<DT_F16><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const float*)workspace, nb, (int)n, (_Float16*)dw);
   return launch_status();
 }
 

@@ -168,8 +168,9 @@ def invalidate_packed_experts(model: nn.Module) -> int:
 class RmsNormFunction(torch.autograd.Function):
     """The fused RMSNorm with a backward, so that a trainer's forward runs the kernel the rollout ran (the same
     bits, which the tensor-operation forward does not give in every element: its ``torch.rsqrt`` on the GPU and the
-    kernel's ``1 / sqrt`` differ by an fp32 ulp now and then). Backward: the RMSNorm derivative in fp32 tensor
-    operations, ``d_x = inv (d_h - h mean(d_h h))`` with ``h = x inv``, ``d_h = d_y w``, ``d_w = sum d_y r(h)``."""
+    kernel's ``1 / sqrt`` differ by an fp32 ulp now and then). Backward: the RMSNorm derivative,
+    ``d_x = inv (d_h - h mean(d_h h))`` with ``h = x inv``, ``d_h = d_y w``, ``d_w = sum d_y r(h)``, in fp32: one
+    kernel plus a small reduction (``ops.rms_norm_backward``), tensor operations for rows it does not take."""
 
     @staticmethod
     def forward(ctx, hidden_states, weight, eps):
@@ -180,6 +181,10 @@ class RmsNormFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_y):
         x, w = ctx.saved_tensors
+        n = x.shape[-1]
+        if n % 8 == 0 and n <= 8192 and w.dtype == x.dtype:
+            d_x, d_w = ops.rms_norm_backward(x, w, d_y, ctx.eps, hf_two_rounding=True)
+            return (d_x if ctx.needs_input_grad[0] else None), (d_w if ctx.needs_input_grad[1] else None), None
         x32, dy32 = x.float(), d_y.float()
         inv = torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + ctx.eps)
         h = x32 * inv
@@ -216,11 +221,29 @@ _ORIGINAL_NORM = None  # Qwen3MoeRMSNorm.forward while the fused form is patched
 _ORIGINAL_ROPE = None  # the module's apply_rotary_pos_emb while the fused form is patched in
 
 
+class RopeFunction(torch.autograd.Function):
+    """``ops.rope`` with its backward. ``y = x cos + R(x) sin`` with ``R(x) = (-x2, x1)``; ``R`` is antisymmetric and
+    both halves of HuggingFace's ``sin`` are equal, so ``d_x = d_y cos - R(d_y) sin``: the same kernel on ``-sin``, with
+    the bf16 roundings autograd's tensor operations would make."""
+
+    @staticmethod
+    def forward(ctx, x, cos, sin):
+        ctx.save_for_backward(cos, sin)
+        return ops.rope(x, cos, sin)
+
+    @staticmethod
+    def backward(ctx, d_y):
+        cos, sin = ctx.saved_tensors
+        g = d_y if (d_y.stride(2) == 1 and d_y.stride(0) % 4 == 0 and d_y.stride(1) % 4 == 0) else d_y.contiguous()
+        return ops.rope(g, cos, -sin), None, None
+
+
 def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **kwargs):
     """``apply_rotary_pos_emb`` of HuggingFace's Qwen3-MoE modeling file as one launch per tensor instead of five
     (multiply, negate, concatenate, multiply, add). ``q`` / ``k`` are ``[B, heads, T, D]`` views of ``[B, T, heads, D]``
     projections, ``cos`` / ``sin`` ``[B, T, D]``. Elementwise with the same bf16 roundings, so the bits do not change
-    in any mode; other layouts, dtypes or autograd fall through to the original."""
+    in any mode; with autograd the same kernel runs in both directions (``RopeFunction``; ``cos`` / ``sin`` get no
+    gradient, they come from position ids); other layouts or dtypes fall through to the original."""
     def fits(x):
         return (x.dim() == 4 and x.is_cuda and x.dtype == torch.bfloat16 and x.stride(3) == 1 and x.shape[3] % 8 == 0
                 and (x.shape[0] == 1 or x.stride(0) == x.shape[2] * x.stride(2)) and x.stride(1) % 4 == 0 and x.stride(2) % 4 == 0)
@@ -228,7 +251,7 @@ def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **
     if (not args and not kwargs and unsqueeze_dim == 1 and fits(q) and fits(k) and cos.dim() == 3 and cos.dtype == torch.bfloat16
             and sin.dtype == torch.bfloat16 and cos.shape == sin.shape and cos.shape[0] == q.shape[0] == k.shape[0]
             and cos.shape[1] == q.shape[2] == k.shape[2] and cos.shape[2] == q.shape[3] == k.shape[3]
-            and not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad))):
+            and not (torch.is_grad_enabled() and (cos.requires_grad or sin.requires_grad))):
         B, _, T, D = q.shape
         c2, s2 = cos.reshape(B * T, D), sin.reshape(B * T, D)
 
@@ -236,6 +259,8 @@ def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **
             H = x.shape[1]
             rows = x.transpose(1, 2)  # [B, T, H, D]
             flat = rows.as_strided((B * T, H, D), (rows.stride(1), rows.stride(2), 1), rows.storage_offset())
+            if torch.is_grad_enabled() and x.requires_grad:
+                return RopeFunction.apply(flat, c2, s2).view(B, T, H, D).transpose(1, 2)
             return ops.rope(flat, c2, s2).view(B, T, H, D).transpose(1, 2)
 
         return one(q), one(k)

@@ -139,6 +139,34 @@ def rms_norm(
     return y.reshape(x.shape) if out is None else out
 
 
+def rms_norm_backward(x: torch.Tensor, weight: torch.Tensor, d_y: torch.Tensor, eps: float = 1e-6, *,
+                      hf_two_rounding: bool = False):
+    """``(d_x, d_weight)`` of ``rms_norm(x, weight, eps)`` (no residual) for bf16 / fp16 rows of at most 8192 entries
+    (a multiple of 8), in two launches."""
+    _need_gpu("input", x)
+    n = x.shape[-1]
+    assert x.dtype in (torch.bfloat16, torch.float16) and n % 8 == 0 and n <= 8192 and d_y.shape == x.shape
+    x2 = x.reshape(-1, n)
+    g2 = d_y.reshape(-1, n).to(x.dtype)
+    if x2.stride(-1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    if g2.stride(-1) != 1 or g2.stride(0) % 8 or g2.data_ptr() % 16:
+        g2 = g2.contiguous()
+    w = weight.to(x.dtype).contiguous()
+    rows = x2.shape[0]
+    d_x = _empty((rows, n), dtype=x.dtype, device=x.device)
+    d_w = _empty((n,), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    ws = _workspace(lib.vx_rms_norm_bwd_workspace_bytes(rows, n), x.device)
+    _lib.check(
+        lib.vx_rms_norm_bwd(x2.data_ptr(), w.data_ptr(), g2.data_ptr(), d_x.data_ptr(), d_w.data_ptr(), _DT[x.dtype], rows, n,
+                            x2.stride(0), g2.stride(0), d_x.stride(0), float(eps), 1 if hf_two_rounding else 0,
+                            ws.data_ptr(), ws.numel(), _stream()),
+        "vx_rms_norm_bwd",
+    )
+    return d_x.reshape(x.shape), d_w
+
+
 def log_softmax(x: torch.Tensor, dim: int = -1) -> torch.Tensor:
     if dim != -1 and dim != x.ndim - 1:
         raise ValueError("This implementation only supports log_softmax along the last dimension")
