@@ -300,6 +300,13 @@ int vx_moe_gemm_nn(const void* a, int64_t lda, const int* a_src, const void* w, 
                    int64_t K, const void* a2, int64_t lda2, const void* w2, int64_t ldw2, int64_t w2_gstride,
                    int64_t K2, void* c, int64_t ldc, int64_t N, const int* tile_group, const int* tile_row0,
                    const int* tile_rows, int64_t max_tiles, int bm, int64_t a_rows, hipStream_t stream);
+/* Gradient of vx_router_topk's weights with respect to the logits (the router of the reference's block is softmax ->
+ * top-k -> renormalise -> cast as differentiable tensor operations, modeling_qwen3_moe.py:128-134): idx = the
+ * selected experts [T, k] int64, d_weights [T, k] (bf16 or fp32), d_logits [T, E] in the logits' type. E <= 512,
+ * k <= 64. */
+int vx_router_topk_bwd(const void* logits, const int64_t* idx, const void* d_weights, void* d_logits, int64_t T, int E,
+                       int k, int64_t ld, int64_t ld_out, int logits_bf16, int weights_bf16, int renorm,
+                       hipStream_t stream);
 /* The elementwise step of the same backward between the products (fused_moe.py:150-250: silu, its derivative, the
  * routing-weight gradient), one launch, bf16 with a rounding wherever one of the reference's tensor operations
  * rounds. For sorted row r, w = rw[flat[r]]: hw = silu(g) u w; d_rw[flat[r]] = sum_i (silu(g) u)(d_hw);

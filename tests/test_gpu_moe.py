@@ -372,6 +372,25 @@ def test_wide_backward_products_give_the_bits_of_the_narrow_ones(T, k, E, N, K, 
         assert float(wide[E - 1].abs().max()) == 0.0, "an expert without rows gets zeros"
 
 
+@pytest.mark.parametrize("T,E,k,renorm,dtype", [(300, 128, 8, True, torch.bfloat16), (37, 60, 4, False, torch.float32),
+                                                 (5, 512, 64, True, torch.float32), (1, 8, 2, True, torch.bfloat16)])
+def test_router_backward_matches_autograd_of_the_tensor_operations(T, E, k, renorm, dtype):
+    # vx_router_topk_bwd against autograd through softmax -> gather (the kernel's selection) -> renormalise in fp32
+    gen = torch.Generator().manual_seed(T + E)
+    logits = (2.0 * torch.randn(T, E, generator=gen)).to(dtype).cuda()
+    w, sel = ops.router_topk(logits, k, renorm=renorm, out_dtype=torch.bfloat16, index_dtype=torch.int64)
+    d_w = torch.randn(T, k, generator=gen).to(torch.bfloat16).cuda()
+    got = ops.router_topk_backward(logits, sel, d_w, renorm)
+    ref = logits.float().clone().requires_grad_()
+    picked = torch.softmax(ref, -1).gather(-1, sel)
+    if renorm:
+        picked = picked / picked.sum(-1, keepdim=True)
+    picked.backward(d_w.float())
+    err, scale = (got.float() - ref.grad).abs(), float(ref.grad.abs().max())
+    tol = 1e-5 if dtype == torch.float32 else 2.0 ** -8
+    assert got.dtype == dtype and float(err.max()) <= tol * scale + 1e-9, f"router gradient: {float(err.max()):.4g} vs scale {scale:.4g}"
+
+
 @pytest.mark.parametrize("n,I,T,k", [(520, 64, 130, 4), (4096, 768, 512, 8), (7, 8, 7, 1)])
 def test_backward_elementwise_kernel_equals_the_tensor_operations(n, I, T, k):
     # vx_moe_swiglu_bwd against the bf16 tensor operations the reference's backward runs (fused_moe.py:150-250): every

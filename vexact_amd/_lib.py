@@ -60,6 +60,7 @@ PROTOTYPES = {
     "vx_rms_norm_bwd_workspace_bytes": (_L, [_L, _L]),
     "vx_rms_norm_bwd": (_I, [_P, _P, _P, _P, _P, _I, _L, _L, _L, _L, _L, _F, _I, _P, _L, _P]),
     "vx_logprobs_bwd": (_I, [_P, _P, _P, _P, _P, _I, _L, _L, _L, _L, _P]),
+    "vx_router_topk_bwd": (_I, [_P, _P, _P, _P, _L, _I, _I, _L, _L, _I, _I, _I, _P]),
     "vx_moe_swiglu_bwd": (_I, [_P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _L, _L, _L, _L, _L, _P]),
     "vx_moe_gemm_tn": (_I, [_P, _L, _P, _P, _L, _P, _P, _L, _L, _L, _L, _P, _L, _L, _L, _P]),
     "vx_expert_histogram": (_I, [_P, _I, _L, _I, _P, _P]),

@@ -722,6 +722,74 @@ __global__ __launch_bounds__(256) void moe_swiglu_bwd_kernel(const bf16_t* __res
   if (lane == 0) d_rw[f] = f32_to_bf16(part);
 }
 
+// ---------------------------------------------------------------------------------------
+// Gradient of the router (softmax over E logits in fp32 -> the k selected probabilities -> optional renormalisation
+// -> cast; the reference runs these as tensor operations, modeling_qwen3_moe.py:128-134) with respect to the logits:
+//   p = softmax(l), sel_i = p[idx_i], (renorm) s = sum sel, w_i = sel_i / s, d_sel_i = (d_w_i - sum_j d_w_j w_j) / s,
+//   d_l_j = p_j ((j == idx_i ? d_sel_i : 0) - sum_i d_sel_i sel_i).
+// One wavefront per token, E <= 512, k <= 64; every sum in a fixed lane order.
+// ---------------------------------------------------------------------------------------
+template <bool LB, bool WB>
+__global__ __launch_bounds__(256) void router_topk_bwd_kernel(const void* __restrict__ logits_, const int64_t* __restrict__ idx,
+                                                              const void* __restrict__ d_w_, void* __restrict__ d_logits_,
+                                                              int64_t T, int E, int k, int64_t ld, int64_t ldo, int renorm) {
+  __shared__ float ps[4][512], dp[4][512];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t t_ = (int64_t)blockIdx.x * 4 + wv;
+  const bool live = t_ < T;
+  const int64_t t = live ? t_ : T - 1;  // a wavefront past the end recomputes the last token and stores nothing
+  auto ldl = [&](int j) {
+    return LB ? bf16_to_f32(((const bf16_t*)logits_)[t * ld + j]) : ((const float*)logits_)[t * ld + j];
+  };
+  float l[8], m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int j = lane + 64 * i;
+    l[i] = j < E ? ldl(j) : -INFINITY;
+    m = fmaxf(m, l[i]);
+  }
+  m = wave_max(m);
+  float z = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    l[i] = lane + 64 * i < E ? expf(l[i] - m) : 0.f;
+    z += l[i];
+  }
+  z = wave_sum(z);
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int j = lane + 64 * i;
+    l[i] /= z;
+    if (j < E) { ps[wv][j] = l[i]; dp[wv][j] = 0.f; }
+  }
+  __syncthreads();
+  int my = -1;
+  float sel = 0.f, dw = 0.f;
+  if (lane < k) {
+    my = (int)idx[t * k + lane];
+    sel = ps[wv][my];
+    dw = WB ? bf16_to_f32(((const bf16_t*)d_w_)[t * k + lane]) : ((const float*)d_w_)[t * k + lane];
+  }
+  float d_sel = dw;
+  if (renorm) {
+    const float s = wave_sum(sel);
+    const float dot = wave_sum(dw * (sel / s));
+    d_sel = lane < k ? (dw - dot) / s : 0.f;
+  }
+  const float c = wave_sum(d_sel * sel);
+  if (lane < k) dp[wv][my] = d_sel;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int j = lane + 64 * i;
+    if (j < E && live) {
+      const float g = l[i] * (dp[wv][j] - c);
+      if (LB) ((bf16_t*)d_logits_)[t * ldo + j] = f32_to_bf16(g);
+      else ((float*)d_logits_)[t * ldo + j] = g;
+    }
+  }
+}
+
 static inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 }  // namespace vx
@@ -777,6 +845,24 @@ int vx_moe_gemm_nn(const void* a, int64_t lda, const int* a_src, const void* w, 
     return launch_status();
   }
   moe_gemm_nn_kernel<NN_ROWS><<<dim3((unsigned)((N + 127) / 128), (unsigned)max_tiles), 256, 0, stream>>>(p);
+  return launch_status();
+}
+
+int vx_router_topk_bwd(const void* logits, const int64_t* idx, const void* d_weights, void* d_logits, int64_t T, int E,
+                       int k, int64_t ld, int64_t ld_out, int logits_bf16, int weights_bf16, int renorm,
+                       hipStream_t stream) {
+  if (!logits || !idx || !d_weights || !d_logits || T < 0 || E <= 0 || k <= 0) return VX_ERR_ARG;
+  if (E > 512 || k > 64 || k > E) return VX_ERR_UNSUPPORTED;
+  if (T == 0) return VX_OK;
+  const int64_t blocks = (T + 3) / 4;
+  if (blocks > 0x7fffffffLL) return VX_ERR_ARG;
+#define VX_RB(LB, WB) \
+  router_topk_bwd_kernel<LB, WB><<<(unsigned)blocks, 256, 0, stream>>>(logits, idx, d_weights, d_logits, T, E, k, ld, ld_out, renorm)
+  if (logits_bf16 && weights_bf16) VX_RB(true, true);
+  else if (logits_bf16) VX_RB(true, false);
+  else if (weights_bf16) VX_RB(false, true);
+  else VX_RB(false, false);
+#undef VX_RB
   return launch_status();
 }
 

@@ -510,14 +510,25 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const typename Elem<D
   for (int j = threadIdx.x; j < n; j += 256) dw_part[(int64_t)blockIdx.x * n + j] = rb_red[j];
 }
 
+// 64 columns per workgroup; wavefront v of 8 adds the partial rows v, v + 8, ... in ascending order, then the eight sums
+// are added in wavefront order
 template <int DT>
-__global__ __launch_bounds__(256) void rms_norm_bwd_finish_kernel(const float* __restrict__ dw_part, int nblocks, int n,
+__global__ __launch_bounds__(512) void rms_norm_bwd_finish_kernel(const float* __restrict__ dw_part, int nblocks, int n,
                                                                   typename Elem<DT>::T* __restrict__ dw) {
-  const int j = blockIdx.x * 256 + threadIdx.x;
-  if (j >= n) return;
+  __shared__ float part[8][64];
+  const int lane = threadIdx.x & 63, v = threadIdx.x >> 6;
+  const int j = blockIdx.x * 64 + lane;
   float s = 0.f;
-  for (int b = 0; b < nblocks; b++) s += dw_part[(int64_t)b * n + j];
-  Elem<DT>::st(dw + j, s);
+  if (j < n)
+    for (int b = v; b < nblocks; b += 8) s += dw_part[(int64_t)b * n + j];
+  part[v][lane] = s;
+  __syncthreads();
+  if (v == 0 && j < n) {
+    float t = part[0][lane];
+#pragma unroll
+    for (int i = 1; i < 8; i++) t += part[i][lane];
+    Elem<DT>::st(dw + j, t);
+  }
 }
 
 // Gradient of out[i] = logits[i, label_i] - logsumexp(logits[i, :]) with respect to the logits, from the forward's
@@ -746,9 +757,9 @@ int vx_rms_norm_bwd(const void* x, const void* weight, const void* dy, void* dx,
   // no rows: the weight gradient is zero (no partial rows are read)
   const int nb = rows > 0 ? (int)blocks : 0;
   if (dtype == DT_BF16)
-    rms_norm_bwd_finish_kernel<DT_BF16><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const float*)workspace, nb, (int)n, (bf16_t*)dw);
+    rms_norm_bwd_finish_kernel<DT_BF16><<<(unsigned)((n + 63) / 64), 512, 0, stream>>>((const float*)workspace, nb, (int)n, (bf16_t*)dw);
   else
-    rms_norm_bwd_finish_kernel<DT_F16><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>((const float*)workspace, nb, (int)n, (_Float16*)dw);
+    rms_norm_bwd_finish_kernel<DT_F16><<<(unsigned)((n + 63) / 64), 512, 0, stream>>>((const float*)workspace, nb, (int)n, (_Float16*)dw);
   return launch_status();
 }
 

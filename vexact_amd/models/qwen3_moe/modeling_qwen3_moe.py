@@ -109,6 +109,8 @@ class RouterTopKFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_weights, _):
         router_logits, selected = ctx.saved_tensors
+        if router_logits.shape[-1] <= 512 and selected.shape[-1] <= 64 and router_logits.dtype in (torch.float32, torch.bfloat16):
+            return ops.router_topk_backward(router_logits, selected, d_weights, ctx.renorm), None, None, None
         p = torch.softmax(router_logits.float(), dim=-1)
         d_sel = d_weights.float()
         if ctx.renorm:

@@ -641,6 +641,25 @@ def router_topk(
     return w, idx
 
 
+def router_topk_backward(logits: torch.Tensor, selected: torch.Tensor, d_weights: torch.Tensor, renorm: bool = True) -> torch.Tensor:
+    """Gradient of ``router_topk(logits, k, renorm)[0]`` with respect to ``logits [T, E]`` (E <= 512, k <= 64)."""
+    _need_gpu("logits", logits)
+    T, E = logits.shape
+    k = selected.shape[1]
+    assert logits.dtype in (torch.float32, torch.bfloat16) and selected.dtype == torch.int64 and selected.shape == (T, k)
+    lg = logits if logits.stride(1) == 1 else logits.contiguous()
+    dw = d_weights if d_weights.dtype in (torch.float32, torch.bfloat16) else d_weights.float()
+    dw, sel = dw.contiguous(), selected.contiguous()
+    out = _empty((T, E), dtype=logits.dtype, device=logits.device)
+    _lib.check(
+        _lib.load().vx_router_topk_bwd(lg.data_ptr(), sel.data_ptr(), dw.data_ptr(), out.data_ptr(), T, E, k, lg.stride(0),
+                                       out.stride(0), int(lg.dtype == torch.bfloat16), int(dw.dtype == torch.bfloat16),
+                                       int(renorm), _stream()),
+        "vx_router_topk_bwd",
+    )
+    return out
+
+
 def moe_tile_rows(num_tokens: int, wide_ok: bool = True, packed_only: bool = False) -> int:
     """Rows per expert tile, chosen from the token count only (any choice gives the same bits).
     ``wide_ok``: both GEMM depths are multiples of 64, which the 256-row kernel needs.
