@@ -260,3 +260,15 @@ def test_dense_swiglu_equals_unfused_chain_and_is_row_invariant(N, K):
     down = torch.empty(256, N, dtype=torch.bfloat16, device="cuda").normal_(0, 0.03, generator=g)
     y = ops.swiglu_mlp(x, wg, wu, down)
     assert_bitwise(y, ops.gemm_nt(ref, down), "swiglu_mlp")
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 2048, 1000), (2048, 4096, 8192), (2560, 2560, 64), (4096, 2048, 8)])
+def test_weight_gradient_layout_gives_the_bits_of_the_transposed_copies(M, N, K):
+    # matmul(d_y.t(), x): both operands with the contraction index slow go to the grouped weight-gradient kernel as
+    # they lie; the same product through transposed copies and the NT kernels must give the same bits
+    g = torch.Generator().manual_seed(M + K)
+    dy = torch.randn(K, M, generator=g).to(torch.bfloat16).cuda()
+    x = torch.randn(K, N, generator=g).to(torch.bfloat16).cuda()
+    direct = ops.matmul(dy.t(), x)
+    copies = ops.gemm_nt(dy.t().contiguous(), x.t().contiguous())
+    assert_bitwise(direct, copies, "d_y^T x: grouped kernel vs transposed copies")

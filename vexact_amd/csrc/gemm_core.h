@@ -135,7 +135,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
 #pragma unroll
       for (int u = 0; u < U; u++) {
         const bool ok = kstep0 + 32 * u + 8 * g < K;
-        const int ko = ok ? kstep0 + 32 * u : 0;
+        // a piece past K is never dereferenced: the row's first piece is read instead (wp already points 8 g in)
+        const int ko = ok ? kstep0 + 32 * u : -8 * g;
         wa[u] = ldg16(wp + ko, ok);
         if constexpr (EPI == EPI_SWIGLU) wb[u] = ldg16(wp2 + ko, ok);
       }
@@ -318,7 +319,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(GemmParams p) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const int c8 = (tid + 256 * j) & 7;
-      const int ko = (k0 + c8 * 8 < K) ? k0 : 0;
+      // a piece past K is never dereferenced: the row's first piece is read instead (the row pointers already
+      // point 8 c8 in), since with K < 64 even k0 = 0 would reach past the row, and past the tensor in its last rows
+      const int ko = (k0 + c8 * 8 < K) ? k0 : -8 * c8;
       gx[j] = ldg16_raw(xrow[j] + ko);
       gw[j] = ldg16_raw(wrow[j] + ko);
     }

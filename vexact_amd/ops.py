@@ -360,6 +360,21 @@ def swiglu_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down
     return gemm_nt(gemm_swiglu(x, w_gate, w_up), w_down)
 
 
+_ROW_SPANS: dict = {}
+
+
+def _row_span(rows: int, device) -> torch.Tensor:
+    """``[0, rows]`` as an int32 device tensor (the row offsets of a single group), made once per size."""
+    key = (int(rows), str(device))
+    t = _ROW_SPANS.get(key)
+    if t is None:
+        if len(_ROW_SPANS) > 256:
+            _ROW_SPANS.clear()
+        t = torch.tensor([0, int(rows)], dtype=torch.int32, device=device)
+        _ROW_SPANS[key] = t
+    return t
+
+
 def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``a[M,K] @ b[K,N] (+ bias[N])`` with the dtype of ``a``; any strides.
 
@@ -388,6 +403,14 @@ def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None
             c += bias
         return c
     lib = _lib.load()
+    if (a.dtype == torch.bfloat16 and bias is None and a.stride(0) == 1 and b.stride(1) == 1 and M % 8 == 0 and N % 8 == 0
+            and a.stride(1) % 8 == 0 and b.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0
+            and ((M + 255) // 256) * ((N + 255) // 256) >= 96 and not torch.cuda.is_current_stream_capturing()):
+        # a is the transposed view of a row-major [K, M] tensor and b is row-major [K, N] (a linear layer's weight
+        # gradient, d_y^T x): the contraction index is the slow index of both, which the grouped weight-gradient
+        # kernel reads as it lies (one group holding every row) instead of two transposed copies; same MFMA chain per
+        # output element as the other kernels. Only with enough 256 x 256 output tiles to occupy the chip.
+        return moe_gemm_tn(a.t(), b, _row_span(K, a.device), 1, out=c.view(1, M, N)).view(M, N)
     if a.dtype == torch.bfloat16 and K % 8 == 0:
         w_nk = b.t()  # [N, K] view
         x = a
