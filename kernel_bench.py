@@ -7,7 +7,7 @@ out, and the replay is timed with events. Prints time, algorithmic bytes (or flo
 fraction of the MI355X peak. ``--nograph`` launches eagerly once and times nothing: that is the form
 to run under ``rocprofv3 --pmc``.
 
-    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,other,configs,mfma,copy,dropin
+    python kernel_bench.py --what moe,attn,gemm,small,prefill,dense,train,sampler,other,configs,mfma,copy,dropin,trainlayer
 """
 
 from __future__ import annotations
@@ -412,6 +412,8 @@ def run(a, quiet: bool = False) -> list:
                 report(f"{nm} gemm M={M} N=4096 K=4096", timeit(lambda li: ops.matmul(xx, ww.t()), n_layers=2), flops=2 * M * 4096 * 4096)
     if "dropin" in what:
         results.extend(dropin_decode(a, quiet))
+    if "trainlayer" in what:
+        results.extend(dropin_train_layers(quiet))
     if "copy" in what:
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()
@@ -509,6 +511,97 @@ def dropin_decode(a, quiet: bool = False) -> list:
         ms = e0.elapsed_time(e1) / 10
         say(f"HF Qwen3MoeForCausalLM drop-in decode, batch {B}, {how}: {ms:.2f} ms/step = {B / ms * 1e3:.0f} tok/s", flush=True)
         res.append({"name": f"HF drop-in decode step, batch {B}, {how}", "us": round(ms * 1e3, 1), "tok_s": round(B / ms * 1e3)})
+    return res
+
+
+def dropin_train_layers(quiet: bool = False, layers: int = 2, seqs: int = 8, seq_len: int = 1024) -> list:
+    """The trainer's side of the drop-in: ``layers`` HuggingFace ``Qwen3MoeDecoderLayer``s of the 30B-A3B shape under
+    the patches, batch-invariant mode and a packed (cache-less) context, forward + backward over ``seqs`` sequences of
+    ``seq_len`` tokens; and the paged prefill of the same tokens in inference mode for comparison."""
+    import types
+
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+    from transformers.models.qwen3_moe.configuration_qwen3_moe import Qwen3MoeConfig
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import Qwen3MoeForCausalLM
+
+    from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
+    from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches
+
+    say = (lambda *x, **k: None) if quiet else print
+    cfg = Qwen3MoeConfig(vocab_size=32000, hidden_size=2048, intermediate_size=6144, num_hidden_layers=layers,
+                         num_attention_heads=32, num_key_value_heads=4, head_dim=128, num_experts=128, num_experts_per_tok=8,
+                         moe_intermediate_size=768, norm_topk_prob=True, max_position_embeddings=40960, rms_norm_eps=1e-6,
+                         rope_parameters={"rope_type": "default", "rope_theta": 1.0e6})
+    cfg._attn_implementation = "triton-invariant"
+    ALL_ATTENTION_FUNCTIONS["triton-invariant"] = flash_attention_forward
+    apply_qwen3_moe_patches()
+    with torch.device("meta"):
+        model = Qwen3MoeForCausalLM(cfg)
+    model = model.to_empty(device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(5)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if "norm" in name:
+                p.fill_(1.0)
+            else:
+                p.normal_(0.0, 0.02, generator=g)
+    for p in model.parameters():
+        p.data = p.data.to(torch.bfloat16)
+    rot = model.model.rotary_emb
+    inv = 1.0 / (1.0e6 ** (torch.arange(0, 128, 2, device="cuda").float() / 128))
+    rot.inv_freq, rot.original_inv_freq = inv, inv.clone()
+    T, page = seqs * seq_len, 16
+    i32 = dict(dtype=torch.int32, device="cuda")
+    ctx, qsl = torch.full((seqs,), seq_len, **i32), torch.arange(0, T + 1, seq_len, **i32)
+    pos = torch.arange(seq_len, device="cuda").repeat(seqs)[None]
+    x0 = torch.randn(1, T, 2048, device="cuda", generator=g).to(torch.bfloat16)
+    dy = torch.randn(1, T, 2048, device="cuda", generator=g).to(torch.bfloat16)
+
+    def through_layers(x):
+        pe = rot(x, pos)
+        for layer in model.model.layers:
+            x = layer(x, position_ids=pos, position_embeddings=pe)
+        return x
+
+    def train_step():
+        for p in model.parameters():
+            p.grad = None
+        through_layers(x0.clone().requires_grad_()).backward(dy)
+
+    def timed(fn, reps=5):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    res = []
+    set_kv_cache_context(is_paged_attn=False, context_lens=ctx, query_start_loc=qsl, max_seqlen_q=seq_len)
+    try:
+        with set_batch_invariant_mode(True):
+            ms = timed(train_step)
+    finally:
+        clear_kv_cache_context()
+    say(f"HF decoder layer, trainer forward + backward, {seqs} x {seq_len} packed tokens: {ms / layers:.2f} ms per layer", flush=True)
+    res.append({"name": f"HF decoder layer forward + backward, {seqs} x {seq_len} tokens", "us": round(ms / layers * 1e3, 1)})
+    pages = seq_len // page
+    store = KVCacheStore(cfg, types.SimpleNamespace(page_size=page, max_cache_blocks=seqs * pages + 4), torch.device("cuda"))
+    set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache,
+                         block_tables=torch.arange(seqs * pages, **i32).reshape(seqs, pages), context_lens=ctx,
+                         slot_mapping=torch.arange(T, **i32), query_start_loc=qsl, max_seqlen_q=seq_len)
+    try:
+        with torch.inference_mode(), set_batch_invariant_mode(True):
+            ms = timed(lambda: through_layers(x0))
+    finally:
+        clear_kv_cache_context()
+    say(f"HF decoder layer, paged prefill of the same tokens (inference mode): {ms / layers:.2f} ms per layer", flush=True)
+    res.append({"name": f"HF decoder layer paged prefill, {seqs} x {seq_len} tokens", "us": round(ms / layers * 1e3, 1)})
     return res
 
 
