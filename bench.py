@@ -444,11 +444,12 @@ def main():
 def other_configs():
     """The reference's other benchmark configurations at their own shapes, graph-replayed and timed with HIP
     events (kernel_bench.py): C1 op chain at M = 1 / 7 / 64, C2 decode attention, C3 chunked prefill attention,
-    C4 fused MoE block at T = 1 / 64 / 256 / 4096, and the q/k/v projection of an 8192-token prefill chunk.
+    C4 fused MoE block at T = 1 / 64 / 256 / 4096, the q/k/v projection of an 8192-token prefill chunk, and the
+    training side's kernels (packed attention forward / backward, the MoE backward products at 8192 tokens).
     Each line carries its algorithmic bytes or flops and the fraction of the HBM / bf16 MFMA peak."""
     import kernel_bench
 
-    res = kernel_bench.run(kernel_bench.parse(["--what", "configs,mfma", "--batch", "256", "--layers", "2", "--reps", "3"]),
+    res = kernel_bench.run(kernel_bench.parse(["--what", "configs,mfma,train", "--batch", "256", "--layers", "2", "--reps", "3"]),
                            quiet=True)
     mfma = [r for r in res if r["bound"] == "mfma"]
     return res, mfma
