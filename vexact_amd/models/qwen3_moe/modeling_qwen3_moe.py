@@ -345,11 +345,22 @@ def fused_attention_forward(self, hidden_states, position_embeddings, attention_
     ops.qk_norm_rope_store(qkv, self.q_norm.weight, self.k_norm.weight, cos[0], sin[0], None, ctx.slot_mapping, q,
                            ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx], Hq, Hkv, D,
                            self.q_norm.variance_epsilon)
-    out, _ = flash_attn_varlen_func(
-        q, ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx], cu_seqlens_q=ctx.query_start_loc,
-        max_seqlen_q=ctx.max_seqlen_q, seqused_k=ctx.context_lens, page_table=ctx.block_tables, dropout_p=0.0,
-        softmax_scale=self.scaling, causal=True)
-    return self.o_proj(out.reshape(1, T, Hq * D)), None
+    # The kernel writes every row that belongs to a sequence with at least one key; what it leaves alone here are the
+    # padding rows of a captured bucket, whose values nobody reads, so the output skips the NaN fill that
+    # torch.empty adds under deterministic algorithms (one more launch per layer).
+    k_cache, v_cache = ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx]
+    if not (ctx.query_start_loc.dtype == ctx.context_lens.dtype == ctx.block_tables.dtype == torch.int32
+            and ctx.query_start_loc.is_contiguous() and ctx.context_lens.is_contiguous() and ctx.block_tables.stride(-1) == 1
+            and ctx.query_start_loc.is_cuda and ctx.context_lens.is_cuda and ctx.block_tables.is_cuda
+            and k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.dtype == v_cache.dtype == torch.bfloat16):
+        out, _ = flash_attn_varlen_func(
+            q, k_cache, v_cache, cu_seqlens_q=ctx.query_start_loc, max_seqlen_q=ctx.max_seqlen_q,
+            seqused_k=ctx.context_lens, page_table=ctx.block_tables, dropout_p=0.0, softmax_scale=self.scaling, causal=True)
+    else:
+        out = ops.paged_attention(q, k_cache, v_cache, ctx.query_start_loc, ctx.context_lens, ctx.block_tables,
+                                  float(self.scaling), max_seqlen_q=int(ctx.max_seqlen_q or 0),
+                                  out=ops._empty((T, Hq, v_cache.shape[-1]), dtype=torch.bfloat16, device=x.device))
+    return self.o_proj(out.reshape(1, T, -1)), None
 
 
 _ORIGINAL_LAYER = None  # Qwen3MoeDecoderLayer.forward while the fused form is patched in
