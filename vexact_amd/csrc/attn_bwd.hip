@@ -380,7 +380,8 @@ __global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwd
   const int k0 = p.cu_k[seq], kv_len = p.cu_k[seq + 1] - k0;
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int i_base = blockIdx.x * (16 * BWL_WAVES);
+  // the query tile is rotated by head and sequence for the reason given at the key tiles of the dK / dV kernel
+  const int i_base = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x) * (16 * BWL_WAVES);
   if (i_base >= qlen || kv_len <= 0) return;  // uniform over the block
   const int kvh = h / (p.Hq / p.Hkv);
   const int shift = kv_len - qlen;
@@ -481,7 +482,10 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
   const int k0 = p.cu_k[seq], kv_len = p.cu_k[seq + 1] - k0;
   const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int j_base = blockIdx.x * (16 * NW);
+  // Workgroup ids go round the 8 XCDs, so with 8 (or 16, ...) key tiles per sequence the tile number would pick the
+  // XCD: the tiles that see every query on one, those that see a few on another. Rotating the tile number by the head
+  // and the sequence spreads every kind over all of them (which workgroup computes a tile changes no result).
+  const int j_base = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x) * (16 * NW);
   if (j_base >= kv_len) return;  // uniform over the block
   const int G = p.Hq / p.Hkv;
   const int shift = kv_len - qlen;

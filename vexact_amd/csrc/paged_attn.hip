@@ -70,8 +70,11 @@ struct AttnParams {
 // items and there are total_q / rpb + num_seqs in all. Returns false when there is nothing to do.
 __device__ __forceinline__ bool locate_row_block(const AttnParams& p, int rpb, int& seq, int& bx) {
   if (!p.compact) {
+    // Workgroup ids go round the 8 XCDs, so with a multiple of 8 row blocks per sequence blockIdx.x would pick the
+    // XCD, and under a causal mask the row blocks that see the most keys would all run on the same ones: the row
+    // block is blockIdx.x rotated by head group and sequence (which workgroup computes a block changes no result).
     seq = blockIdx.z;
-    bx = blockIdx.x;
+    bx = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
     return true;
   }
   const int w = blockIdx.x;
