@@ -59,24 +59,29 @@ struct AttnParams {
   float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernels)
   // General launches over batches whose sequences differ in their number of query rows:
   int compact;      // != 0: blockIdx.x numbers (sequence, row block) pairs compactly, see locate_row_block
+  int grid_heads, grid_sg;  // plain form: head groups and sequences per group of sequences in blockIdx.x
   int single_mode;  // 0: every sequence; 1: only sequences with one query row (decode kernels inside a general
                     // launch); 2: all others (the general kernel beside them)
 };
 
-// Which sequence and which of its row blocks (rpb query rows each) a workgroup of a general kernel works on.
-// Plain form: blockIdx.z and blockIdx.x, a grid of ceil(max_q / rpb) x num_seqs, most of it empty when one long
-// chunk shares a batch with decode tokens. Compact form: item w = blockIdx.x belongs to the last sequence s with
-// cu_q[s] / rpb + s <= w, as its row block w - (cu_q[s] / rpb + s); every sequence owns at least ceil(qlen / rpb)
-// items and there are total_q / rpb + num_seqs in all. Returns false when there is nothing to do.
-__device__ __forceinline__ bool locate_row_block(const AttnParams& p, int rpb, int& seq, int& bx) {
+// Which sequence, which of its row blocks (rpb query rows each) and which group of heads a workgroup of a general
+// kernel works on. Plain form: a grid of (head groups x grid_sg sequences) x ceil(max_q / rpb) x groups of sequences,
+// most of it empty when one long chunk shares a batch with decode tokens. Workgroup ids go round the eight XCDs and
+// are dispatched in order, so the fastest index holds what has equal work (the head groups of a few sequences, eight
+// ids in all) and the row block comes next, running downwards: under a causal mask a sequence's blocks that see the
+// most keys start first and its short ones fill the tail. (With the row block as the fastest index, a multiple of 8
+// blocks per sequence pinned every block height to one XCD and long blocks started last.) Compact form (blockIdx.y =
+// head group): item w = blockIdx.x belongs to the last sequence s with cu_q[s] / rpb + s <= w, as its row block
+// w - (cu_q[s] / rpb + s); every sequence owns at least ceil(qlen / rpb) items and there are total_q / rpb + num_seqs
+// in all. Returns false when there is nothing to do.
+__device__ __forceinline__ bool locate_row_block(const AttnParams& p, int rpb, int& seq, int& bx, int& hg) {
   if (!p.compact) {
-    // Workgroup ids go round the 8 XCDs, so with a multiple of 8 row blocks per sequence blockIdx.x would pick the
-    // XCD, and under a causal mask the row blocks that see the most keys would all run on the same ones: the row
-    // block is blockIdx.x rotated by head group and sequence (which workgroup computes a block changes no result).
-    seq = blockIdx.z;
-    bx = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
-    return true;
+    hg = (int)(blockIdx.x % p.grid_heads);
+    bx = (int)(gridDim.y - 1 - blockIdx.y);
+    seq = (int)(blockIdx.z * p.grid_sg + blockIdx.x / p.grid_heads);
+    return seq < p.num_seqs;
   }
+  hg = blockIdx.y;
   const int w = blockIdx.x;
   int lo = 0, hi = p.num_seqs - 1;
   while (lo < hi) {  // cu_q[s] / rpb + s is strictly increasing in s
@@ -664,8 +669,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw
   // hpw > 1 the wavefronts of a block walk the same keys at the same time, so K and V mostly come
   // from the CU's L1 after the first wavefront has fetched them.
   const int rows_per_block = 16 * (4 * QT / hpw);
-  int seq, bx;
-  if (!locate_row_block(p, rows_per_block, seq, bx)) return;
+  int seq, bx, hg;
+  if (!locate_row_block(p, rows_per_block, seq, bx, hg)) return;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   if (p.single_mode == 2 && qlen == 1) return;  // a decode kernel of the same launch takes these
@@ -678,7 +683,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p, int hpw
 #pragma unroll
   for (int t = 0; t < QT; t++) {
     const int s = wave * QT + t;
-    head_of[t] = blockIdx.y * hpw + s % hpw;
+    head_of[t] = hg * hpw + s % hpw;
     i0_of[t] = bx * rows_per_block + 16 * (s / hpw);
     any = any || i0_of[t] < qlen;
   }
@@ -788,8 +793,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
   extern __shared__ __attribute__((aligned(1024))) uint8_t pf_lds[];
 
   const int rows_per_block = 16 * (PFL_SLOTS / hpw);
-  int seq, bx;
-  if (!locate_row_block(p, rows_per_block, seq, bx)) return;
+  int seq, bx, hg;
+  if (!locate_row_block(p, rows_per_block, seq, bx, hg)) return;
   const int q0 = p.cu_q[seq];
   const int qlen = p.cu_q[seq + 1] - q0;
   if (p.single_mode == 2 && qlen == 1) return;  // a decode kernel of the same launch takes these
@@ -807,7 +812,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
     for (int e = threadIdx.x; e < rows_per_block * hpw * (D / 8); e += 64 * PFL_WAVES) {
       const int row = i_base + e / (hpw * (D / 8)), rem = e % (hpw * (D / 8));
       if (row < qlen)
-        *(uint4*)(p.o + (int64_t)(q0 + row) * p.sot + (int64_t)(blockIdx.y * hpw + rem / (D / 8)) * p.soh +
+        *(uint4*)(p.o + (int64_t)(q0 + row) * p.sot + (int64_t)(hg * hpw + rem / (D / 8)) * p.soh +
                   8 * (rem % (D / 8))) = make_uint4(0, 0, 0, 0);
     }
     return;
@@ -817,10 +822,10 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
 #pragma unroll
   for (int t = 0; t < QT; t++) {
     const int s = wave * QT + t;
-    head_of[t] = blockIdx.y * hpw + s % hpw;
+    head_of[t] = hg * hpw + s % hpw;
     i0_of[t] = i_base + 16 * (s / hpw);
   }
-  const int kvh = (blockIdx.y * hpw) / (p.Hq / p.Hkv);
+  const int kvh = (hg * hpw) / (p.Hq / p.Hkv);
 
   // ---- this wavefront's query tiles go to its own LDS region (read back every block, which frees
   // 32 registers); piece c of row r at piece c ^ r, like the key rows
@@ -1216,10 +1221,17 @@ static int launch_attn(const AttnParams& p_in, int mode, int max_q, int total_q,
     // (sequence, row block) pairs: the plain grid of ceil(rows / rpb) x num_seqs, or the compact numbering when
     // that is smaller (sequences with very different numbers of query rows)
     auto row_grid = [&](int rb, unsigned heads) {
-      const int64_t plain = (int64_t)((rows + rb - 1) / rb) * p.num_seqs;
+      const int64_t blocks = (rows + rb - 1) / rb;
+      const int64_t plain = blocks * p.num_seqs;
       const int64_t comp = (int64_t)total_q / rb + p.num_seqs;
-      p.compact = comp < plain ? 1 : 0;
-      return p.compact ? dim3((unsigned)comp, heads, 1) : dim3((unsigned)((rows + rb - 1) / rb), heads, (unsigned)p.num_seqs);
+      p.compact = (comp < plain || blocks > 65535 || p.num_seqs > 65535) ? 1 : 0;  // grid.y and grid.z end at 65535
+      if (p.compact) return dim3((unsigned)comp, heads, 1);
+      // eight consecutive workgroup ids = the head groups of 8 / heads sequences at one row block (measured on 4 head
+      // groups: 1 / 2 / 4 / 8 sequences give 135 / 115 / 111 / 111 us on 8 x 1024-token prompts and 555 / 554 / 622 /
+      // 868 us on 512-token chunks behind prefixes up to 8192, where more sequences in flight share less of the L2)
+      p.grid_heads = (int)heads;
+      p.grid_sg = std::max(1, std::min(p.num_seqs, (int)(8u / std::max(1u, heads))));
+      return dim3(heads * (unsigned)p.grid_sg, (unsigned)blocks, (unsigned)((p.num_seqs + p.grid_sg - 1) / p.grid_sg));
     };
     dim3 grid = row_grid(rpb, (unsigned)(p.Hq / hpw));
     if constexpr (DK == 128 && DV == 128) {
