@@ -58,7 +58,7 @@ struct AttnParams {
   const int* seq_order;  // optional [B]: decode kernels take sequence seq_order[i] as their i-th (longest first balances the tail)
   float* lse;  // optional [T, Hq]: natural-log sum of exp(scale * s) over a row's visible keys (general kernels)
   // General launches over batches whose sequences differ in their number of query rows:
-  int compact;      // != 0: blockIdx.x numbers (sequence, row block) pairs compactly, see locate_row_block
+  int compact;      // != 0: (sequence, row block) pairs are numbered compactly, see locate_row_block
   int grid_heads, grid_sg;  // plain form: head groups and sequences per group of sequences in blockIdx.x
   int single_mode;  // 0: every sequence; 1: only sequences with one query row (decode kernels inside a general
                     // launch); 2: all others (the general kernel beside them)
@@ -70,8 +70,8 @@ struct AttnParams {
 // are dispatched in order, so the fastest index holds what has equal work (the head groups of a few sequences, eight
 // ids in all) and the row block comes next, running downwards: under a causal mask a sequence's blocks that see the
 // most keys start first and its short ones fill the tail. (With the row block as the fastest index, a multiple of 8
-// blocks per sequence pinned every block height to one XCD and long blocks started last.) Compact form (blockIdx.y =
-// head group): item w = blockIdx.x belongs to the last sequence s with cu_q[s] / rpb + s <= w, as its row block
+// blocks per sequence pinned every block height to one XCD and long blocks started last.) Compact form: item w
+// (see below for where it comes from) belongs to the last sequence s with cu_q[s] / rpb + s <= w, as its row block
 // w - (cu_q[s] / rpb + s); every sequence owns at least ceil(qlen / rpb) items and there are total_q / rpb + num_seqs
 // in all. Returns false when there is nothing to do.
 __device__ __forceinline__ bool locate_row_block(const AttnParams& p, int rpb, int& seq, int& bx, int& hg) {
@@ -81,8 +81,10 @@ __device__ __forceinline__ bool locate_row_block(const AttnParams& p, int rpb, i
     seq = (int)(blockIdx.z * p.grid_sg + blockIdx.x / p.grid_heads);
     return seq < p.num_seqs;
   }
-  hg = blockIdx.y;
-  const int w = blockIdx.x;
+  // compact == 1: head group fastest, items downwards (a sequence's last row blocks, which see the most keys, first);
+  // compact == 2 (more items than blockIdx.y can count): items in blockIdx.x, upwards
+  hg = p.compact == 1 ? blockIdx.x : blockIdx.y;
+  const int w = p.compact == 1 ? (int)(gridDim.y - 1 - blockIdx.y) : (int)blockIdx.x;
   int lo = 0, hi = p.num_seqs - 1;
   while (lo < hi) {  // cu_q[s] / rpb + s is strictly increasing in s
     const int mid = (lo + hi + 1) >> 1;
@@ -1225,7 +1227,11 @@ static int launch_attn(const AttnParams& p_in, int mode, int max_q, int total_q,
       const int64_t plain = blocks * p.num_seqs;
       const int64_t comp = (int64_t)total_q / rb + p.num_seqs;
       p.compact = (comp < plain || blocks > 65535 || p.num_seqs > 65535) ? 1 : 0;  // grid.y and grid.z end at 65535
-      if (p.compact) return dim3((unsigned)comp, heads, 1);
+      if (p.compact && comp <= 65535) return dim3(heads, (unsigned)comp, 1);
+      if (p.compact) {
+        p.compact = 2;
+        return dim3((unsigned)comp, heads, 1);
+      }
       // eight consecutive workgroup ids = the head groups of 8 / heads sequences at one row block (measured on 4 head
       // groups: 1 / 2 / 4 / 8 sequences give 135 / 115 / 111 / 111 us on 8 x 1024-token prompts and 555 / 554 / 622 /
       // 868 us on 512-token chunks behind prefixes up to 8192, where more sequences in flight share less of the L2)
