@@ -198,9 +198,10 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
  * lse [total_q, Hq] fp32 (modes 1 and 2): each query row's log-sum-exp (m + log2 l) ln 2, as the
  * reference's packed forward saves it (_varlen_attn_fwd_block_kernel,
  * triton_invariant_attention.py:187-191); +inf for a row without a visible key.
- * seq_order [num_seqs] int32 (decode modes 0, 3, 4): a permutation of the sequences; workgroup i of
- * the decode kernels takes sequence seq_order[i]. Longest context first shortens the tail of a batch
- * with mixed lengths; the results do not depend on it. (No counterpart in the reference.) */
+ * seq_order [num_seqs] int32 (paged modes 0, 1, 3, 4): a permutation of the sequences; workgroup i of
+ * the decode kernels takes sequence seq_order[i] (in mode 1: of the decode kernel that takes the sequences
+ * of one query row). Longest context first shortens the tail of a batch with mixed lengths; the results do
+ * not depend on it. (No counterpart in the reference.) */
 int vx_attention_ex(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
                     const int* cu_seqlens_q, const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
                     int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,

@@ -108,6 +108,14 @@ def test_general_launch_over_prefill_chunks_and_decode_tokens(qh, kh, d):
     for i, a in enumerate(q):
         assert_bitwise(dec[i : i + 1], out[off + a.shape[0] - 1 : off + a.shape[0]], "last chunk row vs decode step")
         off += a.shape[0]
+    # a sequence order (longest context first) for the decode kernel inside the general launch changes nothing
+    from vexact_amd import ops
+    k_cache, v_cache, table = OA.make_paged_kv_cache(k, v, page)
+    order = torch.argsort(torch.tensor(kv_lens), descending=True, stable=True).to(torch.int32).cuda()
+    ordered = ops.paged_attention(torch.cat(q, dim=0).cuda(), k_cache.cuda(), v_cache.cuda(), _cu(q_lens).cuda(),
+                                  torch.tensor(kv_lens, dtype=torch.int32).cuda(), table.cuda(), d**-0.5, max(q_lens),
+                                  seq_order=order)
+    assert_bitwise(ordered, out, "general launch with a sequence order")
 
 
 def test_page_table_aliases_match():

@@ -1142,8 +1142,7 @@ static int launch_attn(const AttnParams& p_in, int mode, int max_q, int total_q,
   const bool hybrid = mode == 1 && !p.lse && max_q != 1 && decode_form(4, p.num_seqs, p.Hq, p.Hkv, DV) == 1;
   if (hybrid) {
     AttnParams d = p;
-    d.single_mode = 1;
-    d.seq_order = nullptr;
+    d.single_mode = 1;  // seq_order, if given, orders these decode workgroups
     const int64_t max_kv = p.max_kv;
     d.max_chunks = (int)((max_kv + ATT_CHUNK - 1) / ATT_CHUNK);
     const int rc = launch_attn<DK, DV>(d, 4, 1, total_q, stream);
@@ -1326,8 +1325,9 @@ int vx_attention(const void* q, const void* k, const void* v, void* out, const i
 }
 
 // vx_attention with two optional extras: lse [total_q, Hq] fp32 (natural log; modes 1 and 2 only) receives
-// the rows' log-sum-exp, which the backward needs; seq_order [num_seqs] (decode modes) is a permutation
-// of the sequences in which the decode kernels take them, e.g. longest context first.
+// the rows' log-sum-exp, which the backward needs; seq_order [num_seqs] (paged modes) is a permutation
+// of the sequences in which the decode kernels take them, e.g. longest context first (in a general launch it
+// orders the decode kernel that takes the sequences of one query row).
 int vx_attention_ex(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
                     const int* cu_seqlens_q,
                      const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
@@ -1338,7 +1338,7 @@ int vx_attention_ex(const void* q, const void* k, const void* v, void* out, floa
                      int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (!q || !k || !v || !out || !cu_seqlens_q) return VX_ERR_ARG;
   if (lse && mode != 1 && mode != 2) return VX_ERR_UNSUPPORTED;
-  if (seq_order && (mode == 1 || mode == 2)) return VX_ERR_UNSUPPORTED;
+  if (seq_order && mode == 2) return VX_ERR_UNSUPPORTED;
   if (total_q < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return VX_ERR_ARG;
   if (mode < 0 || mode > 4) return VX_ERR_ARG;
   if (mode != 2 && (!seqused_k || !block_table || page_size <= 0 || max_pages <= 0)) return VX_ERR_ARG;

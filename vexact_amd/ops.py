@@ -531,8 +531,9 @@ def paged_attention(
     value the general kernel (identical bits per row). ``decode_kernel`` forces one of the two decode
     forms ("split": one wavefront per 256-key chunk plus a combine launch, "fused": chunks folded
     inside one workgroup per (sequence, kv head)); "auto" picks by batch size. Same bits either way.
-    ``seq_order`` (int32 permutation of the sequences, decode only) is the order in which the decode
-    workgroups take the sequences; longest first shortens the tail of a batch of mixed lengths."""
+    ``seq_order`` (int32 permutation of the sequences) is the order in which the decode workgroups take the
+    sequences (in a general launch: those of the decode kernel that takes the sequences of one query row);
+    longest first shortens the tail of a batch of mixed lengths."""
     T, Hq, Dk = q.shape
     Hkv, Dv = k_cache.shape[2], v_cache.shape[-1]
     o = out if out is not None else torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
@@ -552,9 +553,8 @@ def paged_attention(
         need = lib.vx_paged_attn_decode_workspace_needed(B, Hq, Hkv, Dv, max_pages * page, mode)
         if need > 0:
             ws = workspace if workspace is not None and workspace.numel() * workspace.element_size() >= need else _workspace(need, q.device)
-    if seq_order is not None and (mode == 1 or seq_order.dtype != torch.int32 or seq_order.numel() != B
-                                  or not seq_order.is_contiguous()):
-        raise ValueError("seq_order must be a contiguous int32 permutation of the sequences, for decode steps only")
+    if seq_order is not None and (seq_order.dtype != torch.int32 or seq_order.numel() != B or not seq_order.is_contiguous()):
+        raise ValueError("seq_order must be a contiguous int32 permutation of the sequences")
     _lib.check(
         lib.vx_attention_ex(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr(), None, _ptr(seq_order),
