@@ -475,7 +475,7 @@ __global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwd
 // 64 rows' lse and delta per stage.
 constexpr int BWK_STAGE = 2 * BWL_ARR + 1024;  // Q, dO, then 64 lse and 64 delta values
 constexpr int BWK_LDS = 2 * BWK_STAGE;
-constexpr int BWK_WAVES = 8;  // 128 keys per workgroup (64-key workgroups measured slower: 470 vs 404 us on 8 x 1024 tokens)
+constexpr int BWK_WAVES = 8;  // 128 keys per workgroup (64-key workgroups: 519 vs 493 us on 8 x 1024 tokens, 5 % ahead on 32 x 1024 and 16 x 2048, 3 % behind on 4 x 4096)
 
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams p) {
