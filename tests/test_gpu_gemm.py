@@ -272,3 +272,15 @@ def test_weight_gradient_layout_gives_the_bits_of_the_transposed_copies(M, N, K)
     direct = ops.matmul(dy.t(), x)
     copies = ops.gemm_nt(dy.t().contiguous(), x.t().contiguous())
     assert_bitwise(direct, copies, "d_y^T x: grouped kernel vs transposed copies")
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 2048, 4096), (1024, 520, 64), (1500, 2048, 512)])
+def test_data_gradient_layout_gives_the_bits_of_the_transposed_copy(M, N, K):
+    # matmul(d_y, w) with w row-major [K, N]: the grouped data-gradient kernel with one group, against the NT kernels
+    # on a transposed copy of w; rows alone give the same bits (the choice of kernel by M changes nothing)
+    g = torch.Generator().manual_seed(M + N)
+    dy = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(K, N, generator=g) * 0.05).to(torch.bfloat16).cuda()
+    direct = ops.matmul(dy, w)
+    assert_bitwise(direct, ops.gemm_nt(dy, w.t().contiguous()), "d_y w: grouped kernel vs transposed copy")
+    assert_bitwise(ops.matmul(dy[300:337].contiguous(), w), direct[300:337], "rows 300..336 alone")

@@ -375,13 +375,37 @@ def _row_span(rows: int, device) -> torch.Tensor:
     return t
 
 
+_ONE_GROUP_TILES: dict = {}
+
+
+def _one_group_tiles(rows: int, device):
+    """The 256-row tile table of a single group holding ``rows`` rows, in the form ``moe_gemm_nn`` reads (made
+    once per size)."""
+    from types import SimpleNamespace
+
+    key = (int(rows), str(device))
+    r = _ONE_GROUP_TILES.get(key)
+    if r is None:
+        if len(_ONE_GROUP_TILES) > 64:
+            _ONE_GROUP_TILES.clear()
+        n = (rows + 255) // 256
+        row0 = torch.arange(0, n * 256, 256, dtype=torch.int32, device=device)
+        r = SimpleNamespace(T=rows, k=1, bm=256, max_tiles=n, tile_group=torch.zeros(n, dtype=torch.int32, device=device),
+                            tile_row0=row0, tile_rows=torch.clamp(rows - row0, max=256).to(torch.int32))
+        _ONE_GROUP_TILES[key] = r
+    return r
+
+
 def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``a[M,K] @ b[K,N] (+ bias[N])`` with the dtype of ``a``; any strides.
 
     bf16 operands go through the MFMA kernels: directly when ``b`` is a transposed view of an
     ``[N, K]`` row-major weight (the ``nn.Linear`` case), after packing ``b`` otherwise. fp16 and fp32
     have an MFMA kernel of their own (true fp32 products for fp32). Unaligned bf16 layouts use the
-    generic one-thread-per-output kernel. The choice depends on dtype and layout only, never on M.
+    generic one-thread-per-output kernel. Large bf16 products whose ``b`` is row-major ``[K, N]`` (data gradients)
+    or whose ``a`` is a transposed view as well (weight gradients) run on the grouped backward kernels with a
+    single group instead of going through transposed copies. Every bf16 MFMA kernel gives the same bits for the
+    same row, so which one runs (it may depend on M) changes no result.
     """
     assert a.ndim == 2 and b.ndim == 2, "matmul expects 2-D operands"
     assert a.shape[1] == b.shape[0], "Incompatible dimensions"
@@ -411,6 +435,14 @@ def matmul(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None
         # kernel reads as it lies (one group holding every row) instead of two transposed copies; same MFMA chain per
         # output element as the other kernels. Only with enough 256 x 256 output tiles to occupy the chip.
         return moe_gemm_tn(a.t(), b, _row_span(K, a.device), 1, out=c.view(1, M, N)).view(M, N)
+    if (a.dtype == torch.bfloat16 and bias is None and a.stride(1) == 1 and b.stride(1) == 1 and b.stride(0) != 1
+            and M >= 1024 and K % 64 == 0 and N % 8 == 0 and a.stride(0) % 8 == 0 and b.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and b.data_ptr() % 16 == 0 and (M * a.stride(0) + K) * 2 < (1 << 32)
+            and (64 * b.stride(0) + N) * 2 < (1 << 32) and not torch.cuda.is_current_stream_capturing()):
+        # b is row-major [K, N] (a linear layer's data gradient, d_y w): the grouped data-gradient kernel reads it as
+        # it lies, with all rows in one group, instead of a transposed copy of the weight in front of an NT kernel;
+        # same MFMA chain per output element
+        return moe_gemm_nn(a, b.unsqueeze(0), _one_group_tiles(M, a.device), out=c)
     if a.dtype == torch.bfloat16 and K % 8 == 0:
         w_nk = b.t()  # [N, K] view
         x = a
