@@ -251,7 +251,8 @@ def capture_sizes(max_size: int) -> list[int]:
 class StepBuffers:
     """Static device buffers of one (num_tokens, num_seqs) bucket."""
 
-    def __init__(self, cfg: DecoderConfig, num_tokens: int, num_seqs: int, device, packed_only: bool = False):
+    def __init__(self, cfg: DecoderConfig, num_tokens: int, num_seqs: int, device, packed_only: bool = False,
+                 packed: bool = False):
         """``packed_only``: the model holds fragment-order expert weights only (no 128-row expert tiles)."""
         T, B = num_tokens, num_seqs
         self.num_tokens, self.num_seqs = T, B
@@ -294,7 +295,7 @@ class StepBuffers:
         self.hw = z(T * k, cfg.moe_intermediate, dtype=bf)
         self.eo = z(T * k, H, dtype=bf)
         self.bm = ops.moe_tile_rows(T, wide_ok=(cfg.hidden_size % 64 == 0 and cfg.moe_intermediate % 64 == 0),
-                                    packed_only=packed_only)
+                                    packed_only=packed_only, packed=packed)
         from . import _lib
 
         lib = _lib.load()
@@ -374,7 +375,7 @@ class Qwen3MoeDecoder:
         key = (num_tokens, num_seqs)
         if key not in self.buffers:
             b = self.buffers[key] = StepBuffers(self.cfg, num_tokens, num_seqs, self.device,
-                                                packed_only=self.w.packed_only)
+                                                packed_only=self.w.packed_only, packed=self.w.packed is not None)
             # Steps run one at a time on one stream, so buckets share one decode-attention workspace. A bucket
             # that needs more than the shared one holds gets a new, larger one, which later buckets share;
             # earlier buckets (and graphs captured on them) keep the tensor they were given.
