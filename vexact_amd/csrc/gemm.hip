@@ -100,6 +100,12 @@ int vx_gemm_bf16_nt(const void* x, const void* w, const void* bias, void* c, int
     else if (mt == 2) gemm_stream_kernel<2, EPI_PLAIN, false, 8, 2><<<grid, 256, 0, stream>>>(p);
     else gemm_stream_kernel<4, EPI_PLAIN, false><<<grid, 256, 0, stream>>>(p);
   } else {
+    // 513 .. 1024 rows against a moderate weight matrix: still the ring kernel (64 x 64 tiles, three stages). Measured
+    // against the 128 x 128 tiles that ran here: o projection (2048 x 4096) at 513 / 1024 rows 61 -> 26 / 62 -> 29 us,
+    // q/k/v (5120 x 2048) 35 -> 23 / 46 -> 35 us; a 12288 x 4096 matrix is level at 384 rows and 27 % behind at 512,
+    // hence the bound on tiles x depth.
+    if (M <= 1024 && K % 64 == 0 && nt * ((M + 63) / 64) * K <= ((int64_t)1 << 22) && gemm_ring_launch(p, 0, stream))
+      return launch_status();
     // many rows: 256x256 tiles once they fill at least half the chip, else 128x128 tiles
     const int64_t wide_tiles = ((M + WD_BM - 1) / WD_BM) * ((N + WD_BN - 1) / WD_BN);
     if (wide_tiles >= 128 && gemm_wide_launch(p, stream)) return launch_status();
