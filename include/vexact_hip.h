@@ -179,7 +179,7 @@ int vx_attn_chunk_size(void);
 int64_t vx_paged_attn_decode_workspace_bytes(int64_t num_seqs, int64_t Hq, int64_t Hkv, int64_t Dv,
                                              int64_t max_kv_len);
 /* What a launch with this mode really uses: 0 when it takes the fused form (mode 4, or mode 0 with
- * num_seqs * Hkv >= 512), whose chunk states stay in LDS; then workspace may be NULL. The _bytes figure
+ * num_seqs * Hkv >= 256), whose chunk states stay in LDS; then workspace may be NULL. The _bytes figure
  * above is enough for every mode.
  * Rows of a sequence that has query tokens but no key at all (seqused_k <= 0) are left unwritten in every
  * mode, like the reference, whose grid has no block for them; query rows in front of the first key
