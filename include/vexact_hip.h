@@ -241,8 +241,8 @@ int64_t vx_moe_max_tiles(int64_t n_entries, int E, int bm);
 int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,
                  int* cu, int* scatter_index, int* sorted_token, int* sorted_flat, int* tile_group,
                  int* tile_row0, int* tile_rows, int64_t max_tiles, hipStream_t stream);
-/* The same with a workspace of vx_moe_route_workspace_bytes(T * k, E) bytes (0 below 8192 entries): from
- * 8192 entries on the work is spread over chunks of 1024 entries in three launches (per-chunk counts,
+/* The same with a workspace of vx_moe_route_workspace_bytes(T * k, E) bytes (0 below 3072 entries): from
+ * 3072 entries on the work is spread over chunks of 1024 entries in three launches (per-chunk counts,
  * one scan, per-chunk stable ranks) instead of one workgroup; identical integers. */
 int64_t vx_moe_route_workspace_bytes(int64_t n_entries, int E);
 int vx_moe_route_ws(const void* expert_idx, int idx_i64, int64_t T, int k, int E, int bm, int* splits,

@@ -562,7 +562,7 @@ int64_t vx_moe_max_tiles(int64_t n_entries, int E, int bm) {
 }
 
 // Entries from which the chunked three-launch routing is used when a workspace is given
-constexpr int64_t RB_CHUNKED_FROM = 8192;
+constexpr int64_t RB_CHUNKED_FROM = 3072;  // one workgroup / chunked, 128 experts: 2048 entries 7.7 / 9.0 us, 3072 10.0 / 9.4, 4096 12.4 / 10.3, 8192 21.8 / 11.5
 
 int64_t vx_moe_route_workspace_bytes(int64_t n_entries, int E) {
   if (n_entries < RB_CHUNKED_FROM || E <= 0) return 0;

@@ -748,7 +748,7 @@ class MoeRouting:
 
 def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int] = None, buffers=None,
               chunked: bool = True) -> MoeRouting:
-    """Routing integers of ``selected_experts [T, k]``. From 8192 entries on the work is spread over many
+    """Routing integers of ``selected_experts [T, k]``. From 3072 entries on the work is spread over many
     workgroups (needs a small workspace); ``chunked=False`` keeps the one-workgroup kernel (same integers)."""
     _need_gpu("selected_experts", selected_experts)
     assert selected_experts.dtype in (torch.int32, torch.int64)
