@@ -210,7 +210,24 @@ int vx_attention_ex(const void* q, const void* k, const void* v, void* out, floa
                     int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
                     int max_seqlen_q, void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
-/* Backward of causal varlen attention on packed q [Tq, Hq, D], k / v [Tk, Hkv, D] (D = 64 or 128):
+/* vx_attention_ex for either 16-bit element type (dtype 0 = bf16, 1 = fp16; q, k, v and out share it) and any
+ * head sizes Dk, Dv <= 256: the reference's kernels mask the head dimension to the next power of two and take
+ * fp16 or bf16 (triton_invariant_attention.py:98-103, 485-490, 645-649). bf16 at (Dk, Dv) in {(32, 32), (64, 64),
+ * (128, 128), (192, 128), (256, 256)} with 16-byte addressable rows runs kernels built for exactly those sizes
+ * (this is what vx_attention / vx_attention_ex call); every other case runs the kernels built for the next of
+ * (64, 64), (128, 128), (256, 128), (256, 256) with the missing query columns as zeros, which leaves every bit
+ * as an exact-size kernel would compute it; head sizes or strides that are not multiples of 8 elements, or bases
+ * that are not 16-byte aligned, are served with per-element accesses (correct, slow). fp32 inputs, which the
+ * reference also takes, are not supported (VX_ERR_UNSUPPORTED for any other dtype code). */
+int vx_attention_typed(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
+                       const int* cu_seqlens_q, const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
+                       int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                       int64_t sqt, int64_t sqh, int64_t skb, int64_t skp, int64_t skh, int64_t svb,
+                       int64_t svp, int64_t svh, int64_t sot, int64_t soh, int64_t bt_stride,
+                       int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
+                       int max_seqlen_q, int dtype, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
+/* Backward of causal varlen attention on packed q [Tq, Hq, D], k / v [Tk, Hkv, D] (bf16, D = 64 or 128):
  * dq, dk, dv (bf16) from dout, the forward's out and lse. P and dS are rounded to bf16 before they
  * enter a matrix product, as in the reference; all sums run in an order fixed by the sequence's own
  * lengths. strides[16] = token and head strides (elements) of q, k, v, out, dout, dq, dk, dv.
@@ -223,6 +240,16 @@ int vx_attention_bwd(const void* q, const void* k, const void* v, const void* ou
                      int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int D,
                      const int64_t* strides, float softmax_scale, int max_seqlen_q, int max_seqlen_k,
                      void* workspace, int64_t workspace_bytes, hipStream_t stream);
+/* The same for either 16-bit element type (dtype 0 = bf16, 1 = fp16) and any head sizes up to 256: Dk of
+ * q / k / dq / dk, Dv of v / out / dout / dv, as _NonpagedFlashAttentionVarlen.backward takes them
+ * (triton_invariant_attention.py:786-902, BLOCK_D = next power of two of the larger one). bf16 at Dk = Dv = 128
+ * runs the LDS kernels, everything else register-form kernels built for 64, 128 or 256 (the last two spill and
+ * are slow); rows that are not 16-byte addressable are served per element. */
+int vx_attention_bwd_typed(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                           void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
+                           int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                           const int64_t* strides, float softmax_scale, int max_seqlen_q, int max_seqlen_k, int dtype,
+                           void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 /* ---- fused MoE ------------------------------------------------------------------------- */
 

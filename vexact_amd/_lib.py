@@ -42,8 +42,13 @@ PROTOTYPES = {
         _I,
         [_P] * 10 + [_L, _L, _I, _I, _I, _I] + [_L] * 12 + [_I, _F, _I, _I, _I, _P, _L, _P],
     ),
+    "vx_attention_typed": (
+        _I,
+        [_P] * 10 + [_L, _L, _I, _I, _I, _I] + [_L] * 12 + [_I, _F, _I, _I, _I, _I, _P, _L, _P],
+    ),
     "vx_attention_bwd_workspace_bytes": (_L, [_L, _L]),
     "vx_attention_bwd": (_I, [_P] * 11 + [_L, _L, _L, _I, _I, _I, _P, _F, _I, _I, _P, _L, _P]),
+    "vx_attention_bwd_typed": (_I, [_P] * 11 + [_L, _L, _L, _I, _I, _I, _I, _P, _F, _I, _I, _I, _P, _L, _P]),
     "vx_router_topk": (_I, [_P, _P, _P, _L, _I, _I, _L, _I, _I, _I, _I, _P]),
     "vx_moe_max_tiles": (_L, [_L, _I, _I]),
     "vx_moe_route": (_I, [_P, _I, _L, _I, _I, _I] + [_P] * 8 + [_L, _P]),

@@ -55,9 +55,13 @@ def _head_rules(q, k, v, heads_axis: int) -> None:
 
 
 def _addressable(t: torch.Tensor) -> torch.Tensor:
-    """``[tokens, heads, dim]`` as the kernels can read it: unit stride in ``dim``, 16-byte aligned rows."""
-    ok = t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0 and t.data_ptr() % 16 == 0
-    return t if ok else t.contiguous()
+    """``[tokens, heads, dim]`` as the kernels read it fastest: unit stride in ``dim`` (required) and 16-byte
+    aligned rows. A view whose rows a copy would align is copied; a head size that is not a multiple of 8 elements
+    cannot be aligned and goes to the kernels as it is (they then access it element by element)."""
+    if t.stride(-1) != 1:
+        return t.contiguous()
+    aligned = t.stride(0) % 8 == 0 and t.stride(1) % 8 == 0 and t.data_ptr() % 16 == 0
+    return t if aligned or t.shape[-1] % 8 != 0 else t.contiguous()
 
 
 # ----------------------------------------------------------------------------- autograd functions

@@ -15,285 +15,9 @@
 // the accumulator registers, and their A operands (the moving rows transposed) come from 16-byte
 // row loads and an 8 x 8 bf16 transpose in registers. Every sum runs in a fixed order that depends
 // only on the sequence's own lengths, so a sequence's gradients do not depend on the batch.
-#include <algorithm>
-
-#include "common.h"
+#include "attn_bwd_core.h"
 
 namespace vx {
-
-struct AttnBwdParams {
-  const bf16_t *q, *k, *v, *o, *d_o;
-  const float* lse;  // [T, Hq] natural log
-  float* delta;      // [T, Hq] workspace
-  bf16_t *dq, *dk, *dv;
-  int64_t sqt, sqh, skt, skh, svt, svh, sot, soh, sdt, sdh, sdqt, sdqh, sdkt, sdkh, sdvt, sdvh;
-  const int *cu_q, *cu_k;
-  int Hq, Hkv, num_seqs;
-  float scale;
-};
-
-// delta[t, h] = sum_d f32(O[t, h, d]) f32(dO[t, h, d]): 16 lanes per (token, head) row, 8 dims each,
-// then a fixed butterfly over the 16 lanes
-template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_delta_kernel(AttnBwdParams p, int64_t total_q) {
-  const int64_t i = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  const int c = threadIdx.x & 15;
-  const bool live = i < total_q * p.Hq;
-  const int64_t ii = live ? i : 0;
-  const int64_t t = ii / p.Hq;
-  const int h = (int)(ii % p.Hq);
-  float s = 0.f;
-  if (8 * c < D) {
-    const uint4 a = ldg16_raw(p.o + t * p.sot + (int64_t)h * p.soh + 8 * c);
-    const uint4 b = ldg16_raw(p.d_o + t * p.sdt + (int64_t)h * p.sdh + 8 * c);
-    s += bf16lo(a.x) * bf16lo(b.x); s += bf16hi(a.x) * bf16hi(b.x);
-    s += bf16lo(a.y) * bf16lo(b.y); s += bf16hi(a.y) * bf16hi(b.y);
-    s += bf16lo(a.z) * bf16lo(b.z); s += bf16hi(a.z) * bf16hi(b.z);
-    s += bf16lo(a.w) * bf16lo(b.w); s += bf16hi(a.w) * bf16hi(b.w);
-  }
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-  if (live && c == 0) p.delta[i] = s;
-}
-
-// The moving rows of a 64-row block in the layout the transposed products read: slot idx of half ch
-// holds row 32 ch + 16 (idx / 4) + 4 g + idx % 4, dims 8 r16 .. +8 (16 lanes cover a 256-byte row).
-// rowp(r) = pointer to moving row r of the block, clamped to an existing row (its weight is 0).
-template <int D, class RowPtr>
-__device__ __forceinline__ void bwd_tr_load(RowPtr rowp, uint4 (&rows)[2][8]) {
-  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-  const bool dok = 8 * r16 < D;
-#pragma unroll
-  for (int ch = 0; ch < 2; ch++)
-#pragma unroll
-    for (int idx = 0; idx < 8; idx++) {
-      const int r = 32 * ch + 16 * (idx >> 2) + 4 * g + (idx & 3);
-      rows[ch][idx] = ldg16_raw(rowp(r) + (dok ? 8 * r16 : 0));
-    }
-}
-
-// acc[td] (rows = dims 8 r16' + td, cols = stationary) += (moving rows 0..63, transposed) x pf
-template <int D>
-__device__ __forceinline__ void bwd_tr_product(const uint4 (&rows)[2][8], const uint4 (&pf)[2], f32x4 (&acc)[8]) {
-  const int r16 = threadIdx.x & 15;
-  const bool dok = 8 * r16 < D;
-#pragma unroll
-  for (int ch = 0; ch < 2; ch++) {
-#pragma unroll
-    for (int td = 0; td < 8; td++) {
-      uint32_t w[4];
-#pragma unroll
-      for (int qd = 0; qd < 4; qd++) {
-        const uint4 ra = mask16(rows[ch][2 * qd], dok), rb = mask16(rows[ch][2 * qd + 1], dok);
-        const uint32_t a = (td < 2) ? ra.x : (td < 4) ? ra.y : (td < 6) ? ra.z : ra.w;
-        const uint32_t b = (td < 2) ? rb.x : (td < 4) ? rb.y : (td < 6) ? rb.z : rb.w;
-        w[qd] = (td & 1) ? ((a >> 16) | (b & 0xffff0000u)) : ((a & 0xffffu) | (b << 16));
-      }
-      acc[td] = mfma16(make_uint4(w[0], w[1], w[2], w[3]), pf[ch], acc[td]);
-    }
-  }
-}
-
-// lane (g, c) holds acc[td][r] = element (dim 32 g + 8 r + td) of stationary row c: 16 bytes per r
-template <int D>
-__device__ __forceinline__ void bwd_store_tile(const f32x4 (&acc)[8], bf16_t* rowp) {
-  const int g = (threadIdx.x & 63) >> 4;
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    const int d0 = 32 * g + 8 * r;
-    if (d0 >= D) continue;
-    uint4 pk;
-    pk.x = pack_bf16x2(acc[0][r], acc[1][r]);
-    pk.y = pack_bf16x2(acc[2][r], acc[3][r]);
-    pk.z = pack_bf16x2(acc[4][r], acc[5][r]);
-    pk.w = pack_bf16x2(acc[6][r], acc[7][r]);
-    *(uint4*)(rowp + d0) = pk;
-  }
-}
-
-__device__ __forceinline__ void bwd_pack(const float (&x)[4][4], uint4 (&pf)[2]) {
-  uint32_t pw[4][2];
-#pragma unroll
-  for (int tt = 0; tt < 4; tt++) {
-    pw[tt][0] = pack_bf16x2(x[tt][0], x[tt][1]);
-    pw[tt][1] = pack_bf16x2(x[tt][2], x[tt][3]);
-  }
-  pf[0] = make_uint4(pw[0][0], pw[0][1], pw[1][0], pw[1][1]);
-  pf[1] = make_uint4(pw[2][0], pw[2][1], pw[3][0], pw[3][1]);
-}
-
-// ---- dQ: grid (query tiles / 4, Hq, sequences), wavefront = 16 queries of one head ------------
-template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(AttnBwdParams p) {
-  constexpr int KS = D / 32;
-  const int seq = blockIdx.z, h = blockIdx.y;
-  const int q0 = p.cu_q[seq], qlen = p.cu_q[seq + 1] - q0;
-  const int k0 = p.cu_k[seq], kv_len = p.cu_k[seq + 1] - k0;
-  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-  const int i0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
-  if (i0 >= qlen || kv_len <= 0) return;
-  const int kvh = h / (p.Hq / p.Hkv);
-  const int shift = kv_len - qlen;
-  const int i = i0 + r16;                      // this lane's query (stationary column)
-  const bool qok = i < qlen;
-  const int pos = qok ? shift + i : -1;        // last visible key; -1: nothing visible
-  const int64_t tq = q0 + (qok ? i : qlen - 1);
-  uint4 qf[KS], of[KS];
-  {
-    const bf16_t* qp = p.q + tq * p.sqt + (int64_t)h * p.sqh + 8 * g;
-    const bf16_t* dp = p.d_o + tq * p.sdt + (int64_t)h * p.sdh + 8 * g;
-#pragma unroll
-    for (int s = 0; s < KS; s++) {
-      qf[s] = ldg16_raw(qp + 32 * s);
-      of[s] = ldg16_raw(dp + 32 * s);
-    }
-  }
-  const float c2 = p.scale * 1.44269504f;
-  const float lse2 = p.lse[tq * p.Hq + h] * 1.44269504f;
-  const float delta = p.delta[tq * p.Hq + h];
-  int maxpos = pos;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) maxpos = max(maxpos, __shfl_xor(maxpos, o, 64));
-  maxpos = min(maxpos, kv_len - 1);
-
-  f32x4 acc[8];
-#pragma unroll
-  for (int td = 0; td < 8; td++) acc[td] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16_t* kb_ = p.k + (int64_t)k0 * p.skt + (int64_t)kvh * p.skh;
-  const bf16_t* vb_ = p.v + (int64_t)k0 * p.svt + (int64_t)kvh * p.svh;
-  for (int kb = 0; kb <= maxpos; kb += 64) {
-    // every load of the block is issued before the first is used: one memory round trip per block
-    uint4 kfr[4][KS], vfr[4][KS], rows[2][8];
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++) {
-      const int64_t kr = min(kb + 16 * tt + r16, kv_len - 1);
-      const bf16_t* kp = kb_ + kr * p.skt + 8 * g;
-      const bf16_t* vp = vb_ + kr * p.svt + 8 * g;
-#pragma unroll
-      for (int s = 0; s < KS; s++) {
-        kfr[tt][s] = ldg16_raw(kp + 32 * s);
-        vfr[tt][s] = ldg16_raw(vp + 32 * s);
-      }
-    }
-    bwd_tr_load<D>([&](int r) { return kb_ + (int64_t)min(kb + r, kv_len - 1) * p.skt; }, rows);
-    float ds[4][4];
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++) {
-      f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f}, dp = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < KS; s++) {
-        st = mfma16(kfr[tt][s], qf[s], st);
-        dp = mfma16(vfr[tt][s], of[s], dp);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const int key = kb + 16 * tt + 4 * g + r;
-        const float pr = (key <= pos) ? __builtin_amdgcn_exp2f(st[r] * c2 - lse2) : 0.f;
-        ds[tt][r] = pr * (dp[r] - delta) * p.scale;
-      }
-    }
-    uint4 pf[2];
-    bwd_pack(ds, pf);
-    bwd_tr_product<D>(rows, pf, acc);
-  }
-  if (qok) bwd_store_tile<D>(acc, p.dq + tq * p.sdqt + (int64_t)h * p.sdqh);
-}
-
-// ---- dK, dV: grid (key tiles / 4, Hkv, sequences), wavefront = 16 keys of one kv head ----------
-template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(AttnBwdParams p) {
-  constexpr int KS = D / 32;
-  const int seq = blockIdx.z, kvh = blockIdx.y;
-  const int q0 = p.cu_q[seq], qlen = p.cu_q[seq + 1] - q0;
-  const int k0 = p.cu_k[seq], kv_len = p.cu_k[seq + 1] - k0;
-  const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
-  const int j0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
-  if (j0 >= kv_len) return;
-  const int G = p.Hq / p.Hkv;
-  const int shift = kv_len - qlen;
-  const int j = j0 + r16;                       // this lane's key (stationary column)
-  const bool kok = j < kv_len;
-  const int64_t tk = k0 + (kok ? j : kv_len - 1);
-  uint4 kf[KS], vf[KS];
-  {
-    const bf16_t* kp = p.k + tk * p.skt + (int64_t)kvh * p.skh + 8 * g;
-    const bf16_t* vp = p.v + tk * p.svt + (int64_t)kvh * p.svh + 8 * g;
-#pragma unroll
-    for (int s = 0; s < KS; s++) {
-      kf[s] = ldg16_raw(kp + 32 * s);
-      vf[s] = ldg16_raw(vp + 32 * s);
-    }
-  }
-  const float c2 = p.scale * 1.44269504f;
-  f32x4 dk[8], dv[8];
-#pragma unroll
-  for (int td = 0; td < 8; td++) {
-    dk[td] = f32x4{0.f, 0.f, 0.f, 0.f};
-    dv[td] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-  // first query that sees key j0 (queries before it see none of the tile's keys)
-  const int istart = max(0, j0 - shift);
-  if (qlen > 0) {
-    for (int hh = 0; hh < G; hh++) {
-      const int h = kvh * G + hh;
-      const bf16_t* qb_ = p.q + (int64_t)q0 * p.sqt + (int64_t)h * p.sqh;
-      const bf16_t* db_ = p.d_o + (int64_t)q0 * p.sdt + (int64_t)h * p.sdh;
-      for (int ib = istart; ib < qlen; ib += 64) {
-        // phase 1: the block's Q and dO rows as A operands plus the rows' lse and delta, all loads first
-        uint4 qfr[4][KS], ofr[4][KS];
-        float lse2[4][4], dl[4][4];
-#pragma unroll
-        for (int tt = 0; tt < 4; tt++) {
-          const int64_t ir = min(ib + 16 * tt + r16, qlen - 1);
-          const bf16_t* qp = qb_ + ir * p.sqt + 8 * g;
-          const bf16_t* dp_ = db_ + ir * p.sdt + 8 * g;
-#pragma unroll
-          for (int s = 0; s < KS; s++) {
-            qfr[tt][s] = ldg16_raw(qp + 32 * s);
-            ofr[tt][s] = ldg16_raw(dp_ + 32 * s);
-          }
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const int64_t tq = q0 + min(ib + 16 * tt + 4 * g + r, qlen - 1);
-            lse2[tt][r] = p.lse[tq * p.Hq + h];
-            dl[tt][r] = p.delta[tq * p.Hq + h];
-          }
-        }
-        float pr[4][4], ds[4][4];
-#pragma unroll
-        for (int tt = 0; tt < 4; tt++) {
-          f32x4 st = f32x4{0.f, 0.f, 0.f, 0.f}, dp = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int s = 0; s < KS; s++) {
-            st = mfma16(qfr[tt][s], kf[s], st);
-            dp = mfma16(ofr[tt][s], vf[s], dp);
-          }
-#pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const int iq = ib + 16 * tt + 4 * g + r;    // this register's query (moving row)
-            const bool ok = iq < qlen && kok && j <= shift + iq;
-            const float e = ok ? __builtin_amdgcn_exp2f(st[r] * c2 - lse2[tt][r] * 1.44269504f) : 0.f;
-            pr[tt][r] = e;
-            ds[tt][r] = e * (dp[r] - dl[tt][r]) * p.scale;
-          }
-        }
-        // phase 2: the same rows in the transposable layout (they are in the cache now)
-        uint4 rows_o[2][8], rows_q[2][8];
-        bwd_tr_load<D>([&](int r) { return db_ + (int64_t)min(ib + r, qlen - 1) * p.sdt; }, rows_o);
-        bwd_tr_load<D>([&](int r) { return qb_ + (int64_t)min(ib + r, qlen - 1) * p.sqt; }, rows_q);
-        uint4 pfp[2], pfs[2];
-        bwd_pack(pr, pfp);
-        bwd_pack(ds, pfs);
-        bwd_tr_product<D>(rows_o, pfp, dv);
-        bwd_tr_product<D>(rows_q, pfs, dk);
-      }
-    }
-  }
-  if (kok) {
-    bwd_store_tile<D>(dk, p.dk + tk * p.sdkt + (int64_t)kvh * p.sdkh);
-    bwd_store_tile<D>(dv, p.dv + tk * p.sdvt + (int64_t)kvh * p.sdvh);
-  }
-}
 
 // ---------------------------------------------------------------------------------------
 // Head size 128: the moving side goes through LDS once per workgroup. 8 wavefronts hold 8 stationary
@@ -461,7 +185,7 @@ __global__ __launch_bounds__(64 * BWL_WAVES) void attn_bwd_dq_lds_kernel(AttnBwd
       }
     }
     uint4 pf[2];
-    bwd_pack(ds, pf);
+    bwd_pack<ElemBF16>(ds, pf);
     bwl_tr_product(ks, pf, acc);
   };
   // (unrolling over the two stages would make the LDS offsets immediates but costs 13 registers, which
@@ -580,8 +304,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
       }
     }
     uint4 pfp[2], pfs[2];
-    bwd_pack(pr, pfp);
-    bwd_pack(ds, pfs);
+    bwd_pack<ElemBF16>(pr, pfp);
+    bwd_pack<ElemBF16>(ds, pfs);
     bwl_tr_product(os, pfp, dv);
     bwl_tr_product(qs, pfs, dk);
   };
@@ -595,41 +319,27 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
   }
 }
 
-template <int D>
-static int launch_attn_bwd(const AttnBwdParams& p, int64_t total_q, int num_seqs, int max_q, int max_k, hipStream_t stream) {
-  attn_bwd_delta_kernel<D><<<(unsigned)((total_q * p.Hq + 15) / 16), 256, 0, stream>>>(p, total_q);
-  if constexpr (D == 128) {
+// bf16, head size 128 exactly: the LDS kernels
+static int launch_attn_bwd_lds128(const AttnBwdParams& p, int64_t total_q, int num_seqs, int max_q, int max_k, hipStream_t stream) {
+  attn_bwd_delta_kernel<ElemBF16, 128, false><<<(unsigned)((total_q * p.Hq + 15) / 16), 256, 0, stream>>>(p, total_q);
+  {
     static DeviceOnce once;
     const int dev = once.slot();
     if (once.need(dev)) {
-      if (hipFuncSetAttribute((const void*)attn_bwd_dq_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, BWL_LDS) != hipSuccess) {
+      if (hipFuncSetAttribute((const void*)attn_bwd_dq_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, BWL_LDS) != hipSuccess ||
+          hipFuncSetAttribute((const void*)attn_bwd_dkv_lds_kernel<BWK_WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, BWK_LDS) != hipSuccess) {
         (void)hipGetLastError();
         return VX_ERR_LAUNCH;
       }
       once.mark(dev);
     }
-    attn_bwd_dq_lds_kernel<<<dim3((unsigned)p.Hq, (unsigned)((max_q + 16 * BWL_WAVES - 1) / (16 * BWL_WAVES)), (unsigned)num_seqs),
-                             64 * BWL_WAVES, BWL_LDS, stream>>>(p);
-  } else {
-    attn_bwd_dq_kernel<D><<<dim3((unsigned)((max_q + 63) / 64), (unsigned)p.Hq, (unsigned)num_seqs), 256, 0, stream>>>(p);
   }
-  if constexpr (D == 128) {
-    static DeviceOnce once;
-    const int dev = once.slot();
-    if (once.need(dev)) {
-      if (hipFuncSetAttribute((const void*)attn_bwd_dkv_lds_kernel<BWK_WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, BWK_LDS) != hipSuccess) {
-        (void)hipGetLastError();
-        return VX_ERR_LAUNCH;
-      }
-      once.mark(dev);
-    }
-    const int sg = std::max(1, std::min(num_seqs, 8 / std::max(1, p.Hkv)));  // sequences per group of eight workgroups
-    attn_bwd_dkv_lds_kernel<BWK_WAVES><<<dim3((unsigned)(p.Hkv * sg), (unsigned)((max_k + 16 * BWK_WAVES - 1) / (16 * BWK_WAVES)),
-                                              (unsigned)((num_seqs + sg - 1) / sg)),
-                                         64 * BWK_WAVES, BWK_LDS, stream>>>(p);
-  } else {
-    attn_bwd_dkv_kernel<D><<<dim3((unsigned)((max_k + 63) / 64), (unsigned)p.Hkv, (unsigned)num_seqs), 256, 0, stream>>>(p);
-  }
+  attn_bwd_dq_lds_kernel<<<dim3((unsigned)p.Hq, (unsigned)((max_q + 16 * BWL_WAVES - 1) / (16 * BWL_WAVES)), (unsigned)num_seqs),
+                           64 * BWL_WAVES, BWL_LDS, stream>>>(p);
+  const int sg = std::max(1, std::min(num_seqs, 8 / std::max(1, p.Hkv)));  // sequences per group of eight workgroups
+  attn_bwd_dkv_lds_kernel<BWK_WAVES><<<dim3((unsigned)(p.Hkv * sg), (unsigned)((max_k + 16 * BWK_WAVES - 1) / (16 * BWK_WAVES)),
+                                            (unsigned)((num_seqs + sg - 1) / sg)),
+                                       64 * BWK_WAVES, BWK_LDS, stream>>>(p);
   return launch_status();
 }
 
@@ -640,22 +350,42 @@ extern "C" {
 int64_t vx_attention_bwd_workspace_bytes(int64_t total_q, int64_t Hq) { return total_q * Hq * 4; }
 
 // strides[16]: token and head strides (elements) of q, k, v, out, dout, dq, dk, dv, in that order.
+int vx_attention_bwd_typed(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                           void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
+                           int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                           const int64_t* strides, float softmax_scale, int max_seqlen_q, int max_seqlen_k, int dtype,
+                           void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
 int vx_attention_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
                      void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
                      int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int D,
                      const int64_t* strides, float softmax_scale, int max_seqlen_q, int max_seqlen_k,
                      void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  return vx_attention_bwd_typed(q, k, v, out, dout, lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, total_q, total_k, num_seqs, Hq,
+                                Hkv, D, D, strides, softmax_scale, max_seqlen_q, max_seqlen_k, 0, workspace, workspace_bytes, stream);
+}
+
+// Any head sizes up to 256 (Dk of q / k / dq / dk, Dv of v / out / dout / dv) and either 16-bit element type
+// (dtype 0 = bf16, 1 = fp16). bf16 at Dk = Dv = 128 runs the LDS kernels, everything else the register-form kernels
+// of the next built-for size (64, 128, 256), per element when rows are not 16-byte addressable.
+int vx_attention_bwd_typed(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                           void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
+                           int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
+                           const int64_t* strides, float softmax_scale, int max_seqlen_q, int max_seqlen_k, int dtype,
+                           void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   using namespace vx;
   if (!q || !k || !v || !out || !dout || !lse || !dq || !dk || !dv || !cu_seqlens_q || !cu_seqlens_k || !strides)
     return VX_ERR_ARG;
-  if (total_q < 0 || total_k < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return VX_ERR_ARG;
+  if (total_q < 0 || total_k < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Dk <= 0 || Dv <= 0) return VX_ERR_ARG;
   if (max_seqlen_q < 0 || max_seqlen_k < 0 || num_seqs > 65535 || Hq > 65535) return VX_ERR_ARG;
+  if (dtype != 0 && dtype != 1) return VX_ERR_UNSUPPORTED;
+  if (Dk > 256 || Dv > 256) return VX_ERR_UNSUPPORTED;
   if (total_q == 0 || total_k == 0 || num_seqs == 0 || max_seqlen_q == 0 || max_seqlen_k == 0) return VX_OK;
-  for (int i = 0; i < 16; i++)
-    if (strides[i] % 8 != 0) return VX_ERR_UNSUPPORTED;
-  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dq | (uintptr_t)dk |
-       (uintptr_t)dv) % 16 != 0)
-    return VX_ERR_UNSUPPORTED;
+  const uintptr_t ptrs = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dq |
+                         (uintptr_t)dk | (uintptr_t)dv;
+  if (ptrs % 2 != 0) return VX_ERR_ARG;
+  bool elem = ptrs % 16 != 0 || Dk % 8 != 0 || Dv % 8 != 0;
+  for (int i = 0; i < 16; i++) elem = elem || strides[i] % 8 != 0;
   if (!workspace || workspace_bytes < total_q * Hq * 4 || ((uintptr_t)workspace & 15)) return VX_ERR_WORKSPACE;
   if (total_q * Hq > 0x7fffffffLL * 16) return VX_ERR_ARG;
   AttnBwdParams p = {};
@@ -668,9 +398,17 @@ int vx_attention_bwd(const void* q, const void* k, const void* v, const void* ou
   p.sdkt = strides[12]; p.sdkh = strides[13]; p.sdvt = strides[14]; p.sdvh = strides[15];
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
   p.Hq = Hq; p.Hkv = Hkv; p.num_seqs = (int)num_seqs; p.scale = softmax_scale;
-  if (D == 128) return launch_attn_bwd<128>(p, total_q, (int)num_seqs, max_seqlen_q, max_seqlen_k, stream);
-  if (D == 64) return launch_attn_bwd<64>(p, total_q, (int)num_seqs, max_seqlen_q, max_seqlen_k, stream);
-  return VX_ERR_UNSUPPORTED;
+  p.dk_ = Dk; p.dv_ = Dv; p.elem = elem ? 1 : 0;
+  const int ns = (int)num_seqs;
+  if (dtype == 0 && !elem && Dk == Dv) {
+    if (Dk == 128) return launch_attn_bwd_lds128(p, total_q, ns, max_seqlen_q, max_seqlen_k, stream);
+    if (Dk == 64) return launch_attn_bwd_generic<ElemBF16, 64, false>(p, total_q, ns, max_seqlen_q, max_seqlen_k, stream);
+  }
+  const int Db = std::max(Dk, Dv) <= 64 ? 64 : std::max(Dk, Dv) <= 128 ? 128 : 256;
+  if (dtype == 1) return launch_attn_bwd_f16(p, Db, total_q, ns, max_seqlen_q, max_seqlen_k, stream);
+  if (Db == 64) return launch_attn_bwd_generic<ElemBF16, 64, true>(p, total_q, ns, max_seqlen_q, max_seqlen_k, stream);
+  if (Db == 128) return launch_attn_bwd_generic<ElemBF16, 128, true>(p, total_q, ns, max_seqlen_q, max_seqlen_k, stream);
+  return launch_attn_bwd_generic<ElemBF16, 256, true>(p, total_q, ns, max_seqlen_q, max_seqlen_k, stream);
 }
 
 }  // extern "C"

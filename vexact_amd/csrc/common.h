@@ -67,6 +67,36 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
                                                  __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// The two 16-bit element types of the attention kernels: how eight of them enter the matrix core, how two fp32
+// values round (to nearest even) into a packed pair, and how a packed pair widens again. Kernels take one of these
+// as a template parameter; everything else (layouts, transposes, the order of every sum) is the same for both.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+struct ElemBF16 {
+  static constexpr int kDtype = 0;
+  static __device__ __forceinline__ f32x4 mfma(uint4 a, uint4 b, f32x4 c) { return mfma16(a, b, c); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+  static __device__ __forceinline__ float lo(uint32_t w) { return bf16lo(w); }
+  static __device__ __forceinline__ float hi(uint32_t w) { return bf16hi(w); }
+  // acc + lo + hi of a packed pair in one v_dot2c_f32_bf16 against a pair of ones
+  static __device__ __forceinline__ float add2(uint32_t pk, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), acc, false);
+  }
+};
+struct ElemF16 {
+  static constexpr int kDtype = 1;
+  static __device__ __forceinline__ f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  }
+  static __device__ __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2_t, w)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2_t, w)[1]; }
+  static __device__ __forceinline__ float add2(uint32_t pk, float acc) { return (acc + lo(pk)) + hi(pk); }
+};
+
 // 16-byte global loads. The address must always be dereferenceable (callers clamp it); zeroing
 // is done on the loaded VALUE, and only where the value is consumed, so that a load stays a single
 // global_load_dwordx4 and the wait for it is not pulled up to the issue point.

@@ -545,6 +545,15 @@ def store_kvcache(key, value, k_cache, v_cache, slot_mapping) -> None:
     )
 
 
+def _attn_dtype_code(what: str, *tensors: torch.Tensor) -> int:
+    """0 for bf16, 1 for fp16 (the C ABI's dtype code); every tensor must share it. fp32, which the reference's
+    kernels also take (through TF32 products), is not supported."""
+    dt = tensors[0].dtype
+    if dt not in (torch.bfloat16, torch.float16) or any(t.dtype != dt for t in tensors):
+        raise ValueError(f"{what} supports bfloat16 or float16 tensors of one dtype, got {[str(t.dtype) for t in tensors]}")
+    return 0 if dt == torch.bfloat16 else 1
+
+
 def paged_attention(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -571,10 +580,11 @@ def paged_attention(
     o = out if out is not None else torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
     if T == 0:
         return o
-    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
-        raise ValueError("paged attention supports bfloat16 q/k/v only")
-    if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1:
-        raise ValueError("q, k and v must be contiguous in the head dimension")
+    dtype = _attn_dtype_code("paged attention", q, k_cache, v_cache, o)
+    if Dk > 256 or Dv > 256:
+        raise ValueError(f"head_dim must be <= 256, got {Dk}")
+    if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1 or o.stride(-1) != 1:
+        raise ValueError("q, k, v and out must be contiguous in the head dimension")
     lib = _lib.load()
     B = seqused_k.numel()
     page = k_cache.shape[1]
@@ -588,12 +598,12 @@ def paged_attention(
     if seq_order is not None and (seq_order.dtype != torch.int32 or seq_order.numel() != B or not seq_order.is_contiguous()):
         raise ValueError("seq_order must be a contiguous int32 permutation of the sequences")
     _lib.check(
-        lib.vx_attention_ex(
+        lib.vx_attention_typed(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), o.data_ptr(), None, _ptr(seq_order),
             cu_seqlens_q.data_ptr(), seqused_k.data_ptr(), None, page_table.data_ptr(), T, B, Hq, Hkv, Dk, Dv,
             q.stride(0), q.stride(1), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
             v_cache.stride(0), v_cache.stride(1), v_cache.stride(2), o.stride(0), o.stride(1),
-            page_table.stride(0), max_pages, page, float(softmax_scale), 1, mode, int(max_seqlen_q),
+            page_table.stride(0), max_pages, page, float(softmax_scale), 1, mode, int(max_seqlen_q), dtype,
             _ptr(ws), ws.numel() * ws.element_size() if ws is not None else 0, _stream(),
         ),
         "vx_attention",
@@ -620,15 +630,18 @@ def packed_attention(
     lse = torch.empty((T, Hq), dtype=torch.float32, device=q.device) if return_lse else None
     if T == 0:
         return (o, lse) if return_lse else o
-    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
-        raise ValueError("attention supports bfloat16 q/k/v only")
+    dtype = _attn_dtype_code("attention", q, k, v)
+    if Dk > 256 or Dv > 256:
+        raise ValueError(f"head_dim must be <= 256, got {Dk}")
+    if q.stride(-1) != 1 or k.stride(-1) != 1 or v.stride(-1) != 1:
+        raise ValueError("q, k and v must be contiguous in the head dimension")
     B = cu_seqlens_q.numel() - 1
     _lib.check(
-        _lib.load().vx_attention_ex(
+        _lib.load().vx_attention_typed(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _ptr(lse), None, cu_seqlens_q.data_ptr(), None,
             cu_seqlens_k.data_ptr(), None, T, B, Hq, Hkv, Dk, Dv, q.stride(0), q.stride(1),
             0, k.stride(0), k.stride(1), 0, v.stride(0), v.stride(1), o.stride(0), o.stride(1),
-            0, 0, 0, float(softmax_scale), 1 if causal else 0, 2, int(max_seqlen_q), None, 0, _stream(),
+            0, 0, 0, float(softmax_scale), 1 if causal else 0, 2, int(max_seqlen_q), dtype, None, 0, _stream(),
         ),
         "vx_attention",
     )
@@ -639,15 +652,18 @@ def packed_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
     cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, softmax_scale: float, max_seqlen_q: int, max_seqlen_k: int,
 ):
-    """(dq, dk, dv) of causal ``packed_attention`` (bf16, shapes of q, k, v)."""
+    """(dq, dk, dv) of causal ``packed_attention`` (bf16 or fp16, head sizes up to 256; shapes of q, k, v)."""
     for name, t in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)):
         _need_gpu(name, t)
-        if t.dtype != torch.bfloat16 or t.dim() != 3 or t.stride(2) != 1:
-            raise ValueError(f"attention backward: {name} must be bf16 [tokens, heads, dim] with a contiguous last dim")
+        if t.dim() != 3 or t.stride(2) != 1:
+            raise ValueError(f"attention backward: {name} must be [tokens, heads, dim] with a contiguous last dim")
+    dtype = _attn_dtype_code("attention backward", q, k, v, out, dout)
     T, Hq, D = q.shape
     Tk, Hkv, Dv = v.shape
-    if D != Dv or k.shape != (Tk, Hkv, D) or D not in (64, 128):
-        raise ValueError(f"attention backward supports equal q/k/v head sizes of 64 or 128, got {D} and {Dv}")
+    if k.shape != (Tk, Hkv, D) or out.shape != (T, Hq, Dv) or dout.shape != (T, Hq, Dv):
+        raise ValueError("attention backward: q / k and v / out / dout shapes do not match")
+    if D > 256 or Dv > 256:
+        raise ValueError(f"head_dim must be <= 256, got {D}")
     if lse.dtype != torch.float32 or lse.shape != (T, Hq) or not lse.is_contiguous():
         raise ValueError("attention backward: lse must be a contiguous fp32 [tokens, heads] tensor")
     dq, dk, dv = _empty_like(q), _empty_like(k), _empty_like(v)
@@ -657,11 +673,11 @@ def packed_attention_backward(
     ws = _workspace(lib.vx_attention_bwd_workspace_bytes(T, Hq), q.device)
     strides = (ctypes.c_int64 * 16)(*[s for t in (q, k, v, out, dout, dq, dk, dv) for s in (t.stride(0), t.stride(1))])
     _lib.check(
-        lib.vx_attention_bwd(
+        lib.vx_attention_bwd_typed(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), dq.data_ptr(),
             dk.data_ptr(), dv.data_ptr(), cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), T, Tk,
-            cu_seqlens_q.numel() - 1, Hq, Hkv, D, strides, float(softmax_scale), int(max_seqlen_q), int(max_seqlen_k),
-            ws.data_ptr(), ws.numel(), _stream(),
+            cu_seqlens_q.numel() - 1, Hq, Hkv, D, Dv, strides, float(softmax_scale), int(max_seqlen_q), int(max_seqlen_k),
+            dtype, ws.data_ptr(), ws.numel(), _stream(),
         ),
         "vx_attention_bwd",
     )
