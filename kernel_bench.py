@@ -437,7 +437,7 @@ def dropin_decode(a, quiet: bool = False) -> list:
 
     from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
     from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
-    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, fuse_qkv_weights
 
     say = (lambda *x, **k: None) if quiet else print
     B, page = a.batch, a.page
@@ -465,6 +465,7 @@ def dropin_decode(a, quiet: bool = False) -> list:
     rot.inv_freq, rot.original_inv_freq = inv, inv.clone()
     for layer in model.model.layers:
         layer.mlp.experts.pack_for_decode()
+    fuse_qkv_weights(model)  # the optional load-time step: one q/k/v projection per layer instead of three
     rng = np.random.default_rng(5)
     lens = rng.integers(256, 2049, size=B)
     pages = [(int(n) + 2 + page - 1) // page for n in lens]

@@ -27,7 +27,10 @@ routing_integers_ref   brute-force counting; numpy stable argsort twice (fused_m
 fused_moe_ref          k=1,w=1 => plain SwiGLU MLP; all tokens on one expert => dense formula;
                        fp64 brute force on tiny shapes; HF-eager form within bf16 tolerance
 prepare_gen_ctx_ref    hand-worked example; vectorised numpy twin
-BlockAllocatorRef      scan restatement of the reference allocator; hand-worked sequence
+pad_for_graph_ref      hand-worked example (3 requests in a bucket of 8 tokens / 5 sequences) from the reference's
+                       statements (inferencer.py:306-324), tests/test_host_logic.py
+BlockAllocatorRef      hand-worked sequence on the restatement itself (lowest id first, out-of-blocks takes
+                       nothing, double / foreign frees ignored), tests/test_host_logic.py
 rope_tables_ref        HuggingFace Qwen3MoeRotaryEmbedding bit for bit (three theta / head sizes, positions to
                        40959); position 0 = identity, first pair turns by `position` radians
 rope_ref               HuggingFace apply_rotary_pos_emb bit for bit; pair lengths preserved

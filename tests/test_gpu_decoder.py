@@ -224,9 +224,15 @@ def test_sampled_decode_is_batch_invariant_and_graph_safe():
     assert torch.equal(bg.tokens.cpu()[:5], tok_e[order])
 
 
-def test_model_with_fragment_order_expert_weights_only_keeps_every_bit():
+def test_model_with_fragment_order_expert_weights_only_keeps_every_bit(monkeypatch):
     # one copy of the expert weights: prefill (256-row expert tiles on the packed weights instead of 128-row tiles
-    # on [E, N, K]) and decode give the bits of the model that keeps both
+    # on [E, N, K]) and decode give the bits of the model that keeps both. The model with [E, N, K] tensors is held
+    # to 128-row tiles here (the tile height is chosen from the rows per expert, which at 8 experts / top-2 would
+    # also give it 256-row tiles), so that the two prefills really run different kernels.
+    from vexact_amd import ops
+    real = ops.moe_tile_rows
+    monkeypatch.setattr(ops, "moe_tile_rows",
+                        lambda n, **kw: 128 if not kw.get("packed_only") and real(n, **kw) == 256 else real(n, **kw))
     cfg, w, dec, prompts, blocks = _setup(num_seqs=10, seed=13)
     allseq = list(range(10))
     assert sum(len(p) for p in prompts) > 1024

@@ -314,15 +314,17 @@ def test_fused_rms_norm_patch_gives_the_bits_of_the_unfused_forward():
             assert_bitwise(fused, unfused, f"fused RMSNorm forward, shape {shape}, {dtype}")
             with torch.inference_mode():  # outside the mode the original forward runs
                 assert_bitwise(norm(x), original(norm, x), "outside batch-invariant mode")
-        # Rows of small entries reach arguments where the GPU's torch.rsqrt and the kernel's 1 / sqrt (the CPU's
-        # torch.rsqrt) differ by an fp32 ulp: a few elements in 10^5 then round to the neighbouring bf16 value
+        # Rows of small and of large entries sweep the argument of the reciprocal square root over many binades: the
+        # kernel's HuggingFace form uses the device library's rsqrt, the operation torch.rsqrt runs on this device,
+        # so every element has the unfused forward's bits (1 / sqrt differs from it by an fp32 ulp now and then, which
+        # used to move about one output element in 10^5 to the neighbouring bf16 value)
         for n in (64, 320, 2048):
             norm = hf.Qwen3MoeRMSNorm(n, eps=1e-6).to(BF).cuda()
-            x = (0.05 * torch.randn(600, n, generator=g)).to(BF).cuda()
-            with torch.inference_mode(), set_batch_invariant_mode(True):
-                fused, unfused = norm(x), original(norm, x)
-            ulp = (fused.view(torch.int16).int() - unfused.view(torch.int16).int()).abs()
-            assert int(ulp.max()) <= 1 and int((ulp > 0).sum()) <= 1e-4 * ulp.numel(), f"n={n}: {int((ulp > 0).sum())} elements differ"
+            for scale in (0.05, 1.0, 30.0, 1e-3):
+                x = (scale * torch.randn(600, n, generator=g)).to(BF).cuda()
+                with torch.inference_mode(), set_batch_invariant_mode(True):
+                    fused, unfused = norm(x), original(norm, x)
+                assert_bitwise(fused, unfused, f"fused RMSNorm forward on rows of scale {scale}, n={n}")
         # with autograd the same kernel runs (the trainer's forward is the rollout's), and its backward is the
         # derivative of the original forward
         norm = hf.Qwen3MoeRMSNorm(256, eps=1e-6)
@@ -412,7 +414,7 @@ def test_fused_attention_and_residual_patches_give_the_bits_of_the_unfused_forwa
     from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
     from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
     from vexact_amd.decoder import build_step_metadata
-    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, remove_qwen3_moe_patches
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, fuse_qkv_weights, remove_qwen3_moe_patches, unfuse_qkv_weights
     from vexact_amd.models.qwen3_moe.modeling_qwen3_moe import fused_attention_forward, fused_decoder_layer_forward
 
     page, max_blocks_per_req = 16, 16
@@ -461,25 +463,48 @@ def test_fused_attention_and_residual_patches_give_the_bits_of_the_unfused_forwa
             for t in list(s.key_cache.values()) + list(s.value_cache.values()):
                 t.zero_()
         unfused = run(False, stores[0])
-        fused = run(True, stores[1])
         attn = model.model.layers[0].self_attn
+        ptrs = [p_.data_ptr() for p_ in (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)]
+        fused = run(True, stores[1])   # three projections into one buffer: a forward never touches the parameters
+        assert [p_.data_ptr() for p_ in (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)] == ptrs
+        assert getattr(attn, "_vx_qkv_weight", None) is None
+
+        def same_as_unfused(got, what):
+            for name, a, b in zip(("prefill", "decode"), got, unfused):
+                assert_bitwise(a, b, f"{name} logits, fused attention forward ({what}) vs HuggingFace's")
+            for layer in range(2):
+                assert_bitwise(stores[1].key_cache[layer], stores[0].key_cache[layer], f"key cache of layer {layer} ({what})")
+                assert_bitwise(stores[1].value_cache[layer], stores[0].value_cache[layer], f"value cache of layer {layer} ({what})")
+
+        same_as_unfused(fused, "separate weights")
+        # the explicit load-time step: one weight tensor per module, the parameters its row ranges
+        before = {k: v.clone() for k, v in model.state_dict().items()}
+        assert fuse_qkv_weights(model) == len(model.model.layers)
         assert attn.q_proj.weight.data_ptr() == attn._vx_qkv_weight.data_ptr(), "the parameters are views of the fused weight"
-        for name, a, b in zip(("prefill", "decode"), fused, unfused):
-            assert_bitwise(a, b, f"{name} logits, fused attention forward vs HuggingFace's")
-        for layer in range(2):
-            assert_bitwise(stores[1].key_cache[layer], stores[0].key_cache[layer], f"key cache of layer {layer}")
-            assert_bitwise(stores[1].value_cache[layer], stores[0].value_cache[layer], f"value cache of layer {layer}")
+        after = model.state_dict()
+        assert list(after) == list(before) and all(torch.equal(after[k], before[k]) for k in before), "state_dict values"
+        same_as_unfused(run(True, stores[1]), "one weight")
         # a parameter written in place (what a weight synchronisation does) reaches the fused weight; one that gets
-        # new storage makes the module rebuild it
+        # new storage takes the module back to three projections
         with torch.no_grad():
-            attn.k_proj.weight.data.mul_(0.5)
+            attn.v_proj.weight.data.mul_(0.5)
         again_fused, again_unfused = run(True, stores[1]), run(False, stores[0])
         assert_bitwise(again_fused[1], again_unfused[1], "after an in-place weight update")
         assert not torch.equal(again_fused[1], fused[1])
+        model.load_state_dict(before)   # in place as well: copies into the fused storage
+        assert attn.q_proj.weight.data_ptr() == attn._vx_qkv_weight.data_ptr()
+        unfused = run(False, stores[0])
+        same_as_unfused(run(True, stores[1]), "after load_state_dict")
         attn.v_proj.weight.data = attn.v_proj.weight.data.clone() * 2
         again_fused, again_unfused = run(True, stores[1]), run(False, stores[0])
         assert_bitwise(again_fused[1], again_unfused[1], "after a parameter got new storage")
-        assert attn.v_proj.weight.data_ptr() == attn._vx_qkv_weight[attn.q_proj.weight.shape[0] + attn.k_proj.weight.shape[0]].data_ptr()
+        # and back: storages of their own again, which is what safetensors' save_file insists on
+        assert unfuse_qkv_weights(model) == len(model.model.layers)
+        qkv = (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
+        assert len({w.untyped_storage().data_ptr() for w in qkv}) == 3 and attn._vx_qkv_weight is None
+        from safetensors.torch import save
+        assert len(save({k: v for k, v in model.state_dict().items() if "self_attn" in k})) > 0
+        assert_bitwise(run(True, stores[1])[1], again_unfused[1], "after unfusing")
     finally:
         hf.Qwen3MoeAttention.forward = fused_attention_forward  # what remove_qwen3_moe_patches expects to undo
         hf.Qwen3MoeDecoderLayer.forward = fused_decoder_layer_forward

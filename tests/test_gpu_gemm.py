@@ -43,6 +43,22 @@ def test_stream_and_tiled_kernels_agree_bitwise():
     assert_bf16_close(ref, O.matmul_ref(a, w.t(), bias), max_ulp=2, what="biased gemm vs oracle")
 
 
+@pytest.mark.parametrize("K", [8, 16, 24, 40])
+@pytest.mark.parametrize("M", [1, 17, 64])
+def test_streaming_and_tiled_kernels_on_contraction_depths_below_their_step(M, K):
+    # K below the streaming kernel's 32-wide step (and the tiled kernel's 64): the pieces of a step that lie past K
+    # are replaced by a re-read of the row's first piece and zeroed, so nothing outside the row is touched. The weight
+    # tensor ends where its allocation ends, the case in which a read past the last row would leave mapped memory.
+    N = 80
+    a = _gen((M, K), 40 + K)
+    w = _gen((N, K), 41 + K, scale=0.3)
+    ag, wg = a.cuda(), w.cuda()
+    ref = ops.gemm_nt_variant(ag, wg, kind=1)
+    for mt in (1, 2, 4):
+        assert_bitwise(ops.gemm_nt_variant(ag, wg, kind=0, mt=mt), ref, f"stream mt={mt} vs tiled at K={K}")
+    assert_bf16_close(ref, O.matmul_ref(a, w.t()), max_ulp=2, what=f"K={K} vs oracle")
+
+
 @pytest.mark.parametrize(
     "M,N,K,bias",
     [

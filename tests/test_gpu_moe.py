@@ -195,7 +195,7 @@ def test_wide_expert_tiles_agree_bitwise():
     T, H, I, E, k = 8300, 512, 192, 24, 4
     x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=21)
     xg, wg, sg, gg, ug, dg = (t.cuda() for t in (x, w, sel, gate, up, down))
-    assert ops.moe_tile_rows(T) == 256
+    assert ops.moe_tile_rows(T, top_k=k, num_experts=E) == 256
     full = fused_moe_forward(E, wg, sg, xg, gg, ug, dg)
     outs = {}
     for bm in (128, 256):
@@ -438,7 +438,7 @@ def test_backward_on_256_row_tiles_gives_the_gradient_bits_of_128_row_tiles(monk
         fused_moe_forward(E, leaves[0], sel.cuda(), *leaves[1:]).backward(dy)
         return [t.grad for t in leaves]
 
-    assert ops.moe_tile_rows(T) == 256
+    assert ops.moe_tile_rows(T, top_k=k, num_experts=E) == 256
     wide = grads()
     monkeypatch.setattr(ops, "moe_tile_rows", lambda *a, **kw: 128)
     for name, a, b in zip(("routing weights", "hidden states", "gate", "up", "down"), wide, grads()):
@@ -610,3 +610,35 @@ def test_packed_expert_weights_on_256_row_tiles_give_the_same_bits(T, H, I, E, k
     yp = ops.fused_moe(xg, wg, sg, gu[:, :I], gu[:, I:], dg, E, packed=(pgu, pdn))
     assert_bitwise(yp, y, "fused MoE with packed weights at a prefill size")
 
+
+
+def test_rows_of_nan_or_garbage_cannot_leave_the_expert_table():
+    # A captured bucket's padding rows reach the router with whatever the attention output buffer held (rows of a
+    # sequence without keys are never written): NaN, infinities, anything. Their expert indices must stay inside the
+    # table, out-of-range indices handed to the routing kernel are clamped, and the other rows keep their bits.
+    T, H, I, E, k = 40, 256, 128, 16, 4
+    x, _, _, gate, up, down = _inputs(T, H, I, E, k, seed=21, w_scale=0.1)
+    g = torch.Generator().manual_seed(22)
+    router_w = (torch.randn(E, H, generator=g) * 0.1).to(torch.bfloat16).cuda()
+    xg = x.cuda()
+    bad = xg.clone()
+    bad[3] = float("nan")
+    bad[17] = float("inf")
+    bad[18, ::2] = float("-inf")
+    bad[39] = torch.randint(-32768, 32767, (H,), generator=g).to(torch.int16).view(torch.bfloat16).cuda()  # arbitrary bit patterns
+    garbage = [3, 17, 18, 39]
+    clean = [t for t in range(T) if t not in garbage]
+    outs = {}
+    for name, rows in (("clean", xg), ("bad", bad)):
+        logits = ops.gemm_nt(rows, router_w)
+        for dt in (torch.bfloat16, torch.float32):
+            w, idx = ops.router_topk(logits.to(dt), k)
+            assert int(idx.min()) >= 0 and int(idx.max()) < E, f"{name} rows, {dt} logits: expert index outside [0, {E})"
+        w, idx = ops.router_topk(logits, k)
+        outs[name] = fused_moe_forward(E, w, idx, rows, gate.cuda(), up.cuda(), down.cuda())
+    assert_bitwise(outs["bad"][clean], outs["clean"][clean], "rows beside the garbage rows")
+    # indices outside the table (a caller's bug, or garbage read as integers) are clamped by the routing kernel
+    wild = torch.randint(-5, E + 5, (T, k), generator=g, dtype=torch.int32).cuda()
+    r = ops.moe_route(wild, E)
+    assert int(r.splits.sum()) == T * k and int(r.cu[-1]) == T * k
+    assert sorted(r.scatter_index.flatten().tolist()) == list(range(T * k))

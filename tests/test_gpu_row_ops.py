@@ -218,3 +218,22 @@ def test_rms_norm_backward_matches_autograd(rows, n, dtype):
     one = ops.rms_norm_backward(x[rows // 2: rows // 2 + 1].contiguous(), w, dy[rows // 2: rows // 2 + 1].contiguous(), 1e-6,
                                 hf_two_rounding=True)
     assert_bitwise(one[0], d_x[rows // 2: rows // 2 + 1], "row alone")
+
+
+@pytest.mark.parametrize("shape,dtype", [((37, 2048), torch.bfloat16), ((2, 50, 128), torch.float16), ((9, 100), torch.bfloat16),
+                                         ((4, 64), torch.float32)])
+def test_batch_invariant_rms_norm_backward_matches_autograd(shape, dtype):
+    # BatchInvariantRMSNormFunction.backward (the reference's: batch_invariant_ops.py:701-725) on vx_rms_norm_bwd in its
+    # one-rounding form; rows the kernel does not take (fp32, a length that is not a multiple of 8) use tensor operations
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(shape, generator=g).to(dtype).cuda().requires_grad_()
+    w = (1.0 + 0.2 * torch.randn(shape[-1], generator=g)).to(dtype).cuda().requires_grad_()
+    dy = torch.randn(shape, generator=g).to(dtype).cuda()
+    y = batch_invariant_rms_norm(x, w, 1e-6)
+    y.backward(dy)
+    xr, wr = x.detach().float().requires_grad_(), w.detach().float().requires_grad_()
+    (xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + 1e-6) * wr).backward(dy.float())
+    assert x.grad.dtype == dtype and w.grad.dtype == dtype and x.grad.shape == x.shape and w.grad.shape == w.shape
+    for name, got, want in (("input", x.grad, xr.grad), ("weight", w.grad, wr.grad)):
+        err, scale = (got.float() - want).abs(), float(want.abs().max())
+        assert float(err.max()) <= 2.0 ** -6 * scale, f"{name} gradient: max err {float(err.max()):.4g} vs scale {scale:.4g}"

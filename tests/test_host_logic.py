@@ -50,6 +50,54 @@ def test_hand_worked_metadata_example():
     assert m["query_start_loc"].tolist() == [0, 1, 4] and m["max_seqlen_q"] == 3
 
 
+def test_hand_worked_graph_padding_example():
+    # Literal pin of the padding restatement (vexact/inferencer/inferencer.py:306-324), worked by hand from the
+    # reference's statements: buffers zeroed / filled with -1, the step copied in, then rows of padded requests zeroed
+    # in the block table and their query_start_loc set to the real token count. Page 4, three requests, a bucket of
+    # 8 tokens and 5 sequences, table rows of 4 blocks.
+    reqs = [dict(num_computed_tokens=6, tokens_this_step=2, block_ids=[5, 2]),       # positions 4, 5 -> block 2 rows 0, 1
+            dict(num_computed_tokens=1, tokens_this_step=1, block_ids=[7]),          # position 0 -> block 7 row 0
+            dict(num_computed_tokens=9, tokens_this_step=3, block_ids=[0, 3, 9])]    # positions 6, 7, 8 -> block 3 rows 2, 3; block 9 row 0
+    want = dict(slot_mapping=[8, 9, 28, 14, 15, 36, -1, -1],       # slot_mapping.fill_(-1), [:6] copied
+                positions=[4, 5, 0, 6, 7, 8, 0, 0],                # position_ids zeroed, [:6] copied
+                context_lens=[6, 1, 9, 0, 0],                      # context_lens zeroed, [:3] copied
+                block_tables=[[5, 2, -1, -1], [7, -1, -1, -1], [0, 3, 9, -1], [0, 0, 0, 0], [0, 0, 0, 0]],
+                query_start_loc=[0, 2, 3, 6, 6, 6])                # [num_seqs + 1 : graph_num_seqs + 1] = total_tokens
+    ref = OMeta.pad_for_graph_ref(OMeta.prepare_gen_ctx_ref(reqs, 4, 4), 8, 5)
+    for k, v in want.items():
+        assert ref[k].tolist() == v, k
+    assert ref["max_seqlen_q"] == 3
+    # the product against the same literals: the Python builder + StepBuffers.load, and the one-pass native builder
+    cfg = tiny_config()
+    cfg.page_size, cfg.max_model_len = 4, 16
+    b = StepBuffers(cfg, 8, 5, "cpu")
+    assert b.load(build_step_metadata(reqs, 4, 4), np.arange(6))[:2] == (6, 3)
+    for k, v in want.items():
+        assert getattr(b, k).tolist() == v, k
+    b2 = StepBuffers(cfg, 8, 5, "cpu")
+    b2.meta_host.fill_(0x5A)
+    assert b2.load_requests(reqs, np.arange(6), 4) == (6, 3, 3)
+    for k, v in want.items():
+        assert getattr(b2, k).tolist() == v, k
+
+
+def test_hand_worked_block_allocator_restatement():
+    # The scan restatement itself (vexact/batch_invariant_ops/kv_cache_context.py:177-217) on a hand-worked sequence:
+    # min() of the free set per block, nothing allocated when the request does not fit, frees of ids that are not
+    # allocated ignored, freed ids handed out again lowest first.
+    r = OMeta.BlockAllocatorRef(6, 4)
+    assert r.allocate(9) == [0, 1, 2]                   # ceil(9 / 4) = 3 blocks
+    assert r.allocate(9, 3) == []                       # already covered
+    assert r.allocate(13, 3) == [3]                     # one more block
+    assert r.allocate(100) is None and sorted(r.free) == [4, 5] and sorted(r.allocated) == [0, 1, 2, 3]
+    r.release([1, 3, 3, 5])                             # 3 twice: second ignored; 5 was never allocated: ignored
+    assert sorted(r.free) == [1, 3, 4, 5] and sorted(r.allocated) == [0, 2]
+    assert r.allocate(8) == [1, 3]
+    assert r.allocate(4) == [4]
+    assert r.allocate(0) == [] and r.allocate(5, 2) == []
+    assert r.allocate(8) is None and sorted(r.free) == [5]   # two needed, one free: None and nothing taken
+
+
 def test_bucket_padding_rules():
     cfg = tiny_config()
     rng = np.random.default_rng(1)
@@ -301,6 +349,13 @@ def test_expert_tile_heights_and_unfilled_outputs():
     assert [ops.moe_tile_rows(t, packed_only=True) for t in (256, 448, 449, 832, 833, 2048)] == [32, 32, 64, 64, 256, 256]
     assert [ops.moe_tile_rows(t, packed=True) for t in (256, 448, 449, 832, 833, 2048)] == [32, 32, 64, 64, 256, 256]
     assert ops.moe_tile_rows(5000, wide_ok=False) == 128 and ops.moe_tile_rows(5000, wide_ok=False, packed_only=True) == 64
+    # keyed on the rows an average expert receives, not on the token count: 256 experts / top-8 reach a tile height at
+    # twice the tokens, 16 experts / top-2 at half of them (4096 tokens x 2 / 16 = 512 rows per expert = 8192 tokens of
+    # the measured 128-expert / top-8 shape)
+    assert [ops.moe_tile_rows(t, num_experts=256) for t in (896, 898, 1408, 1410, 4095, 4096)] == [32, 64, 64, 128, 128, 256]
+    assert [ops.moe_tile_rows(t, top_k=2, num_experts=16) for t in (224, 225, 352, 353, 1023, 1024)] == [32, 64, 64, 128, 128, 256]
+    assert [ops.moe_tile_rows(t, packed=True, top_k=2, num_experts=16) for t in (224, 225, 416, 417)] == [32, 64, 64, 256]
+    assert ops.moe_tile_rows(4096, top_k=1, num_experts=1) == 256 and ops.moe_tile_rows(20, top_k=1, num_experts=1) == 32
     # outputs that a kernel overwrites completely skip the NaN fill of deterministic mode and leave the switch as it was
     was = torch.are_deterministic_algorithms_enabled()
     try:
@@ -317,3 +372,31 @@ def test_expert_tile_heights_and_unfilled_outputs():
         torch.utils.deterministic.fill_uninitialized_memory = True
         torch.use_deterministic_algorithms(was)
 
+
+
+def test_gemm_piece_addresses_below_the_step_width_stay_inside_the_row():
+    # The weight-streaming GEMM loads, per lane group g = 0..3 and unrolled slot u, the 16-byte piece at element
+    # kstep0 + 32 u + 8 g of a row of K elements (K a multiple of 8); a piece past K is replaced by the row's first
+    # piece (offset -8 g from the lane's base pointer, which already points 8 g into the row) and zeroed. The tiled
+    # kernel does the same with 64-wide steps and piece index c8 = 0..7. Every address touched must lie inside the row.
+    def offsets_stream(K, U):
+        out = []
+        for kstep0 in range(0, K, 32 * U):
+            for u in range(U):
+                for g in range(4):
+                    ok = kstep0 + 32 * u + 8 * g < K
+                    out.append(8 * g + (kstep0 + 32 * u if ok else -8 * g))   # lane base + offset
+        return out
+
+    def offsets_tiled(K):
+        out = []
+        for k0 in range(0, K, 64):
+            for c8 in range(8):
+                ok = k0 + 8 * c8 < K
+                out.append(8 * c8 + (k0 if ok else -8 * c8))
+        return out
+
+    for K in (8, 16, 24, 32, 40, 56, 64, 72, 200):
+        for U in (1, 2, 4, 8):
+            assert all(0 <= o <= K - 8 for o in offsets_stream(K, U)), (K, U)
+        assert all(0 <= o <= K - 8 for o in offsets_tiled(K)), K

@@ -87,7 +87,11 @@ def mean_batch_invariant(input, dim, keepdim=False, dtype: torch.dtype | None = 
 
 
 class BatchInvariantRMSNormFunction(torch.autograd.Function):
-    """One-rounding RMSNorm forward on the HIP kernel; backward in plain torch."""
+    """One-rounding RMSNorm (the reference's ``_rms_norm_kernel`` form) on the HIP kernels, forward and backward.
+    The reference's backward is a chain of fp32 tensor operations (batch_invariant_ops.py:701-725); here
+    ``ops.rms_norm_backward`` computes the same derivative, ``d_x = inv (d - h mean(d h))`` with ``h = x inv``,
+    ``d = d_y w``, and ``d_w = sum d_y h``, in one kernel plus an ordered reduction. Rows it does not take (fp32,
+    more than 8192 entries, a length that is not a multiple of 8) go through the tensor operations."""
 
     @staticmethod
     def forward(ctx, input, weight, eps):
@@ -99,11 +103,15 @@ class BatchInvariantRMSNormFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         input, weight = ctx.saved_tensors
+        n = input.shape[-1]
+        if input.dtype in (torch.bfloat16, torch.float16) and n % 8 == 0 and n <= 8192:
+            d_x, d_w = ops.rms_norm_backward(input, weight, grad_output, ctx.eps, hf_two_rounding=False)
+            return (d_x if ctx.needs_input_grad[0] else None), (d_w.to(weight.dtype) if ctx.needs_input_grad[1] else None), None
         x = input.float()
         inv_rms = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + ctx.eps)
         normed = x * inv_rms
         g = grad_output.float()
-        grad_weight = (g * normed).reshape(-1, input.shape[-1]).sum(0).to(weight.dtype)
+        grad_weight = (g * normed).reshape(-1, n).sum(0).to(weight.dtype)
         d = g * weight.float()
         grad_input = (inv_rms * (d - normed * (d * normed).mean(-1, keepdim=True))).to(input.dtype)
         return grad_input, grad_weight, None

@@ -59,7 +59,7 @@ class FusedMoeExpertFunction(torch.autograd.Function):
         dy = grad_output.reshape(-1, H).to(torch.bfloat16)
         # 256-row expert tiles (the wide kernels) when every contraction depth is a multiple of 64
         wide_ok = H % 64 == 0 and gate_w.shape[1] % 64 == 0 and up_w.shape[1] % 64 == 0
-        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok))
+        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok, top_k=k, num_experts=E))
         # recomputed with the forward's kernels, so these are the values the forward used
         g = ops.moe_gemm(x, gate_w, r, row_src=r.sorted_token)
         u = ops.moe_gemm(x, up_w, r, row_src=r.sorted_token)
@@ -116,7 +116,7 @@ class FusedMoeStackedFunction(torch.autograd.Function):
         T, k = x.shape[0], selected_experts.reshape(x.shape[0], -1).shape[1]
         dy = grad_output.reshape(-1, H).to(torch.bfloat16)
         wide_ok = H % 64 == 0 and inter % 64 == 0
-        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok))
+        r = ops.moe_route(selected_experts.reshape(T, k), E, bm=ops.moe_tile_rows(T, wide_ok=wide_ok, top_k=k, num_experts=E))
         gu = ops.moe_gemm(x, gate_up_w, r, row_src=r.sorted_token)                 # [T k, 2I]: gate | up, as the forward
         d_hw = ops.moe_gemm_nn(dy, down_w, r, a_src=r.sorted_token)
         d_gu = ops._empty_like(gu)

@@ -44,5 +44,5 @@ def group_gemm_same_nk(
     bounds = cumsum_M.to(torch.int64)
     group_of_row = torch.searchsorted(bounds, torch.arange(rows, device=a.device, dtype=torch.int64), right=True)
     group_of_row = group_of_row.clamp_(max=G - 1).to(torch.int32).view(rows, 1)
-    routing = ops.moe_route(group_of_row, G, bm=ops.moe_tile_rows(max(1, rows // 8), wide_ok=w.shape[-1] % 64 == 0))
+    routing = ops.moe_route(group_of_row, G, bm=ops.moe_tile_rows(rows, wide_ok=w.shape[-1] % 64 == 0, top_k=1, num_experts=G))
     return ops.moe_gemm(a, w, routing)

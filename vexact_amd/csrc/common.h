@@ -150,6 +150,16 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return s;
 }
 
+// Reciprocal square root of the two RMSNorm forms. Form 0 is the reference kernel's 1 / sqrt(.) in fp32 (two
+// roundings, batch_invariant_ops.py:653-660). Form 1 is what HuggingFace's module computes with torch.rsqrt on this
+// device: measured on the GPU over 2^24 arguments, torch.rsqrt(x) has the bits of the double-precision quotient
+// 1 / sqrt(x) rounded to fp32 once, whereas fp32 1 / sqrt and the hardware's approximate rsq differ from it in 25 %
+// and 11 % of the arguments. A fused kernel in that form must give the bits of the module's own tensor operations.
+// Once per row and thread, so the double-precision operations do not show in the run time.
+__device__ __forceinline__ float rms_inv(float mean_sq_eps, int mode) {
+  return mode == 0 ? 1.0f / sqrtf(mean_sq_eps) : (float)(1.0 / sqrt((double)mean_sq_eps));
+}
+
 static inline int launch_status() {
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? VX_OK : VX_ERR_LAUNCH;

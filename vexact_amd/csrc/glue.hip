@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(
   float tot = acc;
 #pragma unroll
   for (int o = 16; o > 0; o >>= 1) tot += __shfl_xor(tot, o, 64);
-  const float inv = 1.0f / sqrtf(tot / (float)D + eps);
+  const float inv = rms_inv(tot / (float)D + eps, 1);  // HuggingFace's q / k norm
   float y[4], cs[4], sn[4];
   if (own) {
     const float wf[4] = {bf16lo(wr.x), bf16hi(wr.x), bf16lo(wr.y), bf16hi(wr.y)};

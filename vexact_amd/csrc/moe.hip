@@ -74,7 +74,8 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const void* __restrict
       if (lane + 64 * i == bi) x[i] = -INFINITY;
     const float p = bp / s;
     tot += p;
-    if (lane == j) { wsel = p; isel = bi; }
+    // a row of NaNs wins no comparison: it still gets an expert index inside the table
+    if (lane == j) { wsel = p; isel = min(bi, E - 1); }
   }
   if (lane < k) {
     const float w = renorm ? wsel / tot : wsel;
@@ -462,7 +463,7 @@ __global__ __launch_bounds__(256) void moe_gather_vec_kernel(const bf16_t* __res
   }
   if (!h) return;
   const float tot = block_sum<4>(ss, red);
-  const float inv = 1.0f / sqrtf(tot / (float)H + eps);
+  const float inv = rms_inv(tot / (float)H + eps, mode);
 #pragma unroll
   for (int j = 0; j < MAXV; j++) {
     const int c = 4 * (tid + 256 * j);

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
   if constexpr (G == 64) tot = wave_sum(acc);
   else tot = block_sum<4>(acc, red);
   if (!live) return;
-  const float inv = 1.0f / sqrtf(tot / (float)n + eps);
+  const float inv = rms_inv(tot / (float)n + eps, mode);
   typename E::T* yr = y + row * ys;
   for (int v = t; v * 4 < n; v += G) {
 #pragma unroll
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256) void rms_norm_bf16v_kernel(const bf16_t* x, co
   if constexpr (G == 64) tot = wave_sum(acc);
   else tot = block_sum<4>(acc, red);
   if (!live) return;
-  const float inv = 1.0f / sqrtf(tot / (float)n + eps);
+  const float inv = rms_inv(tot / (float)n + eps, mode);
 #pragma unroll
   for (int j = 0; j < MAXV; j++) {
     const int c = 4 * (t + G * j);
@@ -465,7 +465,7 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const typename Elem<D
     }
 #pragma unroll
     for (int o = G / 2; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o, 64);
-    const float inv = 1.0f / sqrtf(ssq / (float)n + eps);
+    const float inv = rms_inv(ssq / (float)n + eps, mode);
     float dot = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXV; i++)
@@ -535,7 +535,7 @@ __global__ __launch_bounds__(512) void rms_norm_bwd_finish_kernel(const float* _
 // output: lse_i = logits[i, label_i] - out[i], d_logits[i, j] = d_out[i] ((j == label_i) - exp(logits[i, j] - lse_i)).
 // Elementwise over the row; d_logits may be the logits' own memory (every element is read before it is written).
 template <int DT>
-__global__ __launch_bounds__(256) void logprob_bwd_kernel(const typename Elem<DT>::T* __restrict__ logits,
+__global__ __launch_bounds__(256) void logprob_bwd_kernel(const typename Elem<DT>::T* logits,  // may alias d_logits
                                                           const int64_t* __restrict__ labels,
                                                           const float* __restrict__ out, const float* __restrict__ d_out,
                                                           typename Elem<DT>::T* d_logits, int n, int64_t x_stride,
@@ -771,7 +771,16 @@ int vx_logprobs_bwd(const void* logits, const int64_t* labels, const float* out,
   if (rows > 65535) return VX_ERR_UNSUPPORTED;
   // Every workgroup must read the label's logit before any workgroup of the row overwrites it when the gradient goes
   // into the logits' memory: one workgroup per row then; else enough workgroups per row to fill the chip
+  // "In place" is any overlap of the two ranges with equal pointers and strides; every other overlap is rejected
+  // (a row's workgroups would read logits that another row's have already overwritten).
   const bool inplace = d_logits == logits;
+  {
+    const int64_t es = dtype == DT_F32 ? 4 : 2;
+    const uintptr_t x0 = (uintptr_t)logits, x1 = x0 + (uintptr_t)(((rows - 1) * x_stride + n) * es);
+    const uintptr_t d0 = (uintptr_t)d_logits, d1 = d0 + (uintptr_t)(((rows - 1) * d_stride + n) * es);
+    const bool overlap = x0 < d1 && d0 < x1;
+    if (overlap && !(inplace && x_stride == d_stride)) return VX_ERR_ARG;
+  }
   const unsigned gx = inplace ? 1u : (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 2047) / 2048, 2048 / rows + 1));
   const dim3 grid(gx, (unsigned)rows);
   switch (dtype) {

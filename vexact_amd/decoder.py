@@ -295,7 +295,7 @@ class StepBuffers:
         self.hw = z(T * k, cfg.moe_intermediate, dtype=bf)
         self.eo = z(T * k, H, dtype=bf)
         self.bm = ops.moe_tile_rows(T, wide_ok=(cfg.hidden_size % 64 == 0 and cfg.moe_intermediate % 64 == 0),
-                                    packed_only=packed_only, packed=packed)
+                                    packed_only=packed_only, packed=packed, top_k=k, num_experts=cfg.num_experts)
         from . import _lib
 
         lib = _lib.load()

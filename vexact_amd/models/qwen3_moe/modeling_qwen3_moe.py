@@ -168,9 +168,8 @@ def invalidate_packed_experts(model: nn.Module) -> int:
 
 
 class RmsNormFunction(torch.autograd.Function):
-    """The fused RMSNorm with a backward, so that a trainer's forward runs the kernel the rollout ran (the same
-    bits, which the tensor-operation forward does not give in every element: its ``torch.rsqrt`` on the GPU and the
-    kernel's ``1 / sqrt`` differ by an fp32 ulp now and then). Backward: the RMSNorm derivative,
+    """The fused RMSNorm with a backward, so that a trainer's forward runs the kernel the rollout ran (which has
+    the bits of the tensor-operation forward under batch-invariant mode). Backward: the RMSNorm derivative,
     ``d_x = inv (d_h - h mean(d_h h))`` with ``h = x inv``, ``d_h = d_y w``, ``d_w = sum d_y r(h)``, in fp32: one
     kernel plus a small reduction (``ops.rms_norm_backward``), tensor operations for rows it does not take."""
 
@@ -204,10 +203,11 @@ def fused_rms_norm_forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
     """``Qwen3MoeRMSNorm.forward`` as one kernel. HuggingFace's forward (cast to fp32, ``pow(2).mean(-1)``, ``rsqrt``,
     two multiplies and two casts: eleven launches under batch-invariant mode) rounds ``x * rsqrt(var + eps)`` to
     the input dtype and then multiplies by the weight; ``ops.rms_norm(..., hf_two_rounding=True)`` keeps both
-    roundings and the batch-invariant mean's summation order. Its ``1 / sqrt`` is the CPU's ``torch.rsqrt``; the
-    GPU's differs from it by an fp32 ulp now and then, which shows in about one output element in 10^5. With
-    autograd the same kernel runs (``RmsNormFunction``), so rollout and trainer agree bit for bit. Outside
-    batch-invariant mode, off the GPU or with a weight of another dtype the original forward runs."""
+    roundings, the batch-invariant mean's summation order and the device's ``rsqrt`` (the operation ``torch.rsqrt``
+    runs on the GPU), so the result has the bits of the original forward under batch-invariant mode (tested on
+    rows of very different magnitudes). With autograd the same kernel runs (``RmsNormFunction``). Outside
+    batch-invariant mode, off the GPU or with a weight of another dtype the original forward runs: the same
+    bits again, hence a rollout and a trainer agree whether or not each of them takes the fused path."""
     from ...batch_invariant_ops import is_batch_invariant_mode_enabled
 
     w = self.weight
@@ -272,45 +272,77 @@ def fused_apply_rotary_pos_emb(q, k, cos, sin, *args, unsqueeze_dim: int = 1, **
 _ORIGINAL_ATTN = None  # Qwen3MoeAttention.forward while the fused form is patched in
 
 
-def _fused_qkv_weight(attn) -> Optional[torch.Tensor]:
-    """``[q_proj.weight; k_proj.weight; v_proj.weight]`` as one tensor, made once per module: the three
-    parameters are then re-pointed at row ranges of it, so there is still one copy of the weights in memory and
-    an in-place write to a parameter (``param.data.copy_``, what the reference's weight sync does,
-    vexact/inferencer/model_loader.py:113) lands in the fused tensor. A parameter that has been given new
-    storage since is noticed by its address and the fused tensor is rebuilt. Returns None when it would have to
-    be built while a graph is being captured (its memory would belong to the graph's pool): the caller then runs
-    the unfused forward, as it does for every other case it does not take."""
-    ws = (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
-    fused = getattr(attn, "_vx_qkv_weight", None)
-    if fused is not None:
-        row = 0
-        for w in ws:
-            if w.data_ptr() != fused[row].data_ptr() or w.dtype != fused.dtype:
-                fused = None
-                break
-            row += w.shape[0]
-    if fused is None and torch.cuda.is_current_stream_capturing():
-        return None
-    if fused is None:
-        # outside inference mode: tensors made inside it could never take part in autograd again, and these
-        # become the parameters' storage
-        with torch.inference_mode(False), torch.no_grad():
+def _qkv_modules(model):
+    for m in model.modules():
+        if all(hasattr(m, n) and hasattr(getattr(m, n), "weight") for n in ("q_proj", "k_proj", "v_proj")):
+            yield m
+
+
+def fuse_qkv_weights(model) -> int:
+    """Load-time step, optional: give every attention module of ``model`` ONE tensor
+    ``[q_proj.weight; k_proj.weight; v_proj.weight]`` and re-point the three parameters at row ranges of it. The
+    fused attention forward then runs one projection instead of three (same bits: a row of a product depends on its
+    own weight row only). There is still one copy of the weights in memory, and an in-place write to a parameter
+    (``param.data.copy_``, what the reference's weight sync does, vexact/inferencer/model_loader.py:113) lands in the
+    fused tensor. What changes for the caller, and why this is a call of its own and not a side effect of a forward:
+    the three parameters share one storage afterwards, so ``safetensors.save_file(model.state_dict())`` refuses them
+    (``save_model`` or ``unfuse_qkv_weights`` first), and anything that captured the old storages (exported IPC
+    handles, flat-parameter or bucketed weight-sync buffers) no longer aliases the parameters: call this before
+    such captures are made. Call it outside graph capture. Returns the number of modules fused."""
+    n = 0
+    with torch.inference_mode(False), torch.no_grad():  # these tensors become parameter storage: keep them out of inference mode
+        for attn in _qkv_modules(model):
+            ws = (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight)
+            if len({w.dtype for w in ws}) != 1 or len({w.device for w in ws}) != 1 or len({w.shape[1] for w in ws}) != 1:
+                continue
             fused = torch.cat([w.detach() for w in ws], dim=0)
             row = 0
             for w in ws:
                 w.data = fused[row:row + w.shape[0]]
                 row += w.shape[0]
-        attn._vx_qkv_weight = fused
-    return fused
+            attn._vx_qkv_weight = fused
+            n += 1
+    return n
+
+
+def unfuse_qkv_weights(model) -> int:
+    """Undo ``fuse_qkv_weights``: every q / k / v parameter gets storage of its own again (a copy)."""
+    n = 0
+    with torch.inference_mode(False), torch.no_grad():
+        for attn in _qkv_modules(model):
+            if getattr(attn, "_vx_qkv_weight", None) is None:
+                continue
+            for proj in (attn.q_proj, attn.k_proj, attn.v_proj):
+                proj.weight.data = proj.weight.data.clone()
+            attn._vx_qkv_weight = None
+            n += 1
+    return n
+
+
+def _fused_qkv_weight(attn) -> Optional[torch.Tensor]:
+    """The tensor ``fuse_qkv_weights`` made for this module, if the three parameters still are its row ranges (a
+    parameter that has been given new storage since is noticed by its address); else None. Never builds one."""
+    fused = getattr(attn, "_vx_qkv_weight", None)
+    if fused is None:
+        return None
+    row = 0
+    for w in (attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight):
+        if w.data_ptr() != fused[row].data_ptr() or w.dtype != fused.dtype or w.stride(0) != fused.stride(0):
+            return None
+        row += w.shape[0]
+    return fused if row == fused.shape[0] else None
 
 
 def fused_attention_forward(self, hidden_states, position_embeddings, attention_mask=None, past_key_values=None, **kwargs):
-    """``Qwen3MoeAttention.forward`` for a step over the paged cache as four launches in front of the output
-    projection instead of twelve: one q/k/v projection on the concatenated weight, one kernel for the per-head
-    q / k RMSNorm, the rotary embedding and the cache write (``ops.qk_norm_rope_store``; it computes what
-    ``q_norm`` / ``k_norm``, ``apply_rotary_pos_emb`` and ``store_kvcache`` compute, rounding for rounding), the
-    attention kernel, then ``o_proj``. A row of a product depends on its own weight row only, so the concatenated
-    projection gives the three projections' bits. Taken only under batch-invariant mode with a paged context,
+    """``Qwen3MoeAttention.forward`` for a step over the paged cache as a few launches in front of the output
+    projection instead of twelve: the q / k / v projections written side by side into one buffer (one launch on the
+    concatenated weight when ``fuse_qkv_weights`` has been called on the model, else three; the parameters are never
+    touched here), one kernel for the per-head q / k RMSNorm, the rotary embedding and the cache write
+    (``ops.qk_norm_rope_store``; it computes what ``q_norm`` / ``k_norm``, ``apply_rotary_pos_emb`` and
+    ``store_kvcache`` compute, rounding for rounding), the attention kernel, then ``o_proj``. A row of a product
+    depends on its own weight row only, so the concatenated projection gives the three projections' bits. The cache
+    layer is ``kwargs["layer_idx"]`` if given, else the module's, as in the registered attention function.
+    Taken only under batch-invariant mode with a paged context,
     the registered attention function of this package, bf16 tensors of batch 1 and no autograd, bias, HuggingFace
     cache object or sliding window; anything else runs the original forward."""
     from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
@@ -332,23 +364,33 @@ def fused_attention_forward(self, hidden_states, position_embeddings, attention_
         and cos.shape == (1, hidden_states.shape[1], D) and cos.is_contiguous() and sin.is_contiguous()
         and ALL_ATTENTION_FUNCTIONS.get(self.config._attn_implementation) is flash_attention_forward
     )
-    w_qkv = _fused_qkv_weight(self) if fits else None
-    if w_qkv is None:
+    if not fits:
         return _ORIGINAL_ATTN(self, hidden_states, position_embeddings, attention_mask, past_key_values, **kwargs)
+    layer_idx = int(kwargs["layer_idx"]) if "layer_idx" in kwargs else self.layer_idx
     T = hidden_states.shape[1]
     Hq, Hkv = self.q_proj.weight.shape[0] // D, self.k_proj.weight.shape[0] // D
     x = hidden_states[0]
     if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
         x = x.contiguous()
-    qkv = ops.gemm_nt(x, w_qkv)
+    w_qkv = _fused_qkv_weight(self)
+    if w_qkv is not None:
+        qkv = ops.gemm_nt(x, w_qkv)
+    else:  # three projections into column ranges of one buffer
+        qkv = ops._empty((T, (Hq + 2 * Hkv) * D), dtype=torch.bfloat16, device=x.device)
+        col = 0
+        for proj in (self.q_proj, self.k_proj, self.v_proj):
+            n = proj.weight.shape[0]
+            w = proj.weight if proj.weight.stride(1) == 1 and proj.weight.stride(0) % 8 == 0 else proj.weight.contiguous()
+            ops.gemm_nt(x, w, out=qkv[:, col:col + n])
+            col += n
     q = ops._empty((T, Hq, D), dtype=torch.bfloat16, device=x.device)
     ops.qk_norm_rope_store(qkv, self.q_norm.weight, self.k_norm.weight, cos[0], sin[0], None, ctx.slot_mapping, q,
-                           ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx], Hq, Hkv, D,
+                           ctx.key_cache[layer_idx], ctx.value_cache[layer_idx], Hq, Hkv, D,
                            self.q_norm.variance_epsilon)
     # The kernel writes every row that belongs to a sequence with at least one key; what it leaves alone here are the
     # padding rows of a captured bucket, whose values nobody reads, so the output skips the NaN fill that
     # torch.empty adds under deterministic algorithms (one more launch per layer).
-    k_cache, v_cache = ctx.key_cache[self.layer_idx], ctx.value_cache[self.layer_idx]
+    k_cache, v_cache = ctx.key_cache[layer_idx], ctx.value_cache[layer_idx]
     if not (ctx.query_start_loc.dtype == ctx.context_lens.dtype == ctx.block_tables.dtype == torch.int32
             and ctx.query_start_loc.is_contiguous() and ctx.context_lens.is_contiguous() and ctx.block_tables.stride(-1) == 1
             and ctx.query_start_loc.is_cuda and ctx.context_lens.is_cuda and ctx.block_tables.is_cuda

@@ -8,6 +8,7 @@ missing the call raises.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import Optional
 
 import torch
@@ -30,19 +31,28 @@ def _need_gpu(name: str, t: torch.Tensor) -> None:
         raise ValueError(f"{name} must be a CUDA tensor")
 
 
+_EMPTY_LOCK = threading.Lock()
+
+
 def _empty(*size, **kw) -> torch.Tensor:
     """``torch.empty`` for a tensor that the kernel about to be launched writes completely. Under
     ``torch.use_deterministic_algorithms(True)`` (which ``enable_batch_invariant_mode`` turns on, as the
     reference's does) ``torch.empty`` fills what it returns with NaN, one more kernel in front of every op here
     (about 3 us each, some twenty per decoder layer); that fill is skipped for these tensors, whose every
-    element is overwritten anyway. Attention outputs keep it: rows of a sequence without any key stay unwritten."""
+    element is overwritten anyway. Attention outputs keep it: rows of a sequence without any key stay unwritten.
+    The switch is a process-wide flag of torch: the lock keeps two threads of this package from restoring it in
+    the wrong order, and the previous value (not ``True``) is what comes back. A ``torch.empty`` that another
+    thread's own code issues inside that window still loses its fill; the reference runs one generation thread per
+    process (vexact/worker/worker.py:48), which is the arrangement this is meant for."""
     det = torch.utils.deterministic
     if torch.are_deterministic_algorithms_enabled() and det.fill_uninitialized_memory:
-        det.fill_uninitialized_memory = False
-        try:
-            return torch.empty(*size, **kw)
-        finally:
-            det.fill_uninitialized_memory = True
+        with _EMPTY_LOCK:
+            previous = det.fill_uninitialized_memory
+            det.fill_uninitialized_memory = False
+            try:
+                return torch.empty(*size, **kw)
+            finally:
+                det.fill_uninitialized_memory = previous
     return torch.empty(*size, **kw)
 
 
@@ -731,26 +741,31 @@ def router_topk_backward(logits: torch.Tensor, selected: torch.Tensor, d_weights
     return out
 
 
-def moe_tile_rows(num_tokens: int, wide_ok: bool = True, packed_only: bool = False, packed: bool = False) -> int:
-    """Rows per expert tile, chosen from the token count only (any choice gives the same bits).
+def moe_tile_rows(num_tokens: int, wide_ok: bool = True, packed_only: bool = False, packed: bool = False,
+                  top_k: int = 8, num_experts: int = 128) -> int:
+    """Rows per expert tile (any choice gives the same bits), chosen from the average number of rows an expert
+    receives, ``num_tokens * top_k / num_experts``: that, not the token count, decides how full a tile is. The
+    crossovers were measured at 128 experts / top-8 and are stated below as token counts of that shape (16 tokens
+    per average expert row); other shapes are mapped onto it.
     ``wide_ok``: both GEMM depths are multiples of 64, which the 256-row kernel needs.
     ``packed``: fragment-order weights are at hand; ``packed_only``: nothing else is, and the 128-row kernel does
     not read them. With fragment-order weights the 256-row kernel overtakes the streaming kernel early (128 experts,
     top-8, measured per block: 448 tokens 256 us on 32-row tiles against 269 on 64-row ones; 768 tokens 309 on 64-row
     tiles against 314 on 256-row ones; 1024 tokens 365 against 311; 1536 tokens 318 against 353 on the 128-row kernel)."""
+    eq = (int(num_tokens) * max(1, int(top_k)) * 16) // max(1, int(num_experts))  # token count of the measured shape
     if packed or packed_only:
-        if num_tokens <= 448:
+        if eq <= 448:
             return 32
-        if num_tokens <= 832 or not wide_ok:
+        if eq <= 832 or not wide_ok:
             return 64
         return 256
     # [E, N, K] tensors only (same block): 384 tokens 269 us on 32-row tiles against 297 on 64-row ones, 512 tokens
     # 311 / 306, 768 tokens 343 on 64-row tiles against 326 on 128-row ones, 1024 tokens 410 / 332
-    if num_tokens <= 448:
+    if eq <= 448:
         return 32
-    if num_tokens <= 704:
+    if eq <= 704:
         return 64
-    if num_tokens < 2048 or not wide_ok:
+    if eq < 2048 or not wide_ok:
         return 128
     return 256
 
@@ -770,7 +785,7 @@ def moe_route(selected_experts: torch.Tensor, num_experts: int, bm: Optional[int
     assert selected_experts.dtype in (torch.int32, torch.int64)
     idx = selected_experts.contiguous()
     T, k = idx.shape
-    bm = bm or moe_tile_rows(T)
+    bm = bm or moe_tile_rows(T, top_k=k, num_experts=num_experts)
     lib = _lib.load()
     max_tiles = lib.vx_moe_max_tiles(T * k, num_experts, bm)
     dev = idx.device
@@ -1077,7 +1092,7 @@ def fused_moe(
     H_, I_ = gate_w.shape[-1], down_w.shape[-1]
     r = moe_route(selected_experts, num_experts,
                   bm=moe_tile_rows(selected_experts.shape[0], wide_ok=(H_ % 64 == 0 and I_ % 64 == 0),
-                                   packed=packed is not None))
+                                   packed=packed is not None, top_k=k, num_experts=num_experts))
     if packed is not None and (r.bm <= 64 or r.bm == 256):
         pgu, pdn = packed
         assert pgu.rows_n == 2 * I_ and pgu.K == H_ and pdn.rows_n == down_w.shape[1] and pdn.K == I_
