@@ -48,6 +48,7 @@ def parse():
                     help="steps of the advancing decode loop (host metadata + copy + replay + token feedback); 0 = skip")
     ap.add_argument("--no-configs", action="store_true", help="skip the reference's other configurations (C1-C4, prefill GEMM)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dropin", action="store_true", help="skip the HuggingFace drop-in decode step (dropin_ms_per_step keys)")
     ap.add_argument("--no-packed-experts", action="store_true",
                     help="every step reads the [E, N, K] expert tensors instead of their fragment-order copies")
     ap.add_argument("--keep-unpacked-experts", action="store_true",
@@ -223,6 +224,21 @@ def main():
         print("bench.py: this build runs on exactly one GPU (all pipeline stages collapsed onto one MI355X); "
               "--gpus must be 1", file=sys.stderr)
         sys.exit(2)
+    out = headline(args)  # everything the built-in decoder holds on the GPU dies with that call's frame
+    if not args.no_dropin and out["config"]["full_model"]:
+        # What a caller of the reference gets by switching imports (a HuggingFace Qwen3MoeForCausalLM through the
+        # registered attention function, the patched modules and batch-invariant mode): the same decode step, captured
+        # in a graph. It needs the memory the built-in decoder held.
+        import gc
+
+        import torch
+        gc.collect()
+        torch.cuda.empty_cache()
+        out.update(dropin_step(args.batch))
+    print(json.dumps(out), flush=True)
+
+
+def headline(args):
     import torch
 
     from vexact_amd import _build, _lib, ops
@@ -438,7 +454,21 @@ def main():
         out["configs"], out["roofline_mfma"] = other_configs()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, w, dec, dmeta, first_tokens, B, args.cpu_seconds)
-    print(json.dumps(out), flush=True)
+    return out
+
+
+def dropin_step(batch):
+    """``dropin_ms_per_step`` (the reference's cache layout, graph captured with ``max_seqlen_q = 1``),
+    ``dropin_ms_per_step_reference_capture`` (captured the way the reference's CudaGraphManager does, with
+    ``max_seqlen_q`` = the bucket's tokens) and ``dropin_ms_per_step_head_major`` (``KVCacheStore(head_major=True)``)."""
+    import kernel_bench
+
+    rows = kernel_bench.dropin_decode(kernel_bench.parse(["--what", "dropin", "--batch", str(batch)]), quiet=True)
+    out = {"dropin": rows}
+    for r in rows:
+        key = "dropin_ms_per_step" + ("_head_major" if r["head_major"] else "_reference_capture" if r["max_seqlen_q"] != 1 else "")
+        out[key] = r["ms_per_step"]
+    return out
 
 
 def other_configs():

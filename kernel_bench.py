@@ -240,18 +240,21 @@ def run(a, quiet: bool = False) -> list:
         del wg, wu, wd
     if "prefill" in what:
         # MoE expert GEMMs over a prefill chunk (256-row expert tiles)
-        for T in (8192, 32768):
+        for T in (4096, 8192, 32768):
             x = rnd(T, H, std=1.0)
             logits = torch.randn(T, E, generator=g, device=dev)
             w, idx = ops.router_topk(logits, k, index_dtype=torch.int32)
-            r = ops.moe_route(idx, E, bm=ops.moe_tile_rows(T))
+            r = ops.moe_route(idx, E, bm=256)
+            rows = r.tile_rows[r.tile_group >= 0]
+            tiles_info = f"{int(rows.numel())} row tiles, {int((rows <= 64).sum())} of at most 64 rows, {int((rows == 256).sum())} full"
             gu = rnd(E, 2 * I, H)
             dn = rnd(E, H, I)
             hw = torch.empty(T * k, I, dtype=torch.bfloat16, device=dev)
             eo = torch.empty(T * k, H, dtype=torch.bfloat16, device=dev)
-            report(f"prefill moe route T={T}", timeit(lambda li: ops.moe_route(idx, E, bm=ops.moe_tile_rows(T)), n_layers=2), T * k * 16)
-            report(f"prefill moe route T={T}, one workgroup", timeit(lambda li: ops.moe_route(idx, E, bm=ops.moe_tile_rows(T), chunked=False), n_layers=2), T * k * 16)
-            report(f"prefill moe gate/up T={T}",
+            if T >= 8192:
+                report(f"prefill moe route T={T}", timeit(lambda li: ops.moe_route(idx, E, bm=256), n_layers=2), T * k * 16)
+                report(f"prefill moe route T={T}, one workgroup", timeit(lambda li: ops.moe_route(idx, E, bm=256, chunked=False), n_layers=2), T * k * 16)
+            report(f"prefill moe gate/up T={T} ({tiles_info})",
                    timeit(lambda li: ops.moe_gemm(x, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=w,
                                                   row_scale_idx=r.sorted_flat, out=hw), n_layers=2),
                    flops=2 * T * k * 2 * I * H)
@@ -411,7 +414,7 @@ def run(a, quiet: bool = False) -> list:
                 ww = (torch.randn(4096, 4096, generator=g, device=dev) * 0.02).to(dt)
                 report(f"{nm} gemm M={M} N=4096 K=4096", timeit(lambda li: ops.matmul(xx, ww.t()), n_layers=2), flops=2 * M * 4096 * 4096)
     if "dropin" in what:
-        results.extend(dropin_decode(a, quiet))
+        results.extend(dropin_decode(a, quiet, layouts=(True,) if a.dropin_head_major else None))
     if "trainlayer" in what:
         results.extend(dropin_train_layers(quiet))
     if "copy" in what:
@@ -422,7 +425,7 @@ def run(a, quiet: bool = False) -> list:
     return results
 
 
-def dropin_decode(a, quiet: bool = False) -> list:
+def dropin_decode(a, quiet: bool = False, layouts=None) -> list:
     """What a caller of the reference gets by switching imports: a HuggingFace ``Qwen3MoeForCausalLM`` of the
     30B-A3B shape (random weights, built on the GPU) behind the registered attention function, the patched MoE
     block and batch-invariant mode, one decode step of ``--batch`` sequences (contexts U[256, 2048], page 16)
@@ -437,7 +440,7 @@ def dropin_decode(a, quiet: bool = False) -> list:
 
     from vexact_amd.batch_invariant_ops import flash_attention_forward, set_batch_invariant_mode
     from vexact_amd.batch_invariant_ops.kv_cache_context import KVCacheStore, clear_kv_cache_context, set_kv_cache_context
-    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, fuse_qkv_weights
+    from vexact_amd.models.qwen3_moe import apply_qwen3_moe_patches, fuse_qkv_weights, remove_qwen3_moe_patches
 
     say = (lambda *x, **k: None) if quiet else print
     B, page = a.batch, a.page
@@ -470,10 +473,6 @@ def dropin_decode(a, quiet: bool = False) -> list:
     lens = rng.integers(256, 2049, size=B)
     pages = [(int(n) + 2 + page - 1) // page for n in lens]
     pool = sum(pages) + 8
-    store = KVCacheStore(cfg, types.SimpleNamespace(page_size=page, max_cache_blocks=pool), torch.device("cuda"),
-                         head_major=a.dropin_head_major)
-    for t in list(store.key_cache.values()) + list(store.value_cache.values()):
-        t.normal_(0, 1)
     perm, bt, o = rng.permutation(pool), np.zeros((B, max(pages)), np.int32), 0
     for i, pg in enumerate(pages):
         bt[i, :pg] = perm[o:o + pg]
@@ -490,28 +489,43 @@ def dropin_decode(a, quiet: bool = False) -> list:
         return model.lm_head(out.last_hidden_state)
 
     res = []
-    for msq, how in ((1, "max_seqlen_q = 1"), (B, "max_seqlen_q = bucket tokens")):
-        set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache, block_tables=bt_d,
-                             context_lens=ctx, slot_mapping=slot, query_start_loc=qsl, max_seqlen_q=msq)
-        try:
-            with torch.inference_mode(), set_batch_invariant_mode(True):
-                forward()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
+    layouts = (False, True) if layouts is None else layouts
+    for head_major in layouts:
+        store = KVCacheStore(cfg, types.SimpleNamespace(page_size=page, max_cache_blocks=pool), torch.device("cuda"),
+                             head_major=head_major)
+        for t in list(store.key_cache.values()) + list(store.value_cache.values()):
+            t.normal_(0, 1)
+        where = "KVCacheStore(head_major=True)" if head_major else "the reference's cache layout"
+        # the reference's CudaGraphManager captures with max_seqlen_q = the bucket's tokens (cudagraph_utils.py:163)
+        for msq, how in ((1, "max_seqlen_q = 1"), (B, "max_seqlen_q = bucket tokens"))[: 1 if head_major else 2]:
+            set_kv_cache_context(is_paged_attn=True, key_cache=store.key_cache, value_cache=store.value_cache, block_tables=bt_d,
+                                 context_lens=ctx, slot_mapping=slot, query_start_loc=qsl, max_seqlen_q=msq)
+            try:
+                with torch.inference_mode(), set_batch_invariant_mode(True):
                     forward()
-                for _ in range(3):
-                    graph.replay()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(10):
-                    graph.replay()
-                e1.record()
-                torch.cuda.synchronize()
-        finally:
-            clear_kv_cache_context()
-        ms = e0.elapsed_time(e1) / 10
-        say(f"HF Qwen3MoeForCausalLM drop-in decode, batch {B}, {how}: {ms:.2f} ms/step = {B / ms * 1e3:.0f} tok/s", flush=True)
-        res.append({"name": f"HF drop-in decode step, batch {B}, {how}", "us": round(ms * 1e3, 1), "tok_s": round(B / ms * 1e3)})
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        forward()
+                    for _ in range(3):
+                        graph.replay()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(10):
+                        graph.replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+            finally:
+                clear_kv_cache_context()
+            ms = e0.elapsed_time(e1) / 10
+            say(f"HF Qwen3MoeForCausalLM drop-in decode, batch {B}, {where}, {how}: {ms:.2f} ms/step = {B / ms * 1e3:.0f} tok/s", flush=True)
+            res.append({"name": f"HF drop-in decode step, batch {B}, {where}, {how}", "us": round(ms * 1e3, 1),
+                        "ms_per_step": round(ms, 3), "tok_s": round(B / ms * 1e3), "head_major": head_major, "max_seqlen_q": msq})
+            del graph
+        del store
+        torch.cuda.empty_cache()
+    del model
+    torch.cuda.empty_cache()
+    remove_qwen3_moe_patches()
     return res
 
 
