@@ -58,7 +58,7 @@ __device__ __forceinline__ void bwl_issue_rows(const bf16_t* base, int64_t row_s
     const int piece = (lane & 15) ^ bwl_swz(row);
     const uint32_t voff = (uint32_t)(min(first_row + row, last_row) - r0) * (uint32_t)(row_stride * 2) + 16u * (uint32_t)piece;
     const uint32_t dst = lds_arr + (RPW * wave + 4 * j) * 256;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(voff), "s"(sb) : "memory", "m0");
+    lds_load16_sv(dst, voff, (const void*)sb);
   }
 }
 // A operand of a score product: row 16 tt + r16 of the array, dims 32 s + 8 g .. +8
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dkv_lds_kernel(AttnBwdParams
     if (wave < 2) {  // 64 lse values (wavefront 0) and 64 delta values (wavefront 1), one dword per lane
       const float* src = (wave == 0 ? p.lse : p.delta) + (int64_t)(q0 + min(ib + lane, qlen - 1)) * p.Hq + h;
       const uint32_t dst = sb + 2 * BWL_ARR + wave * 256;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+      lds_load4_v(dst, src);
     }
   };
   if (nsteps > 0) issue_step(0, 0);

@@ -989,10 +989,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
         const bool ok = kb + row < kv_len;
         const bf16_t* kp = src.krow(tl, kb, ld_tt, ok ? (row & 15) : 0) + 8 * ((lane & 15) ^ (row & 15));
         const bf16_t* vp = src.vrow(tl, kb, ld_tt, ok ? (row & 15) : 0) + 8 * ((lane & 15) ^ ((row & 7) << 1));
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                     :: "s"(dst0 + 4 * j * 256), "v"(kp) : "memory", "m0");
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                     :: "s"(dst0 + 4 * j * 256 + ATT_BLOCK * 256), "v"(vp) : "memory", "m0");
+        lds_load16_v(dst0 + 4 * j * 256, kp);
+        lds_load16_v(dst0 + 4 * j * 256 + ATT_BLOCK * 256, vp);
       }
     } else {
       // first key of the wavefront's tile, clamped like every key address: a tile that starts past the end
@@ -1032,10 +1030,8 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
         const uint32_t dk = (uint32_t)min(row_in[j], last_in);  // 0 .. 15
         const uint32_t koff = dk * (uint32_t)(src.skp * 2) + kslot[j];
         const uint32_t voff = dk * (uint32_t)(src.svp * 2) + vslot[j];
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(dst0 + 4 * j * 256), "v"(koff), "s"(ksb) : "memory", "m0");
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(dst0 + 4 * j * 256 + ATT_BLOCK * 256), "v"(voff), "s"(vsb) : "memory", "m0");
+        lds_load16_sv(dst0 + 4 * j * 256, koff, (const void*)ksb);
+        lds_load16_sv(dst0 + 4 * j * 256 + ATT_BLOCK * 256, voff, (const void*)vsb);
       }
     }
   };

@@ -150,6 +150,29 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return s;
 }
 
+// Direct-to-LDS loads (global memory -> LDS without staging registers). The LDS byte address of lane 0 goes into m0, the
+// 64 lanes' pieces land behind it in lane order. Written as asm, not through __builtin_amdgcn_global_load_lds, on
+// purpose: told that the instruction writes LDS, the compiler waits for it (vmcnt(0)) before the next LDS read it
+// schedules, while the kernels keep several steps of these loads in flight and wait explicitly before the barrier that
+// precedes their first use. Each statement sets m0 and consumes it in its own text and names m0 as clobbered; nothing
+// else in these kernels lives in m0 (no indexed register arrays, no other LDS-DMA or message instructions), so the
+// compiler's warning that a clobber of a reserved register is not saved and restored for the asm's sake does not bite.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+// 16 bytes per lane from (wave-uniform base in scalar registers) + (32-bit byte offset per lane)
+__device__ __forceinline__ void lds_load16_sv(uint32_t lds_dst, uint32_t voff, const void* sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(lds_dst), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+// 16 bytes per lane from a full per-lane address
+__device__ __forceinline__ void lds_load16_v(uint32_t lds_dst, const void* vaddr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(lds_dst), "v"(vaddr) : "memory", "m0");
+}
+// 4 bytes per lane from a full per-lane address
+__device__ __forceinline__ void lds_load4_v(uint32_t lds_dst, const void* vaddr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" :: "s"(lds_dst), "v"(vaddr) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 // Reciprocal square root of the two RMSNorm forms. Form 0 is the reference kernel's 1 / sqrt(.) in fp32 (two
 // roundings, batch_invariant_ops.py:653-660). Form 1 is what HuggingFace's module computes with torch.rsqrt on this
 // device: measured on the GPU over 2^24 arguments, torch.rsqrt(x) has the bits of the double-precision quotient

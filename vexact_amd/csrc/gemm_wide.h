@@ -172,8 +172,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(GemmParams p, int tiles_
   auto issue_one = [&](int q, int stage) {
     const uint32_t dst = lds0 + stage * STAGE + (q < NXQ ? q * 8192 : XBYTES + (q - NXQ) * 8192);
     const bf16_t* base = q < NXQ ? p.x + ld_k : wsrc + ld_wbase + (PACKED ? 16 * ld_k : ld_k);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
+    lds_load16_sv(dst, ld_off[q], base);
   };
   auto advance_loads = [&]() {  // next step of the stream; past the last tile it re-reads (unused)
     ld_k += WD_BK;
@@ -482,8 +481,7 @@ __global__ __launch_bounds__(256) void gemm_ring_kernel(GemmParams p) {
       const bool isx = q < BM / 8;
       const uint32_t dst = sb + u * SUB + (isx ? q * 1024 : XB + (q - BM / 8) * 1024);
       const bf16_t* base = (isx ? p.x : p.w) + (st * KSUB + u) * 64;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :: "s"(dst), "v"(ld_off[t]), "s"(base) : "memory", "m0");
+      lds_load16_sv(dst, ld_off[t], base);
     }
   };
 

@@ -244,12 +244,11 @@ __global__ __launch_bounds__(512) void moe_gemm_nn_wide_kernel(MoeNnParams p, in
   int ld_lin = first, ld_k = 0;
   set_load_tile(first, 0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)nw_lds + wave * 1024;
-  // asm, so that the compiler does not wait for these LDS writes before unrelated fragment reads (see gemm_wide.h)
+  // asm inside lds_load16_sv, so that the compiler does not wait for these LDS writes before unrelated fragment reads
   auto issue_one = [&](int q, int stage) {
     const uint32_t dst = lds0 + stage * STAGE + (q < 4 ? q * 8192 : XBYTES + (q - 4) * 8192);
     const bf16_t* base = q < 4 ? ld_xb : ld_wb;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
+    lds_load16_sv(dst, ld_off[q], base);
   };
   auto advance_loads = [&]() {  // next step of the stream; past the last tile it re-reads (unused)
     ld_k += 64;
@@ -539,12 +538,11 @@ __global__ __launch_bounds__(512) void moe_gemm_tn_wide_kernel(MoeTnParams p) {
     }
     landed_valid = ld_valid;
   };
-  // asm, so that the compiler does not wait for these LDS writes before unrelated fragment reads (see gemm_wide.h)
+  // asm inside lds_load16_sv, so that the compiler does not wait for these LDS writes before unrelated fragment reads
   auto issue_one = [&](int q, int stage) {
     const uint32_t dst = lds0 + stage * STAGE + (q < 4 ? q * 8192 : TBYTES + (q - 4) * 8192);
     const bf16_t* base = q < 4 ? p.dy : p.x;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(dst), "v"(ld_off[q]), "s"(base) : "memory", "m0");
+    lds_load16_sv(dst, ld_off[q], base);
   };
   auto advance_loads = [&]() {  // next step of the stream; past the last tile with rows it re-reads (unused)
     ld_s++;
