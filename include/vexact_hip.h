@@ -46,8 +46,10 @@ int vx_mean_dim(const void* in, void* out, int dtype, int64_t M, int64_t N, int6
 /* RMSNorm over the last dim of [rows, n].
  *   mode 0: y = round(x * (1/sqrt(mean(x^2) + eps)) * w)          (one rounding)
  *           replaces _rms_norm_kernel / _rms_norm_forward, batch_invariant_ops.py:637-687
- *   mode 1: y = round(w * round(x * (1/sqrt(mean(x^2) + eps))))   (HuggingFace Qwen3 RMSNorm as it
- *           executes when its .mean(-1) is routed through mean_dim, batch_invariant_ops.py:619-622)
+ *   mode 1: y = round(w * round(x * rsqrt(mean(x^2) + eps)))      (HuggingFace Qwen3 RMSNorm as it
+ *           executes when its .mean(-1) is routed through mean_dim, batch_invariant_ops.py:619-622;
+ *           rsqrt = the double-precision quotient 1/sqrt rounded once to fp32, which is what
+ *           torch.rsqrt returns on this GPU, so the result has the bits of the module's forward)
  * residual (optional): the row is first replaced by round(x + residual) and that sum is written to
  * sum_out (optional; may alias x or residual). */
 int vx_rms_norm(const void* x, const void* residual, const void* weight, void* y, void* sum_out,
