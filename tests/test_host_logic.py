@@ -345,7 +345,8 @@ def test_expert_tile_heights_and_unfilled_outputs():
 
     # tile height is a function of the token count; a model that holds fragment-order expert weights only never
     # gets 128-row tiles (the one kernel that cannot read them)
-    assert [ops.moe_tile_rows(t) for t in (1, 448, 449, 704, 705, 2047, 2048, 100000)] == [32, 32, 64, 64, 128, 128, 256, 256]
+    assert [ops.moe_tile_rows(t) for t in (1, 16, 17, 448, 449, 704, 705, 2047, 2048, 100000)] == [16, 16, 32, 32, 64, 64, 128, 128, 256, 256]
+    assert ops.moe_tile_rows(16, packed=True) == 16 and ops.moe_tile_rows(3, top_k=2, num_experts=16) == 16
     assert [ops.moe_tile_rows(t, packed_only=True) for t in (256, 448, 449, 832, 833, 2048)] == [32, 32, 64, 64, 256, 256]
     assert [ops.moe_tile_rows(t, packed=True) for t in (256, 448, 449, 832, 833, 2048)] == [32, 32, 64, 64, 256, 256]
     assert ops.moe_tile_rows(5000, wide_ok=False) == 128 and ops.moe_tile_rows(5000, wide_ok=False, packed_only=True) == 64

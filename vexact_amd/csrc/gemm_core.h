@@ -51,8 +51,10 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u, float w) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Streaming kernel. 256 threads = 4 wavefronts; wavefront v owns weight rows
-// [n0 + 16 v, n0 + 16 v + 16); the block covers 64 weight rows and BM = 16*MT activation rows.
+// Streaming kernel. 64 NW threads = NW wavefronts (4 unless said otherwise); wavefront v owns weight rows
+// [n0 + 16 v, n0 + 16 v + 16); the block covers 16 NW weight rows and BM = 16*MT activation rows.
+// NW = 1 is for launches of a few tiles (a single token's eight experts): four times the workgroups, so that
+// the weight stream is pulled by every CU instead of the hundred that 4-wavefront blocks would occupy.
 // ---------------------------------------------------------------------------------------
 // U  = k-steps of weight loads a wavefront keeps in flight (one group);
 // KD = divisor of the staged K chunk: KC = 32768 / (BM * KD) elements per LDS fill (64 KB / KD of
@@ -61,13 +63,15 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u, float w) {
 // wavefront feed to one MFMA (16 weight rows x 32 k) is contiguous and in lane order, so a wavefront
 // streams one linear run of (K / 32) KB per 16-row block instead of 16 rows of pitch ldw. p.ldw is then
 // the number of 32-wide k-chunks stored per row block (K rounded up to a multiple of 32 U, zero filled).
-template <int MT, int EPI, bool GROUPED, int U = 8, int KD = 1, bool PACKED = false>
-__global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
+template <int MT, int EPI, bool GROUPED, int U = 8, int KD = 1, bool PACKED = false, int NW = 4>
+__global__ __launch_bounds__(64 * NW) void gemm_stream_kernel(GemmParams p) {
+  constexpr int NT = 64 * NW;  // threads
   constexpr int BM = 16 * MT;
   constexpr int KC = 32768 / (BM * KD);  // K elements staged per LDS fill
   constexpr int RB = KC * 2 + 16;        // +16: rows land on distinct bank groups
   __shared__ __attribute__((aligned(16))) uint8_t xs[BM * RB];
   static_assert(KC % (32 * U) == 0, "a staged chunk must hold whole groups");
+  static_assert(!PACKED || 8 % U == 0, "a fragment-order image is zero-filled to multiples of 8 k-chunks: a group of U chunks must not cross that");
 
   int row0, rows;
   int64_t wbase = 0;
@@ -84,7 +88,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 64 + wave * 16;
+  const int n0 = blockIdx.x * (16 * NW) + wave * 16;
   const int K = p.K;
   const bf16_t* wp;
   const bf16_t* wp2 = nullptr;
@@ -149,14 +153,15 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
     }
   };
 
-  // Activation staging: thread owns pieces tid + 256 j (j < NP) of the BM x KC tile; piece =
+  // Activation staging: thread owns pieces tid + NT j (j < NP) of the BM x KC tile; piece =
   // (row pc / PPR, 16-byte column pc % PPR). Row sources are resolved once.
   constexpr int PPR = KC / 8;            // 16-byte pieces per staged row
-  constexpr int NP = BM * PPR / 256;     // pieces per thread (16)
+  constexpr int NP = BM * PPR / NT;      // pieces per thread
+  static_assert(BM * PPR % NT == 0, "pieces must split evenly over the threads");
   int64_t xoff[NP];                      // element offset of the piece's row in x, -1 = zero row
 #pragma unroll
   for (int j = 0; j < NP; j++) {
-    const int pc = threadIdx.x + 256 * j;
+    const int pc = threadIdx.x + NT * j;
     const int r = pc / PPR;
     int64_t off = -1;
     if (r < rows) {
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   auto stage_load = [&](int kc) {
 #pragma unroll
     for (int j = 0; j < NP; j++) {  // all loads of the fill in flight together
-      const int c8 = (threadIdx.x + 256 * j) % PPR;
+      const int c8 = (threadIdx.x + NT * j) % PPR;
       const bool ok = xoff[j] >= 0 && kc + c8 * 8 < K;
       stage[j] = ldg16_raw(p.x + (ok ? xoff[j] + kc : 0));
     }
@@ -180,7 +185,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(GemmParams p) {
   auto stage_store = [&](int kc) {
 #pragma unroll
     for (int j = 0; j < NP; j++) {
-      const int pc = threadIdx.x + 256 * j;
+      const int pc = threadIdx.x + NT * j;
       const int c8 = pc % PPR;
       const bool ok = xoff[j] >= 0 && kc + c8 * 8 < K;
       *(uint4*)(xs + (pc / PPR) * RB + c8 * 16) = mask16(stage[j], ok);

@@ -620,6 +620,15 @@ int vx_moe_route(const void* expert_idx, int idx_i64, int64_t T, int k, int E, i
                          tile_group, tile_row0, tile_rows, max_tiles, nullptr, 0, stream);
 }
 
+// One-wavefront blocks for the streaming kernel: when 4-wavefront blocks would be few (a step of one to four tokens:
+// 8 .. 34 expert tiles) and every wavefront has a long run to stream (K >= 1024), four times the workgroups put a
+// weight stream on every CU. Measured at 128 experts / top-8, hidden 2048, gate/up on 16-row tiles: 1 token 23.8 ->
+// 18.2 us, 3 tokens 41.9 -> 31.9, 4 tokens 46.5 -> 41.0, level from 6 tokens on; the down projection (K = 768, four
+// times the blocks already) is level or slower, and so are 32-row tiles.
+static inline bool stream_narrow_launch(int64_t max_tiles, int64_t N, int64_t K) {
+  return K >= 1024 && max_tiles * ((N + 63) / 64) < 512;
+}
+
 // Grouped GEMM over a tile table: C[rows of tile] = X[row_src[rows]] * W[group]^T.
 // epi 0: plain bf16 store. epi 1: SwiGLU with w = gate rows, w2 = up rows, scaled per row by
 // row_scale[row_scale_idx[row]].  bm in {16, 32, 64} selects the streaming kernel, 128 the tiled one,
@@ -654,8 +663,16 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
     if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true, 8, 2><<<grid, 256, 0, stream>>>(p); \
     else gemm_stream_kernel<MT, EPI_PLAIN, true, 8, 2><<<grid, 256, 0, stream>>>(p);               \
   } while (0)
+  // a launch of a few 16-row tiles as one-wavefront blocks of 16 weight rows, 256-element activation chunks
+#define VX_GG1(MT)                                                                                 \
+  do {                                                                                             \
+    const dim3 grid((unsigned)((N + 15) / 16), my);                                                \
+    if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true, 8, 8, false, 1><<<grid, 64, 0, stream>>>(p); \
+    else gemm_stream_kernel<MT, EPI_PLAIN, true, 8, 8, false, 1><<<grid, 64, 0, stream>>>(p);  \
+  } while (0)
+  const bool narrow = stream_narrow_launch(max_tiles, N, K);
   switch (bm) {
-    case 16: VX_GG(1); break;
+    case 16: if (narrow) VX_GG1(1); else VX_GG(1); break;
     case 32: VX_GG(2); break;
     case 64: VX_GG(4); break;
     case 128: {
@@ -671,6 +688,7 @@ int vx_moe_gemm(const void* x, int64_t ldx, const void* w, const void* w2, int64
     default: return VX_ERR_ARG;
   }
 #undef VX_GG
+#undef VX_GG1
   return launch_status();
 }
 
@@ -728,12 +746,20 @@ int vx_moe_gemm_packed(const void* x, int64_t ldx, const void* w, const void* w2
     if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true, 8, 2, true><<<grid, 256, 0, stream>>>(p); \
     else gemm_stream_kernel<MT, EPI_PLAIN, true, 8, 2, true><<<grid, 256, 0, stream>>>(p);                    \
   } while (0)
+#define VX_GP1(MT)                                                                                           \
+  do {                                                                                                       \
+    const dim3 grid1((unsigned)((N + 15) / 16), (unsigned)max_tiles);                                        \
+    if (epi == EPI_SWIGLU) gemm_stream_kernel<MT, EPI_SWIGLU, true, 8, 8, true, 1><<<grid1, 64, 0, stream>>>(p); \
+    else gemm_stream_kernel<MT, EPI_PLAIN, true, 8, 8, true, 1><<<grid1, 64, 0, stream>>>(p);            \
+  } while (0)
+  const bool narrow = stream_narrow_launch(max_tiles, N, K);
   switch (bm) {
-    case 16: VX_GP(1); break;
+    case 16: if (narrow) VX_GP1(1); else VX_GP(1); break;
     case 32: VX_GP(2); break;
     default: VX_GP(4); break;
   }
 #undef VX_GP
+#undef VX_GP1
   return launch_status();
 }
 
