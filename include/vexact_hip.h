@@ -219,8 +219,11 @@ int vx_attention_ex(const void* q, const void* k, const void* v, void* out, floa
  * (this is what vx_attention / vx_attention_ex call); every other case runs the kernels built for the next of
  * (64, 64), (128, 128), (256, 128), (256, 256) with the missing query columns as zeros, which leaves every bit
  * as an exact-size kernel would compute it; head sizes or strides that are not multiples of 8 elements, or bases
- * that are not 16-byte aligned, are served with per-element accesses (correct, slow). fp32 inputs, which the
- * reference also takes, are not supported (VX_ERR_UNSUPPORTED for any other dtype code). */
+ * that are not 16-byte aligned, are served with per-element accesses (correct, slow). dtype 2 = fp32, which the
+ * reference's kernels also take (FP32_OUTPUT, triton_invariant_attention.py:108-113; its backward tests run in it):
+ * a correctness path of one thread per output row, single ascending fp32 sums and true fp32 products (the
+ * reference's tl.dot would use TF32), every mode through the same routine, so paged, packed, prefill and decode
+ * agree bit for bit; it needs no workspace and ignores seq_order. Any other dtype code: VX_ERR_UNSUPPORTED. */
 int vx_attention_typed(const void* q, const void* k, const void* v, void* out, float* lse, const int* seq_order,
                        const int* cu_seqlens_q, const int* seqused_k, const int* cu_seqlens_k, const int* block_table,
                        int64_t total_q, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,
@@ -246,7 +249,8 @@ int vx_attention_bwd(const void* q, const void* k, const void* v, const void* ou
  * q / k / dq / dk, Dv of v / out / dout / dv, as _NonpagedFlashAttentionVarlen.backward takes them
  * (triton_invariant_attention.py:786-902, BLOCK_D = next power of two of the larger one). bf16 at Dk = Dv = 128
  * runs the LDS kernels, everything else register-form kernels built for 64, 128 or 256 (the last two spill and
- * are slow); rows that are not 16-byte addressable are served per element. */
+ * are slow); rows that are not 16-byte addressable are served per element. dtype 2 = fp32 (every tensor fp32):
+ * one thread per gradient row, P recomputed from lse in fp32 without intermediate rounding. */
 int vx_attention_bwd_typed(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
                            void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
                            int64_t total_q, int64_t total_k, int64_t num_seqs, int Hq, int Hkv, int Dk, int Dv,

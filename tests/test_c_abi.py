@@ -19,7 +19,7 @@ def test_library_is_built_and_loads():
     if not os.path.exists(_build.LIB_PATH):
         _build.build()
     lib = _lib.load()
-    assert lib.vx_abi_version() == 7
+    assert lib.vx_abi_version() == 8
     assert lib.vx_status_string(0) == b"ok"
     assert b"workspace" in lib.vx_status_string(-3)
 

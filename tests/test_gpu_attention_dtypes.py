@@ -225,9 +225,9 @@ def test_backward_register_kernels_agree_with_the_lds_kernels_at_128():
 
 
 def test_dtype_and_size_limits_raise():
-    q = torch.zeros(2, 4, 64, device="cuda")
+    q = torch.zeros(2, 4, 64, device="cuda", dtype=torch.float64)
     cu = _cu([2]).cuda()
-    with pytest.raises(ValueError, match="bfloat16 or float16"):
+    with pytest.raises(ValueError, match="bfloat16, float16 or float32"):
         ops.packed_attention(q, q[:, :2], q[:, :2], cu, cu, 0.125, True, 2)
     h = torch.zeros(2, 4, 264, device="cuda", dtype=torch.float16)
     with pytest.raises(ValueError, match="head_dim must be <= 256"):

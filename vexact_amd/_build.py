@@ -14,8 +14,8 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvexact_hip.so")
-SOURCES = ["row_ops.hip", "gemm.hip", "gemm_other.hip", "paged_attn.hip", "paged_attn_pad.hip", "paged_attn_f16.hip", "attn_bwd.hip", "attn_bwd_f16.hip", "moe.hip", "moe_bwd.hip", "glue.hip", "sampler.hip", "host_meta.cpp"]
-HEADERS = ["common.h", "gemm_core.h", "gemm_wide.h", "attn_core.h", "attn_bwd_core.h"]
+SOURCES = ["row_ops.hip", "gemm.hip", "gemm_other.hip", "paged_attn.hip", "paged_attn_pad.hip", "paged_attn_f16.hip", "attn_bwd.hip", "attn_bwd_f16.hip", "attn_f32.hip", "moe.hip", "moe_bwd.hip", "glue.hip", "sampler.hip", "host_meta.cpp"]
+HEADERS = ["common.h", "gemm_core.h", "gemm_wide.h", "attn_core.h", "attn_bwd_core.h", "attn_f32.h", "attn_f32_launch.h"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -ffp-contract=off: kernels that must agree bit for bit share source-level expressions, so the

@@ -16,6 +16,7 @@
 // row loads and an 8 x 8 bf16 transpose in registers. Every sum runs in a fixed order that depends
 // only on the sequence's own lengths, so a sequence's gradients do not depend on the batch.
 #include "attn_bwd_core.h"
+#include "attn_f32_launch.h"
 
 namespace vx {
 
@@ -366,7 +367,7 @@ int vx_attention_bwd(const void* q, const void* k, const void* v, const void* ou
 }
 
 // Any head sizes up to 256 (Dk of q / k / dq / dk, Dv of v / out / dout / dv) and either 16-bit element type
-// (dtype 0 = bf16, 1 = fp16). bf16 at Dk = Dv = 128 runs the LDS kernels, everything else the register-form kernels
+// (dtype 0 = bf16, 1 = fp16) or fp32 (dtype 2: one thread per gradient row). bf16 at Dk = Dv = 128 runs the LDS kernels, everything else the register-form kernels
 // of the next built-for size (64, 128, 256), per element when rows are not 16-byte addressable.
 int vx_attention_bwd_typed(const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
                            void* dq, void* dk, void* dv, const int* cu_seqlens_q, const int* cu_seqlens_k,
@@ -378,9 +379,26 @@ int vx_attention_bwd_typed(const void* q, const void* k, const void* v, const vo
     return VX_ERR_ARG;
   if (total_q < 0 || total_k < 0 || num_seqs < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || Dk <= 0 || Dv <= 0) return VX_ERR_ARG;
   if (max_seqlen_q < 0 || max_seqlen_k < 0 || num_seqs > 65535 || Hq > 65535) return VX_ERR_ARG;
-  if (dtype != 0 && dtype != 1) return VX_ERR_UNSUPPORTED;
+  if (dtype != 0 && dtype != 1 && dtype != 2) return VX_ERR_UNSUPPORTED;
   if (Dk > 256 || Dv > 256) return VX_ERR_UNSUPPORTED;
   if (total_q == 0 || total_k == 0 || num_seqs == 0 || max_seqlen_q == 0 || max_seqlen_k == 0) return VX_OK;
+  if (dtype == 2) {  // fp32: one thread per gradient row (attn_f32.h)
+    const uintptr_t all = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dq |
+                          (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)workspace;
+    if (all % 4 != 0) return VX_ERR_ARG;
+    if (!workspace || workspace_bytes < total_q * Hq * 4) return VX_ERR_WORKSPACE;
+    AttnF32Bwd f = {};
+    f.q = (const float*)q; f.k = (const float*)k; f.v = (const float*)v; f.o = (const float*)out;
+    f.d_o = (const float*)dout; f.lse = lse; f.delta = (float*)workspace;
+    f.dq = (float*)dq; f.dk = (float*)dk; f.dv = (float*)dv;
+    f.sqt = strides[0]; f.sqh = strides[1]; f.skt = strides[2]; f.skh = strides[3];
+    f.svt = strides[4]; f.svh = strides[5]; f.sot = strides[6]; f.soh = strides[7];
+    f.sdt = strides[8]; f.sdh = strides[9]; f.sdqt = strides[10]; f.sdqh = strides[11];
+    f.sdkt = strides[12]; f.sdkh = strides[13]; f.sdvt = strides[14]; f.sdvh = strides[15];
+    f.cu_q = cu_seqlens_q; f.cu_k = cu_seqlens_k;
+    f.Hq = Hq; f.Hkv = Hkv; f.num_seqs = (int)num_seqs; f.dk_ = Dk; f.dv_ = Dv; f.scale = softmax_scale;
+    return launch_attn_f32_backward(f, total_q, total_k, stream);
+  }
   const uintptr_t ptrs = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dq |
                          (uintptr_t)dk | (uintptr_t)dv;
   if (ptrs % 2 != 0) return VX_ERR_ARG;

@@ -246,6 +246,6 @@ const char* vx_status_string(int code) {
   }
 }
 
-int vx_abi_version() { return 7; }
+int vx_abi_version() { return 8; }
 
 }  // extern "C"

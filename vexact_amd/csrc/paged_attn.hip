@@ -6,6 +6,7 @@
 // twin _varlen_attn_fwd_block_kernel (:47-190, :700-784) and _store_cache_kernel / store_kvcache
 // (vexact/batch_invariant_ops/kv_cache_context.py:259-314).
 #include "attn_core.h"
+#include "attn_f32_launch.h"
 
 namespace vx {
 
@@ -129,8 +130,8 @@ int vx_attention_ex(const void* q, const void* k, const void* v, void* out, floa
                             softmax_scale, causal, mode, max_seqlen_q, 0, workspace, workspace_bytes, stream);
 }
 
-// vx_attention_ex for either 16-bit element type (dtype 0 = bf16, 1 = fp16; q, k, v and out share it) and any head
-// sizes up to 256. bf16 at (Dk, Dv) in {(32, 32), (64, 64), (128, 128), (192, 128), (256, 256)} with 16-byte
+// vx_attention_ex for either 16-bit element type (dtype 0 = bf16, 1 = fp16; q, k, v and out share it) or fp32 (dtype 2:
+// a correctness path of one thread per output row, attn_f32.h; no workspace, seq_order ignored) and any head sizes up to 256. bf16 at (Dk, Dv) in {(32, 32), (64, 64), (128, 128), (192, 128), (256, 256)} with 16-byte
 // addressable rows runs the kernels built for exactly those sizes; everything else runs the kernels of the next
 // built-for size with the missing query columns as zeros (same bits as an exact-size kernel would give), and
 // per-element accesses when a head size or stride is not a multiple of 8 elements.
@@ -142,7 +143,7 @@ int vx_attention_typed(const void* q, const void* k, const void* v, void* out, f
                        int64_t max_pages, int page_size, float softmax_scale, int causal, int mode,
                        int max_seqlen_q, int dtype, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (!q || !k || !v || !out || !cu_seqlens_q) return VX_ERR_ARG;
-  if (dtype != 0 && dtype != 1) return VX_ERR_UNSUPPORTED;
+  if (dtype != 0 && dtype != 1 && dtype != 2) return VX_ERR_UNSUPPORTED;
   if (Dk <= 0 || Dv <= 0) return VX_ERR_ARG;
   if (Dk > 256 || Dv > 256) return VX_ERR_UNSUPPORTED;
   if (lse && mode != 1 && mode != 2) return VX_ERR_UNSUPPORTED;
@@ -155,6 +156,24 @@ int vx_attention_typed(const void* q, const void* k, const void* v, void* out, f
   if (decode && !causal) return VX_ERR_UNSUPPORTED;
   if (total_q == 0 || num_seqs == 0) return VX_OK;
   if (num_seqs > 65535 || Hq > 65535) return VX_ERR_UNSUPPORTED;
+  if (dtype == 2) {  // fp32: one thread per output row, the same routine for every mode (attn_f32.h)
+    if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 4 != 0) return VX_ERR_ARG;
+    AttnF32 f = {};
+    f.q = (const float*)q; f.sqt = sqt; f.sqh = sqh;
+    f.k = (const float*)k; f.skb = skb; f.skp = skp; f.skh = skh;
+    f.v = (const float*)v; f.svb = svb; f.svp = svp; f.svh = svh;
+    f.o = (float*)out; f.sot = sot; f.soh = soh;
+    f.lse = lse;
+    f.cu_q = cu_seqlens_q; f.seqused_k = seqused_k; f.cu_k = cu_seqlens_k;
+    f.block_table = block_table; f.bt_stride = bt_stride;
+    f.page_size = page_size;
+    const int64_t mk = mode != 2 ? max_pages * (int64_t)page_size : 0;
+    f.max_kv = (int)(mk > 0x7fffffff ? 0x7fffffff : mk);
+    f.Hq = Hq; f.Hkv = Hkv; f.num_seqs = (int)num_seqs; f.dk = Dk; f.dv = Dv;
+    f.causal = causal; f.packed = mode == 2 ? 1 : 0;
+    f.scale = softmax_scale;
+    return launch_attn_f32_forward(f, total_q, stream);
+  }
   // rows that 16-byte accesses cannot address go element by element
   const bool elem = (sqt | sqh | skb | skp | skh | svb | svp | svh | sot | soh | (int64_t)Dk | (int64_t)Dv) % 8 != 0 ||
                     ((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16 != 0;

@@ -556,12 +556,14 @@ def store_kvcache(key, value, k_cache, v_cache, slot_mapping) -> None:
 
 
 def _attn_dtype_code(what: str, *tensors: torch.Tensor) -> int:
-    """0 for bf16, 1 for fp16 (the C ABI's dtype code); every tensor must share it. fp32, which the reference's
-    kernels also take (through TF32 products), is not supported."""
+    """0 for bf16, 1 for fp16, 2 for fp32 (the C ABI's dtype code); every tensor must share it. fp32, which the
+    reference's kernels also take (its own backward tests run in it), goes to a correctness path of one thread per
+    output row with true fp32 products; the 16-bit types are the tuned ones."""
+    codes = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
     dt = tensors[0].dtype
-    if dt not in (torch.bfloat16, torch.float16) or any(t.dtype != dt for t in tensors):
-        raise ValueError(f"{what} supports bfloat16 or float16 tensors of one dtype, got {[str(t.dtype) for t in tensors]}")
-    return 0 if dt == torch.bfloat16 else 1
+    if dt not in codes or any(t.dtype != dt for t in tensors):
+        raise ValueError(f"{what} supports bfloat16, float16 or float32 tensors of one dtype, got {[str(t.dtype) for t in tensors]}")
+    return codes[dt]
 
 
 def paged_attention(
@@ -662,7 +664,7 @@ def packed_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor, lse: torch.Tensor,
     cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor, softmax_scale: float, max_seqlen_q: int, max_seqlen_k: int,
 ):
-    """(dq, dk, dv) of causal ``packed_attention`` (bf16 or fp16, head sizes up to 256; shapes of q, k, v)."""
+    """(dq, dk, dv) of causal ``packed_attention`` (bf16, fp16 or fp32, head sizes up to 256; shapes of q, k, v)."""
     for name, t in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)):
         _need_gpu(name, t)
         if t.dim() != 3 or t.stride(2) != 1:
