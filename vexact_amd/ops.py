@@ -638,7 +638,9 @@ def packed_attention(
     ``return_lse`` also returns the rows' fp32 log-sum-exp ``[T, Hq]`` (what the backward needs)."""
     T, Hq, Dk = q.shape
     Hkv, Dv = k.shape[1], v.shape[-1]
-    o = torch.empty((T, Hq, Dv), dtype=q.dtype, device=q.device)
+    # zeros, as the reference allocates its packed output (triton_invariant_attention.py:733): the rows of a sequence
+    # that has queries but no keys are written by no kernel (rows that merely see no key under the mask are: as 0)
+    o = torch.zeros((T, Hq, Dv), dtype=q.dtype, device=q.device)
     lse = torch.empty((T, Hq), dtype=torch.float32, device=q.device) if return_lse else None
     if T == 0:
         return (o, lse) if return_lse else o
