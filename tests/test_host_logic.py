@@ -401,3 +401,14 @@ def test_gemm_piece_addresses_below_the_step_width_stay_inside_the_row():
         for U in (1, 2, 4, 8):
             assert all(0 <= o <= K - 8 for o in offsets_stream(K, U)), (K, U)
         assert all(0 <= o <= K - 8 for o in offsets_tiled(K)), K
+
+
+def test_fragment_order_image_holds_whole_load_groups():
+    # The streaming kernel reads a fragment-order weight image in groups of 8 k-chunks (32 k-elements each) without
+    # any mask: the image must therefore be zero-filled to a multiple of 8 chunks that covers K, or the last group of
+    # a row block would run into the next block (past the tensor for the last block of the last expert).
+    from vexact_amd import _lib
+    lib = _lib.load()
+    for K in list(range(1, 600)) + [767, 768, 769, 2047, 2048, 2049, 4096, 12288]:
+        ch = lib.vx_packed_kchunks(K)
+        assert ch % 8 == 0 and 32 * ch >= K and 32 * (ch - 8) < K, (K, ch)
