@@ -1158,7 +1158,7 @@ __global__ __launch_bounds__(64 * PFL_WAVES) void attn_prefill_lds_kernel(AttnPa
 // Which decode form a launch takes: chunks folded inside one workgroup per (sequence, kv head) when that
 // fills the machine (or mode 4), else one wavefront per chunk plus a combine launch (or mode 3); only the
 // latter uses the workspace. A function of the shapes alone. Returns 1 = fused, 0 = split, < 0 = error.
-static int decode_form(int mode, int64_t num_seqs, int Hq, int Hkv, int Dv_caller) {
+static inline int decode_form(int mode, int64_t num_seqs, int Hq, int Hkv, int Dv_caller) {
   // the value head size the kernels are built for: every caller of this function (workspace queries with the
   // caller's size, launches with the built-for size) must reach the same answer
   const int Dv = Dv_caller <= 32 ? 32 : Dv_caller <= 64 ? 64 : Dv_caller <= 128 ? 128 : 256;
