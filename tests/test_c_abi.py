@@ -62,3 +62,39 @@ def test_bad_arguments_are_rejected_before_any_launch():
     assert lib.vx_moe_route(None, 0, 1, 1, 1, 32, None, None, None, None, None, None, None, None, 8, None) == -1
     assert lib.vx_attention(None, None, None, None, None, None, None, None, 1, 1, 4, 2, 128, 128,
                             0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 16, 1.0, 1, 0, 1, None, 0, None) == -1
+
+
+def _header_signatures():
+    """name -> (return type, [parameter types]) parsed from the header: 'ptr' for any pointer or the stream handle,
+    else the scalar type."""
+    text = open(os.path.join(ROOT, "include", "vexact_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    sigs = {}
+    for m in re.finditer(r"([A-Za-z_][A-Za-z0-9_ ]*?[\s\*]+)(vx_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        ret, name, params = m.group(1).strip(), m.group(2), m.group(3).strip()
+
+        def kind(decl: str) -> str:
+            decl = decl.strip()
+            if "*" in decl or decl.startswith("hipStream_t"):
+                return "ptr"
+            return re.sub(r"\s+[A-Za-z_][A-Za-z0-9_]*$", "", re.sub(r"^const\s+", "", decl)).strip()
+
+        plist = [] if params in ("", "void") else [kind(p) for p in params.split(",")]
+        sigs[name] = (kind(ret + " x") if "*" not in ret else "ptr", plist)
+    return sigs
+
+
+def test_ctypes_prototypes_match_the_header_parameter_by_parameter():
+    want = {"ptr": ctypes.c_void_p, "int": ctypes.c_int, "int32_t": ctypes.c_int, "int64_t": ctypes.c_int64, "float": ctypes.c_float,
+            "void": None}
+    sigs = _header_signatures()
+    assert sorted(sigs) == sorted(_lib.PROTOTYPES)
+    for name, (ret, params) in sigs.items():
+        restype, argtypes = _lib.PROTOTYPES[name]
+        assert len(argtypes) == len(params), f"{name}: {len(argtypes)} ctypes arguments, {len(params)} in the header"
+        for i, (a, p) in enumerate(zip(argtypes, params)):
+            assert a is want[p], f"{name}: argument {i} is {p} in the header, {a.__name__} in the binding"
+        if ret == "ptr":
+            assert restype in (ctypes.c_char_p, ctypes.c_void_p), name
+        else:
+            assert restype is want[ret], f"{name}: returns {ret} in the header, {restype.__name__} in the binding"
