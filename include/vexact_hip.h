@@ -9,7 +9,8 @@
  *   - all data pointers are device pointers owned by the caller; `stream` is the HIP stream to
  *     launch on; strides and leading dimensions are in ELEMENTS unless the name says bytes;
  *   - launch geometry depends only on the sizes passed by value, never on device data;
- *   - dtype codes: 0 = float32, 1 = bfloat16, 2 = float16;
+ *   - dtype codes: 0 = float32, 1 = bfloat16, 2 = float16, except where an entry point states its own (the typed
+ *     attention entry points, which grew out of a bf16-only form: 0 = bfloat16, 1 = float16, 2 = float32);
  *   - batch invariance: the bits of an output row depend on that row's own inputs only (not on
  *     the number of rows, their order, or which other rows share the launch).
  *

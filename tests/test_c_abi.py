@@ -98,3 +98,36 @@ def test_ctypes_prototypes_match_the_header_parameter_by_parameter():
             assert restype in (ctypes.c_char_p, ctypes.c_void_p), name
         else:
             assert restype is want[ret], f"{name}: returns {ret} in the header, {restype.__name__} in the binding"
+
+
+def _source_definitions():
+    """name -> [parameter kinds] of every vx_* function DEFINED in csrc (the sources do not include the public header,
+    so nothing else compares the two)."""
+    src_dir = os.path.join(ROOT, "vexact_amd", "csrc")
+    defs = {}
+    for fn in sorted(os.listdir(src_dir)):
+        if not fn.endswith((".hip", ".cpp")):
+            continue
+        text = open(os.path.join(src_dir, fn)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        for m in re.finditer(r"\b(vx_[a-z0-9_]+)\s*\(([^;{}()]*)\)\s*\{", text, flags=re.S):
+            name, params = m.group(1), m.group(2).strip()
+
+            def kind(decl: str) -> str:
+                decl = decl.strip()
+                if "*" in decl or decl.startswith("hipStream_t"):
+                    return "ptr"
+                return re.sub(r"\s+[A-Za-z_][A-Za-z0-9_]*$", "", re.sub(r"^const\s+", "", decl)).strip()
+
+            plist = [] if params in ("", "void") else [kind(p) for p in params.split(",")]
+            assert name not in defs, f"{name} defined twice ({fn})"
+            defs[name] = plist
+    return defs
+
+
+def test_definitions_in_the_sources_match_the_header():
+    sigs, defs = _header_signatures(), _source_definitions()
+    assert sorted(defs) == sorted(sigs), set(defs) ^ set(sigs)
+    for name, (_, params) in sigs.items():
+        assert defs[name] == params, f"{name}: header {params}, definition {defs[name]}"
