@@ -412,3 +412,19 @@ def test_fragment_order_image_holds_whole_load_groups():
     for K in list(range(1, 600)) + [767, 768, 769, 2047, 2048, 2049, 4096, 12288]:
         ch = lib.vx_packed_kchunks(K)
         assert ch % 8 == 0 and 32 * ch >= K and 32 * (ch - 8) < K, (K, ch)
+
+
+def test_host_metadata_and_allocator_under_address_and_ub_sanitizers():
+    # the native step-metadata builder and block allocator on 400 random steps and 50 random allocate / free traces with
+    # exactly sized heap buffers, compiled with -fsanitize=address,undefined: an access outside a buffer aborts the run
+    import os
+    import subprocess
+    import tempfile
+    here = os.path.dirname(os.path.abspath(__file__))
+    with tempfile.TemporaryDirectory() as d:
+        exe = os.path.join(d, "host_meta_sanitized")
+        subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                        "-static-libasan", "-o", exe, os.path.join(here, "host_meta_sanitized.cpp")], check=True)
+        run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "sanitized run ok" in run.stdout
