@@ -172,3 +172,15 @@ def test_paged_layout_gives_the_bits_of_the_packed_layout_and_decode_those_of_pr
     used0[1] = 0
     out0, _ = _forward(lib, torch.cat(q_seqs), k_cache, v_cache, _cu(kv_lens), seqused=used0, table=table, page=page, want_lse=False)
     assert (out0[17 : 17 + 33] == 7.0).all() and torch.equal(out0[:17], paged[:17])
+
+
+def test_addresses_under_address_and_ub_sanitizers():
+    # random packed and paged batches (ragged and empty sequences, odd head sizes and page sizes, a kv length beyond what
+    # the block table addresses) with exactly sized heap buffers, compiled with -fsanitize=address,undefined
+    with tempfile.TemporaryDirectory() as d:
+        exe = os.path.join(d, "attn_f32_sanitized")
+        subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                        "-static-libasan", "-ffp-contract=off", "-o", exe, os.path.join(_HERE, "attn_f32_sanitized.cpp")], check=True)
+        run = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "sanitized run ok" in run.stdout
