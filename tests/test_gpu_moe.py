@@ -590,39 +590,6 @@ def test_packed_expert_weights_give_the_same_bits(T, H, I, E, k):
         assert_bitwise(eo_p, eo, f"down projection on packed weights, {bm}-row tiles")
 
 
-@pytest.mark.parametrize("T,H,I,E,k", [(1, 2048, 768, 128, 8), (4, 2048, 768, 128, 8), (3, 1024, 200, 16, 4), (2, 1104, 72, 8, 2),
-                                       (2, 256, 1024, 8, 2), (5, 1024, 1032, 6, 3)])
-def test_one_wavefront_blocks_for_a_few_tiles_give_the_same_bits(T, H, I, E, k):
-    # A step of a few tokens on 16-row tiles with a contraction depth of at least 1024 is launched as one-wavefront
-    # blocks of 16 weight rows (gate/up at H >= 1024, down at I >= 1024; ragged N = 200 / 72, K = 1104 / 1032 included).
-    # 32-row tiles never are, so they are the yardstick; tensors and fragment-order copies alike.
-    assert ops.moe_tile_rows(T, top_k=k, num_experts=E) == 16
-    x, w, sel, gate, up, down = _inputs(T, H, I, E, k, seed=43)
-    xg, wg, sg, dg = x.cuda(), w.cuda(), sel.cuda(), down.cuda()
-    gu = torch.cat([gate, up], dim=1).cuda()
-    packable = I % 16 == 0
-    if packable:
-        pgu, pdn = ops.pack_expert_weights(gu), ops.pack_expert_weights(dg)
-    res = {}
-    for bm in (16, 32):
-        r = ops.moe_route(sg, E, bm=bm)
-        hw = ops.moe_gemm(xg, gu[:, :I, :], r, w2=gu[:, I:, :], row_src=r.sorted_token, row_scale=wg, row_scale_idx=r.sorted_flat)
-        eo = ops.moe_gemm(hw, dg, r)
-        res[bm] = (hw, eo)
-        if packable:
-            hw_p = ops.moe_gemm_packed(xg, pgu.rows(0, I), r, w2=pgu.rows(I, 2 * I), row_src=r.sorted_token, row_scale=wg,
-                                       row_scale_idx=r.sorted_flat)
-            eo_p = ops.moe_gemm_packed(hw, pdn, r)
-            assert_bitwise(hw_p, hw, f"gate/up on packed weights, {bm}-row tiles")
-            assert_bitwise(eo_p, eo, f"down on packed weights, {bm}-row tiles")
-    assert_bitwise(res[16][0], res[32][0], "gate/up + SwiGLU, 16-row tiles in one-wavefront blocks against 32-row tiles")
-    assert_bitwise(res[16][1], res[32][1], "down projection, 16-row tiles in one-wavefront blocks against 32-row tiles")
-    # the whole block (which picks 16-row tiles by itself at these token counts) against the same block on 32-row tiles
-    out = ops.fused_moe(xg, wg, sg, gu[:, :I, :], gu[:, I:, :], dg, E)
-    r32 = ops.moe_route(sg, E, bm=32)
-    assert_bitwise(out, ops.moe_gather(res[32][1], r32.scatter_index), "fused MoE block on a few tokens")
-
-
 @pytest.mark.parametrize("T,H,I,E,k", [(2500, 256, 128, 8, 2), (1100, 192, 64, 3, 1), (4096, 2048, 768, 16, 4)])
 def test_packed_expert_weights_on_256_row_tiles_give_the_same_bits(T, H, I, E, k):
     # prefill-sized steps: the 256 x 256 kernel reading the fragment-order copy against the same kernel on [E, N, K]
