@@ -757,7 +757,8 @@ def moe_tile_rows(num_tokens: int, wide_ok: bool = True, packed_only: bool = Fal
     top-8, measured per block: 448 tokens 256 us on 32-row tiles against 269 on 64-row ones; 768 tokens 309 on 64-row
     tiles against 314 on 256-row ones; 1024 tokens 365 against 311; 1536 tokens 318 against 353 on the 128-row kernel)."""
     if int(num_tokens) <= 16:
-        # an expert receives at most one row per token: one 16-row tile each, half the matrix instructions of a 32-row
+        # an expert receives at most one row per token (a top-k's experts are distinct; duplicates just make more
+        # tiles): one 16-row tile each, half the matrix instructions of a 32-row
         # tile (gate/up at 1 .. 16 tokens 2 us faster), and the form that a launch of a few tiles runs as one-wavefront
         # blocks (1 token 23.8 -> 18.2 us, 4 tokens 46.5 -> 41.0 us)
         return 16
