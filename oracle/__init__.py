@@ -44,7 +44,8 @@ decoder_step_ref       HuggingFace Qwen3MoeForCausalLM last-token logits, packed
 attention_backward_ref autograd through the fp32 eager attention; one visible key => dV = dO, dQ = dK = 0
 fused_moe_backward_ref autograd through an fp32 restatement of the expert MLPs
 sampler.philox4x32     Random123 known-answer vectors
-sampler.exp32 / log    numpy exp / log within 4e-7 / 2e-6
+sampler.exp32 / log    numpy exp / log within 4e-7 / 2e-6; and, with the keys and Philox, bit for bit the text of the
+                       kernel source's scalar routines compiled for the host (tests/test_oracle_sampler.py)
 sampler.kept_mask_spec the reference's sort + cumsum rule (apply_top_k_top_p_ref) on tie-free rows
 sample_tokens_ref      argmax(probs / q) with the same variates; softmax frequencies (chi-square
                        style bound); (seed, position) keyed: order invariance

@@ -122,3 +122,64 @@ def test_token_depends_on_seed_and_position_only():
     assert np.array_equal(b, a[perm])
     c = S.sample_tokens_ref(x, 0.9, 40, 0.95, seeds, pos + 1)
     assert not np.array_equal(a, c)
+
+
+def test_oracle_arithmetic_is_the_kernel_source_arithmetic(tmp_path):
+    """The sampler's scalar arithmetic (order-preserving keys, exp, -log of a uniform, Philox) is plain C++ inside
+    vexact_amd/csrc/sampler.hip. Its text is compiled here for the host, unchanged, and compared bit for bit with the numpy
+    restatement: what the GPU tests compare token ids against is then the shipped source's arithmetic, not a look-alike."""
+    import ctypes
+    import os
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "vexact_amd", "csrc", "sampler.hip")).read()
+    start = text.index("__device__ __forceinline__ uint32_t float_key(float x)")
+    end = text.index("struct SampleParams {")
+    body = text[start:end]
+    for name in ("float_key", "exp32", "neg_log_uniform", "philox4x32"):
+        assert f" {name}(" in body
+    src = tmp_path / "sampler_math.cpp"
+    src.write_text(
+        "#include <math.h>\n#include <stdint.h>\n#define __device__\n#define __forceinline__ inline\n"
+        "struct uint4 { uint32_t x, y, z, w; };\n"
+        "static inline uint4 make_uint4(uint32_t x, uint32_t y, uint32_t z, uint32_t w) { return uint4{x, y, z, w}; }\n"
+        + body +
+        'extern "C" {\n'
+        "void k_float_key(const float* x, uint32_t* o, int64_t n) { for (int64_t i = 0; i < n; i++) o[i] = float_key(x[i]); }\n"
+        "void k_exp32(const float* x, float* o, int64_t n) { for (int64_t i = 0; i < n; i++) o[i] = exp32(x[i]); }\n"
+        "void k_neg_log_uniform(const uint32_t* x, float* o, int64_t n) { for (int64_t i = 0; i < n; i++) o[i] = neg_log_uniform(x[i]); }\n"
+        "void k_philox(const uint32_t* c, const uint32_t* k, uint32_t* o, int64_t n) {\n"
+        "  for (int64_t i = 0; i < n; i++) { const uint4 r = philox4x32(uint4{c[4 * i], c[4 * i + 1], c[4 * i + 2], c[4 * i + 3]}, k[2 * i], k[2 * i + 1]);\n"
+        "    o[4 * i] = r.x; o[4 * i + 1] = r.y; o[4 * i + 2] = r.z; o[4 * i + 3] = r.w; } }\n"
+        "}\n")
+    so = tmp_path / "sampler_math.so"
+    subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-ffp-contract=off", "-o", str(so), str(src)], check=True)
+    lib = ctypes.CDLL(str(so))
+    rng = np.random.default_rng(5)
+    P = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    n = 400_000
+    # keys: any float, including the signed zeros, infinities and subnormals
+    x = np.concatenate([rng.standard_normal(n).astype(np.float32) * 50, rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32).view(np.float32),
+                        np.array([0.0, -0.0, np.inf, -np.inf, 1e-45, -1e-45], dtype=np.float32)])
+    x = x[~np.isnan(x)]
+    out = np.empty(x.size, dtype=np.uint32)
+    lib.k_float_key(P(x), P(out), ctypes.c_int64(x.size))
+    assert np.array_equal(out, S.float_key(x))
+    # exp on [-32, 0] (what the kernel feeds it) and a little beyond
+    d = np.concatenate([-rng.random(n).astype(np.float32) * 32, np.linspace(-33, 1, 4097, dtype=np.float32), np.array([0.0, -32.0], dtype=np.float32)])
+    out = np.empty(d.size, dtype=np.float32)
+    lib.k_exp32(P(d), P(out), ctypes.c_int64(d.size))
+    assert np.array_equal(out.view(np.uint32), S.exp32(d).view(np.uint32))
+    # -log u for every kind of 32-bit draw
+    u = np.concatenate([rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32), np.array([0, 1, 2, 2**31 - 1, 2**31, 2**32 - 1], dtype=np.uint32),
+                        (np.uint32(1) << np.arange(32, dtype=np.uint32))])
+    out = np.empty(u.size, dtype=np.float32)
+    lib.k_neg_log_uniform(P(u), P(out), ctypes.c_int64(u.size))
+    assert np.array_equal(out.view(np.uint32), S.neg_log_uniform(u).view(np.uint32))
+    # Philox on random counters and keys
+    c = rng.integers(0, 2**32, (20_000, 4), dtype=np.uint64).astype(np.uint32)
+    k = rng.integers(0, 2**32, (20_000, 2), dtype=np.uint64).astype(np.uint32)
+    out = np.empty_like(c)
+    lib.k_philox(P(np.ascontiguousarray(c)), P(np.ascontiguousarray(k)), P(out), ctypes.c_int64(c.shape[0]))
+    assert np.array_equal(out, S.philox4x32(c, k))
