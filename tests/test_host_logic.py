@@ -428,3 +428,67 @@ def test_host_metadata_and_allocator_under_address_and_ub_sanitizers():
         run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "sanitized run ok" in run.stdout
+
+
+def test_attention_row_block_numbering_covers_every_block_once(tmp_path):
+    """Which (sequence, row block, head group) a workgroup of the general attention kernels works on is decided by two pieces
+    of plain C++ in vexact_amd/csrc/attn_core.h: the host lambda that sizes the grid (plain or compact numbering) and the
+    device function locate_row_block. Both are compiled here for the host from the source text, unchanged, and every workgroup
+    of the grid is walked: each block that holds query rows must be reached exactly once, in every form."""
+    import ctypes
+    import os
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "vexact_amd", "csrc", "attn_core.h")).read()
+    a = text.index("__device__ __forceinline__ bool locate_row_block(")
+    locate = text[a:text.index("__device__ __forceinline__ float fast_exp2", a)]
+    b = text.index("    auto row_grid = [&](int rb, unsigned heads) {")
+    row_grid = text[b:text.index("    dim3 grid = row_grid(", b)]
+    src = tmp_path / "row_blocks.cpp"
+    src.write_text(
+        "#include <algorithm>\n#include <stdint.h>\n#define __device__\n#define __forceinline__ inline\n"
+        "struct dim3 { unsigned x, y, z; dim3(unsigned a = 1, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {} };\n"
+        "struct AttnParams { const int* cu_q; int num_seqs, compact, grid_heads, grid_sg; };\n"
+        "static dim3 blockIdx, gridDim;\n" + locate +
+        'extern "C" int walk(const int* cu_q, int num_seqs, int total_q, int max_q, int rpb, unsigned nheads, int* counts, int maxblocks,\n'
+        "                    int* form) {\n"
+        "  AttnParams p = {cu_q, num_seqs, 0, 0, 0};\n"
+        "  const int rows = max_q > 0 ? max_q : total_q;\n" + row_grid +
+        "  const dim3 grid = row_grid(rpb, nheads);\n"
+        "  gridDim = grid;\n  *form = p.compact;\n  int stray = 0;\n"
+        "  for (unsigned z = 0; z < grid.z; z++) for (unsigned y = 0; y < grid.y; y++) for (unsigned x = 0; x < grid.x; x++) {\n"
+        "    blockIdx = dim3(x, y, z);\n    int seq, bx, hg;\n"
+        "    if (!locate_row_block(p, rpb, seq, bx, hg)) continue;\n"
+        "    if (seq < 0 || seq >= num_seqs || hg < 0 || hg >= (int)nheads || bx < 0) { stray++; continue; }\n"
+        "    if ((int64_t)bx * rpb >= cu_q[seq + 1] - cu_q[seq]) continue;  // no query row in this block: the kernel leaves at once\n"
+        "    if (bx >= maxblocks) { stray++; continue; }\n"
+        "    counts[((int64_t)seq * maxblocks + bx) * nheads + hg]++;\n  }\n  return stray;\n}\n")
+    so = tmp_path / "row_blocks.so"
+    subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-o", str(so), str(src)], check=True)
+    lib = ctypes.CDLL(str(so))
+    rng = np.random.default_rng(11)
+    forms = set()
+    batches = [[512] * 4, [1] * 40 + [700], [1, 1, 8192, 1], [0, 5, 0, 0, 33], [70000], [3] * 300, [2048, 1, 1, 1, 1, 1, 1, 1, 900]]
+    batches += [list(rng.integers(0, 300, rng.integers(1, 12))) for _ in range(20)]
+    batches.append([1_100_000, 3])  # more row blocks of 16 than a grid dimension can count
+    for lens in batches:
+        if sum(lens) == 0:
+            continue
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        huge = sum(lens) > 1_000_000
+        for rpb in ((16,) if huge else (16, 32, 64, 128, 256)):
+            for nheads in ((2,) if huge else (1, 2, 4, 8, 32)):
+                for max_q in (int(max(lens)), 0):  # 0 = unknown: the launch then assumes total_q rows per sequence
+                    maxblocks = int((max(lens) + rpb - 1) // rpb)
+                    counts = np.zeros((len(lens), maxblocks, nheads), dtype=np.int32)
+                    form = ctypes.c_int(-1)
+                    stray = lib.walk(cu.ctypes.data_as(ctypes.c_void_p), len(lens), int(sum(lens)), int(max_q), rpb, nheads,
+                                     counts.ctypes.data_as(ctypes.c_void_p), maxblocks, ctypes.byref(form))
+                    forms.add(form.value)
+                    assert stray == 0, (lens, rpb, nheads, max_q)
+                    want = np.zeros_like(counts)
+                    for s, n in enumerate(lens):
+                        want[s, : (n + rpb - 1) // rpb, :] = 1
+                    assert np.array_equal(counts, want), (lens, rpb, nheads, max_q, form.value)
+    assert forms == {0, 1, 2}, forms  # the plain grid, the compact numbering, and its form for more than 65535 items
