@@ -492,3 +492,65 @@ def test_attention_row_block_numbering_covers_every_block_once(tmp_path):
                         want[s, : (n + rpb - 1) // rpb, :] = 1
                     assert np.array_equal(counts, want), (lens, rpb, nheads, max_q, form.value)
     assert forms == {0, 1, 2}, forms  # the plain grid, the compact numbering, and its form for more than 65535 items
+
+
+def test_wide_gemm_tile_walk_reaches_every_tile_once(tmp_path):
+    """The persistent 256 x 256 GEMM kernel hands tiles out by a fixed rule: workgroup b of G starts at
+    (b & 7) (G / 8) + (b >> 3) and steps by G, and tile number -> (rows, columns) goes through tile_at (groups of four row
+    tiles for the dense form, the expert tile table for the grouped one). That text of vexact_amd/csrc/gemm_wide.h is compiled
+    here for the host, unchanged: over all workgroups every output tile must come up exactly once."""
+    import ctypes
+    import os
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "vexact_amd", "csrc", "gemm_wide.h")).read()
+    a = text.index("  const int G = gridDim.x;  // multiple of 8")
+    walk = text[a:text.index("  if (first >= tiles || !tile_at(first).ok) return;", a)]
+    group_m = int(text.split("constexpr int WD_GROUP_M = ")[1].split(";")[0])
+
+    def variant(name, grouped):
+        body = walk.replace("if constexpr (GROUPED)", "if constexpr (%s)" % ("true" if grouped else "false"))
+        return ("extern \"C\" int @NAME@(int M, int tiles_m, int tiles_n, int G_, const int* tg, const int* tr0, const int* trows, int BM, int NOUT,\n"
+                "                int* out /* [tiles][4]: row0, rows, n0, ok */, int* hits) {\n"
+                "  struct { int M; const int* tile_group; const int* tile_row0; const int* tile_rows; int64_t w_gstride; } p = {M, tg, tr0, trows, 1000};\n"
+                "  const int tiles = tiles_m * tiles_n;\n  struct { unsigned x; } gridDim = {(unsigned)G_}, blockIdx = {0};\n"
+                "  for (unsigned b = 0; b < (unsigned)G_; b++) {\n    blockIdx.x = b;\n" + body +
+                "    for (int lin = first; lin < tiles; lin += G) {\n      const WideTile t = tile_at(lin);\n"
+                "      out[4 * lin] = t.row0; out[4 * lin + 1] = t.rows; out[4 * lin + 2] = t.n0; out[4 * lin + 3] = t.ok; hits[lin]++;\n"
+                "    }\n  }\n  return 0;\n}\n").replace("@NAME@", name)
+
+    src = tmp_path / "tile_walk.cpp"
+    src.write_text("#include <algorithm>\n#include <stdint.h>\nusing std::min;\nconstexpr int WD_GROUP_M = %d;\n"
+                   "struct WideTile { int row0, rows, n0; int64_t wbase; bool ok; };\n" % group_m
+                   + variant("walk_dense", False) + variant("walk_grouped", True))
+    so = tmp_path / "tile_walk.so"
+    subprocess.run(["g++", "-O1", "-std=c++17", "-shared", "-fPIC", "-o", str(so), str(src)], check=True)
+    lib = ctypes.CDLL(str(so))
+    P = lambda x: x.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    rng = np.random.default_rng(3)
+    for BM, NOUT in ((256, 256), (128, 256), (256, 128)):
+        for M, N in ((8192, 5120), (300, 256), (4097, 1000), (256 * 7 + 1, 151936), (100, 100)):
+            tiles_m, tiles_n = (M + BM - 1) // BM, (N + NOUT - 1) // NOUT
+            for G in (8, 64, 256):
+                out = np.full((tiles_m * tiles_n, 4), -1, dtype=np.int32)
+                hits = np.zeros(tiles_m * tiles_n, dtype=np.int32)
+                lib.walk_dense(M, tiles_m, tiles_n, G, None, None, None, BM, NOUT, P(out), P(hits))
+                assert (hits == 1).all(), (M, N, BM, G)
+                seen = {(int(r), int(c)) for r, _, c, _ in out}
+                assert seen == {(i * BM, j * NOUT) for i in range(tiles_m) for j in range(tiles_n)}
+                assert all(int(rows) == min(BM, M - int(r0)) and ok == 1 for r0, rows, _, ok in out)
+    # grouped: a table of row tiles (expert, first row, rows), unused entries marked -1 at the end
+    for _ in range(20):
+        n_tiles, spare, tiles_n, G = int(rng.integers(1, 400)), int(rng.integers(0, 9)), int(rng.integers(1, 9)), int(rng.choice([8, 64, 256]))
+        tg = np.concatenate([np.sort(rng.integers(0, 128, n_tiles)), -np.ones(spare)]).astype(np.int32)
+        tr0 = np.concatenate([np.arange(n_tiles) * 256, np.zeros(spare)]).astype(np.int32)
+        trows = np.concatenate([rng.integers(1, 257, n_tiles), np.zeros(spare)]).astype(np.int32)
+        tiles_m = n_tiles + spare
+        out = np.full((tiles_m * tiles_n, 4), -1, dtype=np.int32)
+        hits = np.zeros(tiles_m * tiles_n, dtype=np.int32)
+        lib.walk_grouped(0, tiles_m, tiles_n, G, P(tg), P(tr0), P(trows), 256, 256, P(out), P(hits))
+        assert (hits == 1).all()
+        real = out[out[:, 3] == 1]
+        assert {(int(r), int(c)) for r, _, c, _ in real} == {(int(r), j * 256) for r in tr0[:n_tiles] for j in range(tiles_n)}
+        assert len(real) == n_tiles * tiles_n and (out[out[:, 3] == 0].shape[0] == spare * tiles_n)
