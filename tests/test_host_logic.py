@@ -554,3 +554,83 @@ def test_wide_gemm_tile_walk_reaches_every_tile_once(tmp_path):
         real = out[out[:, 3] == 1]
         assert {(int(r), int(c)) for r, _, c, _ in real} == {(int(r), j * 256) for r in tr0[:n_tiles] for j in range(tiles_n)}
         assert len(real) == n_tiles * tiles_n and (out[out[:, 3] == 0].shape[0] == spare * tiles_n)
+
+
+def test_paged_key_addresses_stay_inside_the_sequence_pages(tmp_path):
+    """Where the attention kernels read a sequence's keys and values is decided by KVSource in
+    vexact_amd/csrc/attn_core.h (page lookup per 16-key tile for power-of-two pages, per key otherwise, packed rows without a
+    table). Its text is compiled for the host with -fsanitize=address and driven the way the kernels drive it (64-key blocks,
+    lanes past the end asking for row 0 of their tile): the block-table row is an exactly sized heap array holding only the
+    sequence's own pages, so a lookup past them aborts, and every address must be the row of an existing key (the right one
+    for keys below the length)."""
+    import os
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "vexact_amd", "csrc", "attn_core.h")).read()
+    a = text.index("enum : int { SRC_FAST = 0, SRC_GENERIC = 1, SRC_PACKED = 2 };")
+    b = text.index("template <int KIND>\nstruct KVSource {", a)
+    struct = text[a:text.index("\n};\n", b) + 4]
+    src = tmp_path / "kv_source.cpp"
+    src.write_text(
+        "#include <algorithm>\n#include <cstdio>\n#include <cstdlib>\n#include <random>\n#include <stdint.h>\n#include <vector>\n"
+        "#define __device__\n#define __forceinline__ inline\nusing std::min;\ntypedef uint16_t bf16_t;\n" + struct + r"""
+#define CHECK(c) do { if (!(c)) { std::fprintf(stderr, "check failed at line %d: %s\n", __LINE__, #c); std::exit(1); } } while (0)
+template <int KIND>
+static void run(std::mt19937_64& rng) {
+  auto rnd = [&](int64_t lo, int64_t hi) { return lo + (int64_t)(rng() % (uint64_t)(hi - lo + 1)); };
+  for (int it = 0; it < 300; it++) {
+    const int ps = KIND == SRC_FAST ? (16 << rnd(0, 4)) : (int)rnd(1, 40);
+    const int kv_len = (int)rnd(1, 700), npages = (kv_len + ps - 1) / ps, pool = npages + (int)rnd(0, 50);
+    std::vector<int> table((size_t)npages);  // exactly the sequence's pages: a lookup past them is a heap overflow
+    for (auto& t : table) t = (int)rnd(0, pool - 1);
+    const int64_t D = 128, skp = 4 * D, skb = (int64_t)ps * skp;  // [blocks, page, 4 heads, D]
+    KVSource<KIND> s;
+    s.kbase = (const bf16_t*)0 + 2 * D; s.vbase = (const bf16_t*)0 + 3 * D;  // kv heads 2 and 3; offsets only, never dereferenced
+    s.bt = KIND == SRC_PACKED ? nullptr : table.data();
+    s.skb = skb; s.skp = skp; s.svb = skb; s.svp = skp;
+    s.ps = ps; s.last = kv_len - 1;
+    s.shift = -1;
+    if ((ps & (ps - 1)) == 0) { s.shift = 0; while ((1 << s.shift) < ps) s.shift++; }
+    if (KIND == SRC_GENERIC && rnd(0, 1)) s.shift = -1;  // the division form also for power-of-two pages
+    for (int kb = 0; kb < kv_len; kb += 64) {
+      const typename KVSource<KIND>::Tiles tl = s.tiles(kb);
+      for (int tt = 0; tt < 4; tt++)
+        for (int lane_row = 0; lane_row < 16; lane_row++) {
+          const int key = kb + 16 * tt + lane_row;
+          const bool ok = key < kv_len;
+          const int within = ok ? lane_row : 0;  // what issue_k / issue_v pass
+          for (int is_v = 0; is_v < 2; is_v++) {
+            const bf16_t* r = is_v ? s.vrow(tl, kb, tt, within) : s.krow(tl, kb, tt, within);
+            const int64_t off = (r - (const bf16_t*)0) - (is_v ? 3 : 2) * D;
+            CHECK(off >= 0 && off % skp == 0);
+            const int64_t row = off / skp;
+            if (KIND == SRC_PACKED) {
+              CHECK(row == (ok ? key : std::min(kb + 16 * tt, kv_len - 1)));
+            } else {
+              const int64_t page = row / ps, in_page = row % ps;
+              bool found = false;  // the row of an existing key of this sequence
+              for (int pg = 0; pg < npages && !found; pg++) found = table[(size_t)pg] == page && pg * ps + in_page < kv_len;
+              CHECK(found);
+              if (ok) CHECK(page == table[(size_t)(key / ps)] && in_page == key % ps);
+            }
+          }
+        }
+    }
+  }
+}
+int main() {
+  std::mt19937_64 rng(99);
+  run<SRC_FAST>(rng);
+  run<SRC_GENERIC>(rng);
+  run<SRC_PACKED>(rng);
+  std::puts("kv source sanitized run ok");
+  return 0;
+}
+""")
+    exe = tmp_path / "kv_source"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-static-libasan",
+                    "-o", str(exe), str(src)], check=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "sanitized run ok" in run.stdout
