@@ -634,3 +634,30 @@ int main() {
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "sanitized run ok" in run.stdout
+
+
+def test_tile_table_bound_holds_for_any_split_of_the_rows():
+    # vx_moe_max_tiles(n, E, bm) sizes the tile table that the routing kernel fills with ceil(rows_e / bm) tiles per expert:
+    # it must be an upper bound for every way n (token, slot) entries can fall on E experts, and it is attained.
+    from vexact_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(2)
+    for _ in range(3000):
+        E, bm = int(rng.integers(1, 300)), int(rng.choice([16, 32, 64, 128, 256]))
+        n = int(rng.integers(0, 5000))
+        kind = rng.integers(0, 3)
+        if kind == 0:      # uniform
+            rows = np.bincount(rng.integers(0, E, n), minlength=E)
+        elif kind == 1:    # everything on a few experts
+            rows = np.bincount(rng.integers(0, min(E, 3), n), minlength=E)
+        else:              # as many experts as possible one past a multiple of the tile height
+            rows = np.zeros(E, dtype=np.int64)
+            left = n
+            for e in range(E):
+                take = min(left, bm * int(rng.integers(0, 3)) + 1)
+                rows[e], left = take, left - take
+            rows[0] += left
+        tiles = int(((rows + bm - 1) // bm).sum())
+        assert tiles <= lib.vx_moe_max_tiles(n, E, bm), (n, E, bm, tiles)
+    # attained: min(E, n) experts with one row beyond whole tiles
+    assert lib.vx_moe_max_tiles(3 * 32 + 3, 3, 32) == 3 + 3 and int(((np.array([33, 33, 33]) + 31) // 32).sum()) == 6
